@@ -1,0 +1,161 @@
+/*
+ * symmetrix_amd.h -- C ABI of the MI355X (gfx950) MACE energy+forces engine.
+ *
+ * Drop-in boundary for the hot path of wcwitt/symmetrix: everything the
+ * reference's `class MACE` (libsymmetrix/source/mace.hpp:12-169) offers to its
+ * three callers -- the pybind module (symmetrix/source/cpp/mace.cpp:12-243), the
+ * LAMMPS pair style (pair_symmetrix/pair_symmetrix_mace.cpp:319-320, :444-495,
+ * :662-698) and the ASE calculator (symmetrix/source/symmetrix/symmetrix_calc.py:
+ * 72-102) -- is reachable through the functions below with plain pointers and
+ * sizes.  `include/symmetrix_amd/mace.hpp` wraps them in a header-compatible
+ * C++ `class MACE`; `symmetrix_amd/mace.py` wraps them for Python.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and a negative SMX_E* code on
+ *     failure; smx_last_error() returns the message of the calling thread's
+ *     last failure (the reference throws C++ exceptions instead,
+ *     libsymmetrix/source/cubic_spline.cpp:19-20, mace.cpp:908-909).
+ *   - Arrays named like the reference's members have the reference's layout
+ *     (row-major, channel index fastest).  Host getters/setters always speak
+ *     double, whatever precision the engine holds internally.
+ *   - One model object is not re-entrant (as the reference's, whose scratch
+ *     state lives in members): one thread at a time per model.
+ *   - There is no CPU fallback: every compute entry point needs a gfx950
+ *     device and fails with SMX_ENODEVICE without one.
+ */
+#ifndef SYMMETRIX_AMD_H
+#define SYMMETRIX_AMD_H
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct smx_model smx_model;
+
+enum {
+    SMX_OK = 0,
+    SMX_EINVAL = -1,    /* bad argument (null pointer, negative size, index out of range) */
+    SMX_EFILE = -2,     /* model file missing, malformed JSON, missing or ill-typed key */
+    SMX_EUNSUPPORTED = -3, /* model outside what the kernels implement (see message) */
+    SMX_ENODEVICE = -4, /* no usable gfx950 device */
+    SMX_EHIP = -5,      /* HIP runtime error (message carries hipGetErrorString) */
+    SMX_ERANGE = -6,    /* spline argument out of range: r <= 0, r >= r_cut or not finite */
+    SMX_ENOMEM = -7
+};
+
+/* smx_model_load flags */
+enum {
+    SMX_FP64 = 0,          /* everything in double, as the reference CPU path */
+    SMX_FP32_FEATURES = 1  /* features, tables and weights in float; positions, H2,
+                              readouts, energies and force sums in double (the split of
+                              MACEKokkos<float>, libsymmetrix/source/mace_kokkos.hpp:34-181) */
+};
+
+const char* smx_last_error(void);
+
+/* MACE::MACE(std::string) / MACE::load_from_json, mace.cpp:12-15, 905-1030.
+ * Reads the symmetrix JSON model file and uploads tables and weights to the
+ * current HIP device. */
+int smx_model_load(const char* json_path, int flags, smx_model** out);
+void smx_model_free(smx_model* m);
+
+/* Public scalar members of class MACE, mace.hpp:19-26,115: keys "num_elements",
+ * "num_channels", "l_max", "num_lm", "L_max", "num_LM", "has_zbl", "num_lme",
+ * "num_lelm1lm2", "precision" (0/1); "r_cut". */
+int smx_model_get_int(const smx_model* m, const char* key, int* out);
+int smx_model_get_double(const smx_model* m, const char* key, double* out);
+/* atomic_numbers[T], atomic_energies[T], mace.hpp:25-26.  *n receives the length. */
+int smx_model_get_atomic_numbers(const smx_model* m, int* out, int cap, int* n);
+int smx_model_get_atomic_energies(const smx_model* m, double* out, int cap, int* n);
+
+/* MACE::compute_node_energies_forces, mace.cpp:17-64.  Host arrays, exactly the
+ * reference's arguments plus explicit lengths: node_types[num_nodes],
+ * num_neigh[num_nodes], neigh_indices[num_edges], neigh_types[num_edges],
+ * xyz[3*num_edges] (x_j - x_i), r[num_edges].  Results stay on the device until
+ * fetched with smx_get_array("node_energies" / "node_forces"). */
+int smx_compute_node_energies_forces(smx_model* m, int num_nodes,
+                                     const int* node_types, const int* num_neigh,
+                                     const int* neigh_indices, const int* neigh_types,
+                                     const double* xyz, const double* r, long num_edges);
+
+/* Same computation with every array already resident in device memory and the
+ * work enqueued on `stream` (a hipStream_t, or NULL for the default stream).
+ * d_node_energies[num_nodes] and d_node_forces[3*num_edges] may be NULL, in
+ * which case results are only kept inside the model.  Does not synchronise. */
+int smx_compute_device(smx_model* m, int num_nodes,
+                       const int* d_node_types, const int* d_num_neigh,
+                       const int* d_neigh_indices, const int* d_neigh_types,
+                       const double* d_xyz, const double* d_r, long num_edges,
+                       double* d_node_energies, double* d_node_forces, void* stream);
+
+/* Number of rows of H1 a following layer-1 call may index (ghost rows of the
+ * LAMMPS modes, pair_symmetrix_mace.cpp:462-471, 674-698).  Defaults to the
+ * num_nodes of the last compute_H1. */
+int smx_set_num_H1_rows(smx_model* m, int rows);
+
+/* Stage-level entry points, one per public method of class MACE
+ * (mace.hpp:29-164).  Edge geometry is remembered from the last
+ * smx_compute_Y (xyz) and smx_compute_R0/R1 (r, types), as the reference
+ * remembers Y, R0 and R1. */
+int smx_compute_Y(smx_model* m, const double* xyz, long n3);                             /* mace.cpp:118-148 */
+int smx_compute_R0(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                   const int* neigh_types, const double* r, long num_edges);            /* mace.cpp:66-90 */
+int smx_compute_R1(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                   const int* neigh_types, const double* r, long num_edges);            /* mace.cpp:92-116 */
+int smx_compute_A0(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                   const int* neigh_types, long num_edges);                             /* mace.cpp:150-201 */
+int smx_reverse_A0(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                   const int* neigh_types, const double* xyz, const double* r, long num_edges); /* mace.cpp:203-271 */
+int smx_compute_M0(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:348-370 */
+int smx_reverse_M0(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:372-395 */
+int smx_compute_H1(smx_model* m, int num_nodes);                                        /* mace.cpp:397-423 */
+int smx_reverse_H1(smx_model* m, int num_nodes);                                        /* mace.cpp:425-451 */
+int smx_compute_Phi1(smx_model* m, int num_nodes, const int* num_neigh,
+                     const int* neigh_indices, long num_edges);                         /* mace.cpp:453-502 */
+int smx_reverse_Phi1(smx_model* m, int num_nodes, const int* num_neigh, const int* neigh_indices,
+                     const double* xyz, const double* r, long num_edges,
+                     int zero_dxyz, int zero_H1_adj);                                   /* mace.cpp:504-605 */
+int smx_compute_A1(smx_model* m, int num_nodes);                                        /* mace.cpp:607-642 */
+int smx_reverse_A1(smx_model* m, int num_nodes);                                        /* mace.cpp:644-679 */
+int smx_compute_M1(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:759-777 */
+int smx_reverse_M1(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:779-794 */
+int smx_compute_H2(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:796-832 */
+int smx_reverse_H2(smx_model* m, int num_nodes, const int* node_types, int zero_H1_adj);/* mace.cpp:834-874 */
+int smx_compute_readouts(smx_model* m, int num_nodes, const int* node_types);           /* mace.cpp:876-903 */
+
+/* Read/write access to the named intermediates, the def_readwrite members of
+ * the pybind class (symmetrix/source/cpp/mace.cpp:14-34): "node_energies",
+ * "node_forces", "A0", "A0_adj", "M0", "M0_adj", "H1", "H1_adj", "Phi1",
+ * "Phi1_adj", "A1", "A1_adj", "M1", "M1_adj", "H2", "H2_adj", plus "Y",
+ * "Y_grad", "R0", "R1" (read-only, evaluated on demand from the remembered
+ * geometry), "M0_grad", "M1_grad" and "H0_weights" (read-only).
+ * smx_get_array copies min(cap, size) doubles to `out` and stores the full
+ * size in *n; out may be NULL to query the size. */
+int smx_get_array(smx_model* m, const char* name, double* out, long cap, long* n);
+int smx_set_array(smx_model* m, const char* name, const double* in, long n);
+
+/* Per-stage timing with HIP events on the stream the kernels run on.  When
+ * enabled, every stage of the next compute is bracketed by events;
+ * smx_get_stage_times synchronises and returns elapsed milliseconds per stage.
+ * Stage names come back as a ';'-separated list from smx_stage_names. */
+int smx_set_profiling(smx_model* m, int enabled);
+const char* smx_stage_names(void);
+int smx_get_stage_times(smx_model* m, float* ms, int cap, int* n);
+
+/* Blocks until all work enqueued for this model has finished. */
+int smx_synchronize(smx_model* m);
+
+/* Caller-side helpers, device resident (counterparts of the force and virial
+ * scatter of pair_symmetrix_mace.cpp:334-368 and symmetrix_calc.py:93-102):
+ * atom_forces[num_atoms][3] = sum over edges of +f_ij on sender j and -f_ij on
+ * receiver i; virial[6] = sum xyz (x) f_ij in LAMMPS order xx,yy,zz,xy,xz,yz.
+ * receiver_atom/sender_atom map edge ends to atom rows; NULL receiver_atom
+ * means the receiver of edge block i is atom i.  Uses the forces of the last
+ * compute.  Outputs are host arrays. */
+int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const int* receiver_atom,
+                      double* atom_forces, double* virial);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,1041 @@
+// Host orchestration and C ABI of the MACE energy+forces engine.
+//
+// Pipeline (the stage list of MACE::compute_node_energies_forces,
+// libsymmetrix/source/mace.cpp:17-64), one HIP kernel or one batched MFMA
+// launch per stage, all on one stream, nothing computed on the host:
+//
+//   prep        CSR offsets, sender lists, species groups        (integers only)
+//   agg0_fwd    Phi0 = sum_j R0 Y H0                             mace.cpp:158-178
+//   A0_lin      A0 = Phi0 . A0_weights[type][l]        (MFMA)    mace.cpp:180-199
+//   M0          symmetric contraction + gradient                 mace.cpp:348-370
+//   H1          H1 = M0 . H1_weights[l]                (MFMA)    mace.cpp:397-423
+//   agg1_fwd    Phi1 = CG . sum_j R1 Y H1[j]                     mace.cpp:453-502
+//   A1          A1 = Phi1 . A1_weights[l]              (MFMA)    mace.cpp:607-642
+//   M1          symmetric contraction + gradient                 mace.cpp:759-777
+//   H2          H2 = H1[l=0].W[type] + M1.W            (MFMA)    mace.cpp:796-832
+//   readout     energies, H1_adj seed, H2_adj          (MFMA)    mace.cpp:876-903
+//   rev_H2, rev_M1, rev_A1, agg1_bwd, sender_reduce, rev_H1, rev_M0,
+//   rev_A0_lin, agg0_bwd                                         mace.cpp:54-63
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdio>
+#include <cstring>
+#include <memory>
+#include <stdexcept>
+#include <string>
+#include <vector>
+
+#include "../../include/symmetrix_amd.h"
+#include "smx_host_model.hpp"
+#include "smx_json.hpp"
+#include "smx_kernels.hpp"
+#include "smx_paths.hpp"
+
+namespace smx {
+
+struct Error : std::runtime_error {
+    int code;
+    Error(int c, const std::string& m) : std::runtime_error(m), code(c) {}
+};
+
+static thread_local std::string g_last_error;
+
+#define HIPCHK(expr)                                                                                   \
+    do {                                                                                               \
+        hipError_t e_ = (expr);                                                                        \
+        if (e_ != hipSuccess)                                                                          \
+            throw ::smx::Error(e_ == hipErrorOutOfMemory ? SMX_ENOMEM : SMX_EHIP,                      \
+                        std::string(#expr) + ": " + hipGetErrorString(e_));                            \
+    } while (0)
+
+// growable device array with std::vector::resize semantics (contents kept, new tail zeroed)
+template <typename T>
+struct DVec {
+    T* p = nullptr;
+    size_t n = 0, cap = 0;
+    ~DVec() { if (p) (void)hipFree(p); }
+    DVec() = default;
+    DVec(const DVec&) = delete;
+    DVec& operator=(const DVec&) = delete;
+    void reserve(size_t m, hipStream_t s, bool keep)
+    {
+        if (m <= cap) return;
+        size_t newcap = m + m / 8 + 64;
+        T* q = nullptr;
+        HIPCHK(hipMalloc(&q, newcap * sizeof(T)));
+        if (p) {
+            if (keep && n) HIPCHK(hipMemcpyAsync(q, p, n * sizeof(T), hipMemcpyDeviceToDevice, s));
+            HIPCHK(hipStreamSynchronize(s));
+            HIPCHK(hipFree(p));
+        }
+        p = q;
+        cap = newcap;
+    }
+    // size to m elements; previous contents are undefined afterwards
+    void size_to(size_t m, hipStream_t s) { reserve(m, s, false); n = m; }
+    // std::vector::resize
+    void resize(size_t m, hipStream_t s)
+    {
+        reserve(m, s, true);
+        if (m > n) HIPCHK(hipMemsetAsync(p + n, 0, (m - n) * sizeof(T), s));
+        n = m;
+    }
+    void upload(const T* host, size_t m, hipStream_t s)
+    {
+        size_to(m, s);
+        if (m) HIPCHK(hipMemcpyAsync(p, host, m * sizeof(T), hipMemcpyHostToDevice, s));
+    }
+};
+
+template <typename T, typename S>
+static void upload_as(DVec<T>& d, const std::vector<S>& h, hipStream_t s)
+{
+    std::vector<T> tmp(h.begin(), h.end());
+    d.upload(tmp.data(), tmp.size(), s);
+    HIPCHK(hipStreamSynchronize(s));  // tmp goes out of scope
+}
+
+static const char* kStageNames =
+    "prep;agg0_fwd;A0_lin;M0;H1;agg1_fwd;A1;M1;H2;readout;rev_H2;rev_M1;rev_A1;agg1_bwd;sender_reduce;"
+    "rev_H1;rev_M0;rev_A0_lin;agg0_bwd";
+enum Stage { ST_PREP, ST_AGG0F, ST_A0LIN, ST_M0, ST_H1, ST_AGG1F, ST_A1, ST_M1, ST_H2, ST_READOUT, ST_REVH2,
+             ST_REVM1, ST_REVA1, ST_AGG1B, ST_SRED, ST_REVH1, ST_REVM0, ST_REVA0LIN, ST_AGG0B, ST_COUNT };
+
+struct EngineBase {
+    virtual ~EngineBase() = default;
+    HostModel hm;
+    int precision = 0;
+    hipStream_t stream = nullptr;   // stream of the current call
+    bool profiling = false;
+    hipEvent_t ev0[ST_COUNT] = {}, ev1[ST_COUNT] = {};
+    bool ev_used[ST_COUNT] = {};
+    int H1_rows_override = -1;
+
+    virtual void compute(int N, const int* node_types, const int* num_neigh, const int* neigh_indices,
+                         const int* neigh_types, const double* xyz, const double* r, long E, bool on_device,
+                         double* d_energies, double* d_forces) = 0;
+    virtual void stage(const char* name, int N, const int* node_types, const int* num_neigh,
+                       const int* neigh_indices, const int* neigh_types, const double* xyz, const double* r,
+                       long E, int flag_a, int flag_b) = 0;
+    virtual void get_array(const char* name, double* out, long cap, long* n) = 0;
+    virtual void set_array(const char* name, const double* in, long n) = 0;
+    virtual void reduce_forces(int num_atoms, const int* sender_atom, const int* receiver_atom,
+                               double* atom_forces, double* virial) = 0;
+
+    void stage_begin(int st)
+    {
+        if (!profiling) return;
+        if (!ev0[st]) { HIPCHK(hipEventCreate(&ev0[st])); HIPCHK(hipEventCreate(&ev1[st])); }
+        HIPCHK(hipEventRecord(ev0[st], stream));
+    }
+    void stage_end(int st)
+    {
+        if (!profiling) return;
+        HIPCHK(hipEventRecord(ev1[st], stream));
+        ev_used[st] = true;
+    }
+};
+
+template <typename F>
+struct Engine : EngineBase {
+    // ---- model on device
+    DVec<F> tab0, tab1, H0, A0w, H1w, A1w;
+    DVec<int> pair_table0, pair_table1;
+    DVec<int> B0_start, B0_lm1, B1_start, B1_lm1;
+    DVec<double> B0_c, B1_c;
+    std::vector<long> A1w_off;   // per l
+    DVec<double> H2w_H1, H2w_M1, ro1, ro2_w1, ro2_w2, E0;
+    struct DevPoly {
+        DVec<int> row_i0, row_i1, row_start, entry_var;
+        DVec<F> coef;
+        int num_rows = 0, num_entries = 0;
+    };
+    std::vector<std::unique_ptr<DevPoly>> P0;
+    DevPoly P1;
+    // pointer tables for the polynomial kernel: [0..num_LM) = P0, then P1
+    DVec<const int*> pp_i0, pp_i1, pp_start, pp_var;
+    DVec<const F*> pp_coef;
+    DVec<int> pp_nrows, pp_nent;
+
+    // ---- geometry of the current edge list (device)
+    DVec<int> g_node_types, g_num_neigh, g_neigh_indices, g_neigh_types;
+    DVec<double> g_xyz, g_r;
+    const int *node_types = nullptr, *num_neigh = nullptr, *neigh_indices = nullptr, *neigh_types = nullptr;
+    const double *xyz = nullptr, *r = nullptr;
+    long E = 0;
+    int N_geo = 0;
+    DVec<int> first_neigh, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
+    int sender_rows = 0;
+
+    // ---- state (mace.hpp members)
+    DVec<F> Phi0, A0, A0_adj, M0, M0_grad, M0_adj, H1, H1_adj, Phi1, dPhi1, A1, A1_adj, M1, M1_grad, M1_adj, msg;
+    DVec<double> H2, H2_adj, hidden, node_energies, node_forces, scratch_d;
+
+    int K() const { return hm.K; }
+    int NLM() const { return hm.num_LM; }
+    int NE() const { return hm.num_lme; }
+
+    explicit Engine(HostModel&& m, int prec)
+    {
+        hm = std::move(m);
+        precision = prec;
+        hipStream_t s = nullptr;
+        auto cat = [](const std::vector<std::vector<double>>& t) {
+            std::vector<double> out;
+            for (auto& v : t) out.insert(out.end(), v.begin(), v.end());
+            return out;
+        };
+        upload_as(tab0, cat(hm.tables0), s);
+        upload_as(tab1, cat(hm.tables1), s);
+        upload_as(pair_table0, hm.pair_table0, s);
+        upload_as(pair_table1, hm.pair_table1, s);
+        upload_as(H0, hm.H0_weights, s);
+        upload_as(A0w, hm.A0_weights, s);
+        upload_as(H1w, hm.H1_weights, s);
+        {
+            std::vector<double> all;
+            for (auto& w : hm.A1_weights) { A1w_off.push_back((long)all.size()); all.insert(all.end(), w.begin(), w.end()); }
+            upload_as(A1w, all, s);
+        }
+        // layer 0 couples Y_lm straight into output slot lm
+        {
+            std::vector<int> st(17), lm(16);
+            std::vector<double> c(16, 1.0);
+            for (int q = 0; q < 16; ++q) { st[q] = q; lm[q] = q; }
+            st[16] = 16;
+            upload_as(B0_start, st, s); upload_as(B0_lm1, lm, s); upload_as(B0_c, c, s);
+        }
+        upload_as(B1_start, hm.B_start, s);
+        upload_as(B1_lm1, hm.B_lm1, s);
+        upload_as(B1_c, hm.B_c, s);
+        upload_as(H2w_H1, hm.H2_weights_for_H1, s);
+        upload_as(H2w_M1, hm.H2_weights_for_M1, s);
+        upload_as(ro1, hm.readout_1_weights, s);
+        upload_as(ro2_w1, hm.readout_2_w1, s);
+        upload_as(ro2_w2, hm.readout_2_w2, s);
+        upload_as(E0, hm.atomic_energies, s);
+        auto up_poly = [&](DevPoly& d, const PolySpec& p) {
+            upload_as(d.row_i0, p.row_i0, s); upload_as(d.row_i1, p.row_i1, s);
+            upload_as(d.row_start, p.row_start, s); upload_as(d.entry_var, p.entry_var, s);
+            upload_as(d.coef, p.coef, s);
+            d.num_rows = (int)p.row_i0.size(); d.num_entries = p.num_entries;
+        };
+        std::vector<const int*> vi0, vi1, vst, vvar;
+        std::vector<const F*> vco;
+        std::vector<int> vnr, vne;
+        auto reg = [&](DevPoly& d) {
+            vi0.push_back(d.row_i0.p); vi1.push_back(d.row_i1.p); vst.push_back(d.row_start.p);
+            vvar.push_back(d.entry_var.p); vco.push_back(d.coef.p); vnr.push_back(d.num_rows); vne.push_back(d.num_entries);
+        };
+        for (int LM = 0; LM < hm.num_LM; ++LM) {
+            P0.emplace_back(new DevPoly());
+            up_poly(*P0.back(), hm.P0[LM]);
+            reg(*P0.back());
+        }
+        up_poly(P1, hm.P1);
+        reg(P1);
+        pp_i0.upload(vi0.data(), vi0.size(), s); pp_i1.upload(vi1.data(), vi1.size(), s);
+        pp_start.upload(vst.data(), vst.size(), s); pp_var.upload(vvar.data(), vvar.size(), s);
+        pp_coef.upload(vco.data(), vco.size(), s);
+        pp_nrows.upload(vnr.data(), vnr.size(), s); pp_nent.upload(vne.data(), vne.size(), s);
+        flags.resize(4, s);
+        HIPCHK(hipStreamSynchronize(s));
+    }
+
+    // ------------------------------------------------------------------
+    // geometry handling
+    void set_geometry_ptrs(int N, const int* nt, const int* nn, const int* ni, const int* nty, const double* x,
+                           const double* rr, long E_, bool on_device)
+    {
+        hipStream_t s = stream;
+        if (on_device) {
+            if (nt) node_types = nt;
+            if (nn) num_neigh = nn;
+            if (ni) neigh_indices = ni;
+            if (nty) neigh_types = nty;
+            if (x) xyz = x;
+            if (rr) r = rr;
+        } else {
+            if (nt) { g_node_types.upload(nt, N, s); node_types = g_node_types.p; }
+            if (nn) { g_num_neigh.upload(nn, N, s); num_neigh = g_num_neigh.p; }
+            if (ni) { g_neigh_indices.upload(ni, E_, s); neigh_indices = g_neigh_indices.p; }
+            if (nty) { g_neigh_types.upload(nty, E_, s); neigh_types = g_neigh_types.p; }
+            if (x) { g_xyz.upload(x, 3 * E_, s); xyz = g_xyz.p; }
+            if (rr) { g_r.upload(rr, E_, s); r = g_r.p; }
+        }
+        if (E_ >= 0) E = E_;
+    }
+    void build_first_neigh(int N)
+    {
+        hipStream_t s = stream;
+        first_neigh.size_to((size_t)N + 1, s);
+        scan_tmp.size_to((size_t)N / 1024 + 2, s);
+        HIPCHK(launch_scan_exclusive(num_neigh, first_neigh.p, N, scan_tmp.p, s));
+        N_geo = N;
+    }
+    void build_type_groups(int N)
+    {
+        hipStream_t s = stream;
+        const int T = hm.T;
+        t_count.size_to(T, s); t_start.size_to((size_t)T + 1, s); t_cursor.size_to(T, s); t_perm.size_to(N, s);
+        scan_tmp.size_to((size_t)std::max(N, T) / 1024 + 2, s);
+        HIPCHK(launch_type_groups(node_types, N, T, t_count.p, t_start.p, t_cursor.p, t_perm.p, scan_tmp.p, s));
+    }
+    void build_sender_lists(int rows)
+    {
+        hipStream_t s = stream;
+        s_count.size_to(rows, s); s_start.size_to((size_t)rows + 1, s); s_cursor.size_to(rows, s);
+        s_list.size_to((size_t)E, s);
+        scan_tmp.size_to((size_t)rows / 1024 + 2, s);
+        HIPCHK(launch_sender_lists(neigh_indices, (int)E, rows, s_count.p, s_start.p, s_cursor.p, s_list.p, scan_tmp.p, s));
+        sender_rows = rows;
+    }
+    // Host-path validation of what the reference leaves unchecked (mace.cpp:17-64 trusts
+    // its caller; cubic_spline_set.cpp:54 reads past the table for r >= r_cut).
+    void validate(int N, int rows)
+    {
+        hipStream_t s = stream;
+        HIPCHK(hipMemsetAsync(flags.p, 0, sizeof(int), s));
+        HIPCHK(launch_check_range(node_types, N, hm.T, flags.p, s));
+        HIPCHK(launch_check_range(neigh_types, E, hm.T, flags.p, s));
+        HIPCHK(launch_check_range(neigh_indices, E, rows, flags.p, s));
+        HIPCHK(launch_check_r(r, E, hm.r_cut, flags.p, s));
+        int f = 0;
+        HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, s));
+        HIPCHK(hipStreamSynchronize(s));
+        if (f & 1) throw Error(SMX_EINVAL, "node_types / neigh_types / neigh_indices hold an index outside the model or the node range");
+        if (f & 2) throw Error(SMX_ERANGE, "an edge length lies outside (0, r_cut): the radial spline tables do not cover it");
+    }
+    int edges_from_counts_check(int N, const int* host_num_neigh, long E_)
+    {
+        long tot = 0;
+        for (int i = 0; i < N; ++i) {
+            if (host_num_neigh[i] < 0) throw Error(SMX_EINVAL, "negative num_neigh entry");
+            tot += host_num_neigh[i];
+        }
+        if (tot != E_) throw Error(SMX_EINVAL, "sum(num_neigh) does not match the number of edges");
+        return 0;
+    }
+
+    // ------------------------------------------------------------------
+    AggParams<F> agg_params(int layer, int N)
+    {
+        AggParams<F> p{};
+        p.num_nodes = N; p.K = hm.K;
+        p.first_neigh = first_neigh.p; p.node_types = node_types; p.neigh_types = neigh_types;
+        p.xyz = xyz; p.r = r; p.T = hm.T; p.spl_nodes = hm.spl_nodes; p.spl_h = hm.spl_h;
+        if (layer == 0) {
+            p.gather = neigh_types; p.Hsrc = H0.p; p.tab = tab0.p; p.pair_table = pair_table0.p;
+            p.B_start = B0_start.p; p.B_lm1 = B0_lm1.p; p.B_c = B0_c.p;
+        } else {
+            p.gather = neigh_indices; p.Hsrc = H1.p; p.tab = tab1.p; p.pair_table = pair_table1.p;
+            p.B_start = B1_start.p; p.B_lm1 = B1_lm1.p; p.B_c = B1_c.p;
+        }
+        return p;
+    }
+    void need(const void* p, const char* what)
+    {
+        if (!p) throw Error(SMX_EINVAL, std::string("stage called before its inputs exist: ") + what);
+    }
+
+    // ---- stages ------------------------------------------------------
+    void st_agg0_fwd(int N)
+    {
+        need(xyz, "xyz (compute_Y)"); need(r, "r (compute_R0)"); need(first_neigh.p, "num_neigh");
+        Phi0.size_to((size_t)N * 16 * K(), stream);
+        auto p = agg_params(0, N);
+        p.out = Phi0.p;
+        HIPCHK(launch_agg_fwd<F>(0, p, stream));
+    }
+    template <typename TA, typename TC, typename CT>
+    GemmParams<TA, TC, CT> gemm_base(const TA* A, long a_stride, TC* C, long c_stride, const CT* W, long w_type_stride,
+                                     bool typed, int N, int transW, int accumulate)
+    {
+        GemmParams<TA, TC, CT> g{};
+        g.A = A; g.a_node_stride = a_stride; g.C = C; g.c_node_stride = c_stride; g.W = W;
+        g.w_type_stride = w_type_stride; g.transW = transW; g.accumulate = accumulate; g.num_nodes = N;
+        if (typed) { g.node_types = node_types; g.perm = t_perm.p; g.tstart = t_start.p; g.T = hm.T; }
+        return g;
+    }
+    // A0[i, l-block] = Phi0[i, l-block] . A0_weights[type_i][l]  (reverse: transposed weights)
+    void st_A0_lin(int N, bool reverse)
+    {
+        const int k = K();
+        const F* src = reverse ? A0_adj.p : Phi0.p;
+        if (reverse) Phi0.size_to((size_t)N * 16 * k, stream); else A0.size_to((size_t)N * 16 * k, stream);
+        F* dst = reverse ? Phi0.p : A0.p;
+        auto g = gemm_base<F, F, F>(src, 16L * k, dst, 16L * k, A0w.p, 4L * k * k, true, N, reverse ? 1 : 0, 0);
+        g.nprob = 4;
+        for (int l = 0; l < 4; ++l)
+            g.prob[l] = GemmProb{(long)l * l * k, k, (long)l * l * k, k, (long)l * k * k, k, k, 2 * l + 1};
+        HIPCHK((launch_gemm<F, F, F>(g, stream)));
+    }
+    void st_poly(int N, bool layer1)
+    {
+        PolyParams<F> p{};
+        p.num_nodes = N; p.K = K(); p.node_types = node_types;
+        const int off = layer1 ? NLM() : 0;
+        p.NP = layer1 ? 1 : NLM();
+        if (layer1) {
+            M1.size_to((size_t)N * K(), stream); M1_grad.size_to((size_t)N * 16 * K(), stream);
+            p.A = A1.p; p.M = M1.p; p.M_grad = M1_grad.p;
+        } else {
+            M0.size_to((size_t)N * NLM() * K(), stream); M0_grad.size_to((size_t)N * NLM() * 16 * K(), stream);
+            p.A = A0.p; p.M = M0.p; p.M_grad = M0_grad.p;
+        }
+        p.row_i0 = pp_i0.p + off; p.row_i1 = pp_i1.p + off; p.row_start = pp_start.p + off;
+        p.entry_var = pp_var.p + off; p.coef = pp_coef.p + off; p.num_rows = pp_nrows.p + off; p.num_entries = pp_nent.p + off;
+        HIPCHK(launch_poly<F>(p, stream));
+    }
+    void st_H1(int N, bool reverse)
+    {
+        const int k = K(), nlm = NLM();
+        if (reverse) M0_adj.size_to(M0.n, stream);
+        else if (H1.n != M0.n) H1.resize(M0.n, stream);   // mace.cpp:400
+        auto g = gemm_base<F, F, F>(reverse ? H1_adj.p : M0.p, (long)nlm * k, reverse ? M0_adj.p : H1.p, (long)nlm * k,
+                                    H1w.p, 0, false, N, reverse ? 1 : 0, 0);
+        g.nprob = hm.L_max + 1;
+        for (int l = 0; l <= hm.L_max; ++l)
+            g.prob[l] = GemmProb{(long)l * l * k, k, (long)l * l * k, k, (long)l * k * k, k, k, 2 * l + 1};
+        HIPCHK((launch_gemm<F, F, F>(g, stream)));
+    }
+    void st_agg1_fwd(int N)
+    {
+        need(xyz, "xyz (compute_Y)"); need(r, "r (compute_R1)"); need(neigh_indices, "neigh_indices");
+        Phi1.size_to((size_t)N * NE() * K(), stream);
+        auto p = agg_params(1, N);
+        p.out = Phi1.p;
+        HIPCHK(launch_agg_fwd<F>(hm.L_max, p, stream));
+    }
+    void st_A1(int N, bool reverse)
+    {
+        const int k = K(), ne = NE();
+        if (reverse) dPhi1.size_to(Phi1.n, stream); else A1.size_to((size_t)N * 16 * k, stream);
+        long lme_off = 0;
+        if (!reverse) {
+            auto g = gemm_base<F, F, F>(Phi1.p, (long)ne * k, A1.p, 16L * k, A1w.p, 0, false, N, 0, 0);
+            g.nprob = 4;
+            for (int l = 0; l < 4; ++l) {
+                const int nel = hm.num_e[l];
+                g.prob[l] = GemmProb{lme_off * k, (long)nel * k, (long)l * l * k, k, A1w_off[l], nel * k, k, 2 * l + 1};
+                lme_off += (2 * l + 1) * nel;
+            }
+            HIPCHK((launch_gemm<F, F, F>(g, stream)));
+        } else {
+            auto g = gemm_base<F, F, F>(A1_adj.p, 16L * k, dPhi1.p, (long)ne * k, A1w.p, 0, false, N, 1, 0);
+            g.nprob = 4;
+            for (int l = 0; l < 4; ++l) {
+                const int nel = hm.num_e[l];
+                g.prob[l] = GemmProb{(long)l * l * k, k, lme_off * k, (long)nel * k, A1w_off[l], k, nel * k, 2 * l + 1};
+                lme_off += (2 * l + 1) * nel;
+            }
+            HIPCHK((launch_gemm<F, F, F>(g, stream)));
+        }
+    }
+    void st_H2(int N)
+    {
+        const int k = K(), nlm = NLM();
+        H2.size_to((size_t)N * k, stream);
+        auto g1 = gemm_base<F, double, double>(H1.p, (long)nlm * k, H2.p, k, H2w_H1.p, (long)k * k, true, N, 0, 0);
+        g1.nprob = 1; g1.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
+        HIPCHK((launch_gemm<F, double, double>(g1, stream)));
+        auto g2 = gemm_base<F, double, double>(M1.p, k, H2.p, k, H2w_M1.p, 0, false, N, 0, 1);
+        g2.nprob = 1; g2.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
+        HIPCHK((launch_gemm<F, double, double>(g2, stream)));
+    }
+    void st_reverse_H2(int N, bool zero_H1_adj)
+    {
+        const int k = K(), nlm = NLM();
+        H1_adj.resize(H1.n, stream); M1_adj.size_to(M1.n, stream);
+        if (zero_H1_adj) HIPCHK(hipMemsetAsync(H1_adj.p, 0, H1_adj.n * sizeof(F), stream));
+        auto g1 = gemm_base<double, F, double>(H2_adj.p, k, H1_adj.p, (long)nlm * k, H2w_H1.p, (long)k * k, true, N, 1, 1);
+        g1.nprob = 1; g1.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
+        HIPCHK((launch_gemm<double, F, double>(g1, stream)));
+        auto g2 = gemm_base<double, F, double>(H2_adj.p, k, M1_adj.p, k, H2w_M1.p, 0, false, N, 1, 0);
+        g2.nprob = 1; g2.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
+        HIPCHK((launch_gemm<double, F, double>(g2, stream)));
+    }
+    void st_readouts(int N, bool zero_energies)
+    {
+        const int k = K(), nlm = NLM();
+        node_energies.resize((size_t)N, stream);
+        H1_adj.size_to(H1.n, stream);
+        H2_adj.size_to(H2.n, stream);
+        hidden.size_to((size_t)N * 16, stream);
+        const int rows = (int)(H1.n / ((size_t)nlm * k));
+        HIPCHK(launch_seed_H1_adj<F>(rows, N, nlm, k, ro1.p, H1_adj.p, stream));
+        auto g1 = gemm_base<double, double, double>(H2.p, k, hidden.p, 16, ro2_w1.p, 0, false, N, 1, 0);
+        g1.nprob = 1; g1.prob[0] = GemmProb{0, 0, 0, 0, 0, k, 16, 1};
+        HIPCHK((launch_gemm<double, double, double>(g1, stream)));
+        HIPCHK(launch_readout<F>(N, k, nlm, node_types, E0.p, ro1.p, H1.p, hidden.p, ro2_w2.p, hm.readout_2_scale,
+                                 node_energies.p, zero_energies ? 1 : 0, stream));
+        auto g2 = gemm_base<double, double, double>(hidden.p, 16, H2_adj.p, k, ro2_w1.p, 0, false, N, 0, 0);
+        g2.nprob = 1; g2.prob[0] = GemmProb{0, 0, 0, 0, 0, 16, k, 1};
+        HIPCHK((launch_gemm<double, double, double>(g2, stream)));
+    }
+    void st_reverse_M1(int N)
+    {
+        A1_adj.size_to(A1.n, stream);
+        HIPCHK(launch_poly_reverse<F>(N, 1, K(), M1_grad.p, M1_adj.p, A1_adj.p, stream));
+    }
+    void st_reverse_M0(int N)
+    {
+        A0_adj.size_to(A0.n, stream);
+        if (A0.n > (size_t)N * 16 * K())
+            HIPCHK(hipMemsetAsync(A0_adj.p, 0, A0_adj.n * sizeof(F), stream));  // mace.cpp:376-377
+        HIPCHK(launch_poly_reverse<F>(N, NLM(), K(), M0_grad.p, M0_adj.p, A0_adj.p, stream));
+    }
+    void st_agg1_bwd(int N, bool zero_dxyz, bool zero_H1_adj)
+    {
+        need(xyz, "xyz"); need(r, "r"); need(neigh_indices, "neigh_indices");
+        const int k = K(), nlm = NLM();
+        node_forces.resize((size_t)3 * E, stream);
+        msg.size_to((size_t)E * nlm * k, stream);
+        auto p = agg_params(1, N);
+        p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
+        stage_begin(ST_AGG1B);
+        HIPCHK(launch_agg_bwd<F>(hm.L_max, p, stream));
+        stage_end(ST_AGG1B);
+        // edges beyond the first N receivers carry no layer-1 adjoint
+        const long EN = E;  // first_neigh[N] == E whenever the list covers exactly N receivers
+        (void)EN;
+        stage_begin(ST_SRED);
+        H1_adj.resize(H1.n, stream);
+        const int rows = (int)(H1.n / ((size_t)nlm * k));
+        if (sender_rows != rows) build_sender_lists(rows);
+        HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, stream));
+        stage_end(ST_SRED);
+    }
+    void st_agg0_bwd(int N)
+    {
+        need(xyz, "xyz"); need(r, "r");
+        node_forces.resize((size_t)3 * E, stream);
+        auto p = agg_params(0, N);
+        p.d_out = Phi0.p; p.forces = node_forces.p; p.accumulate_forces = 1; p.msg = nullptr;
+        HIPCHK(launch_agg_bwd<F>(0, p, stream));
+    }
+
+    // ------------------------------------------------------------------
+    void compute(int N, const int* nt, const int* nn, const int* ni, const int* nty, const double* x,
+                 const double* rr, long E_, bool on_device, double* d_energies, double* d_forces) override
+    {
+        if (N < 0 || E_ < 0) throw Error(SMX_EINVAL, "negative num_nodes or num_edges");
+        if (hm.has_zbl || hm.A0_scaled || hm.A1_scaled)
+            throw Error(SMX_EUNSUPPORTED, "models with ZBL or density normalisation are not implemented on the device yet");
+        if (!on_device) edges_from_counts_check(N, nn, E_);
+        stage_begin(ST_PREP);
+        set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, on_device);
+        build_first_neigh(N);
+        build_type_groups(N);
+        sender_rows = -1;
+        if (!on_device) validate(N, N);
+        build_sender_lists(N);
+        stage_end(ST_PREP);
+
+        node_energies.size_to((size_t)N, stream);
+        node_forces.size_to((size_t)3 * E, stream);
+        if (N == 0) return;
+
+        stage_begin(ST_AGG0F); st_agg0_fwd(N); stage_end(ST_AGG0F);
+        stage_begin(ST_A0LIN); st_A0_lin(N, false); stage_end(ST_A0LIN);
+        stage_begin(ST_M0); st_poly(N, false); stage_end(ST_M0);
+        stage_begin(ST_H1); st_H1(N, false); stage_end(ST_H1);
+        stage_begin(ST_AGG1F); st_agg1_fwd(N); stage_end(ST_AGG1F);
+        stage_begin(ST_A1); st_A1(N, false); stage_end(ST_A1);
+        stage_begin(ST_M1); st_poly(N, true); stage_end(ST_M1);
+        stage_begin(ST_H2); st_H2(N); stage_end(ST_H2);
+        stage_begin(ST_READOUT); st_readouts(N, true); stage_end(ST_READOUT);
+        stage_begin(ST_REVH2); st_reverse_H2(N, false); stage_end(ST_REVH2);
+        stage_begin(ST_REVM1); st_reverse_M1(N); stage_end(ST_REVM1);
+        stage_begin(ST_REVA1); st_A1(N, true); stage_end(ST_REVA1);
+        st_agg1_bwd(N, true, false);
+        stage_begin(ST_REVH1); st_H1(N, true); stage_end(ST_REVH1);
+        stage_begin(ST_REVM0); st_reverse_M0(N); stage_end(ST_REVM0);
+        stage_begin(ST_REVA0LIN); st_A0_lin(N, true); stage_end(ST_REVA0LIN);
+        stage_begin(ST_AGG0B); st_agg0_bwd(N); stage_end(ST_AGG0B);
+
+        if (d_energies) HIPCHK(hipMemcpyAsync(d_energies, node_energies.p, (size_t)N * sizeof(double), hipMemcpyDeviceToDevice, stream));
+        if (d_forces && E) HIPCHK(hipMemcpyAsync(d_forces, node_forces.p, (size_t)3 * E * sizeof(double), hipMemcpyDeviceToDevice, stream));
+    }
+
+    // stage-level entry points (host arrays)
+    void stage(const char* name, int N, const int* nt, const int* nn, const int* ni, const int* nty,
+               const double* x, const double* rr, long E_, int fa, int fb) override
+    {
+        const std::string s(name);
+        if (N < 0) throw Error(SMX_EINVAL, "negative num_nodes");
+        if (hm.has_zbl || hm.A0_scaled || hm.A1_scaled)
+            throw Error(SMX_EUNSUPPORTED, "models with ZBL or density normalisation are not implemented on the device yet");
+        if (nn && E_ >= 0) edges_from_counts_check(N, nn, E_);
+        set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, false);
+        if (nn) build_first_neigh(N);
+        if (s == "Y" || s == "R0" || s == "R1") return;  // geometry remembered; evaluated inside the fused kernels
+        if (s == "A0") { build_type_groups(N); st_agg0_fwd(N); st_A0_lin(N, false); }
+        else if (s == "reverse_A0") { build_type_groups(N); st_A0_lin(N, true); st_agg0_bwd(N); }
+        else if (s == "M0") st_poly(N, false);
+        else if (s == "reverse_M0") st_reverse_M0(N);
+        else if (s == "H1") st_H1(N, false);
+        else if (s == "reverse_H1") st_H1(N, true);
+        else if (s == "Phi1") { need(node_types, "node_types (compute_R1)"); st_agg1_fwd(N); }
+        else if (s == "reverse_Phi1") { sender_rows = -1; st_agg1_bwd(N, fa != 0, fb != 0); }
+        else if (s == "A1") st_A1(N, false);
+        else if (s == "reverse_A1") st_A1(N, true);
+        else if (s == "M1") st_poly(N, true);
+        else if (s == "reverse_M1") st_reverse_M1(N);
+        else if (s == "H2") { build_type_groups(N); st_H2(N); }
+        else if (s == "reverse_H2") { build_type_groups(N); st_reverse_H2(N, fa != 0); }
+        else if (s == "readouts") st_readouts(N, false);
+        else throw Error(SMX_EINVAL, "unknown stage " + s);
+    }
+
+    // ------------------------------------------------------------------
+    struct Named { DVec<F>* f; DVec<double>* d; };
+    Named find(const std::string& n)
+    {
+        if (n == "A0") return {&A0, nullptr};
+        if (n == "A0_adj") return {&A0_adj, nullptr};
+        if (n == "M0") return {&M0, nullptr};
+        if (n == "M0_grad") return {&M0_grad, nullptr};
+        if (n == "M0_adj") return {&M0_adj, nullptr};
+        if (n == "H1") return {&H1, nullptr};
+        if (n == "H1_adj") return {&H1_adj, nullptr};
+        if (n == "Phi0") return {&Phi0, nullptr};
+        if (n == "Phi1") return {&Phi1, nullptr};
+        if (n == "Phi1_adj" || n == "dPhi1") return {&dPhi1, nullptr};
+        if (n == "A1") return {&A1, nullptr};
+        if (n == "A1_adj") return {&A1_adj, nullptr};
+        if (n == "M1") return {&M1, nullptr};
+        if (n == "M1_grad") return {&M1_grad, nullptr};
+        if (n == "M1_adj") return {&M1_adj, nullptr};
+        if (n == "H0_weights") return {&H0, nullptr};
+        if (n == "H2") return {nullptr, &H2};
+        if (n == "H2_adj") return {nullptr, &H2_adj};
+        if (n == "node_energies") return {nullptr, &node_energies};
+        if (n == "node_forces") return {nullptr, &node_forces};
+        return {nullptr, nullptr};
+    }
+    void get_array(const char* name, double* out, long cap, long* n) override
+    {
+        const std::string s(name);
+        hipStream_t st = stream;
+        const double* src = nullptr;
+        size_t len = 0;
+        if (s == "Y" || s == "Y_grad") {
+            need(xyz, "xyz (compute_Y)");
+            scratch_d.size_to((size_t)E * 64, st);
+            HIPCHK(launch_sph_harm(xyz, E, scratch_d.p, scratch_d.p + (size_t)E * 16, st));
+            src = s == "Y" ? scratch_d.p : scratch_d.p + (size_t)E * 16;
+            len = s == "Y" ? (size_t)E * 16 : (size_t)E * 48;
+        } else if (s == "R0" || s == "R1") {
+            need(r, "r (compute_R0/R1)"); need(first_neigh.p, "num_neigh"); need(node_types, "node_types");
+            const bool l1 = s == "R1";
+            const int nspl = l1 ? hm.nspl1 : hm.nspl0;
+            scratch_d.size_to((size_t)E * nspl, st);
+            HIPCHK(launch_radial<F>(N_geo, first_neigh.p, node_types, neigh_types, r, l1 ? tab1.p : tab0.p,
+                                    l1 ? pair_table1.p : pair_table0.p, hm.T, hm.spl_nodes, hm.spl_h, nspl, scratch_d.p, st));
+            src = scratch_d.p; len = (size_t)E * nspl;
+        } else {
+            Named v = find(s);
+            if (!v.f && !v.d) throw Error(SMX_EINVAL, "unknown array '" + s + "'");
+            if (v.d) { src = v.d->p; len = v.d->n; }
+            else {
+                len = v.f->n;
+                if (std::is_same<F, double>::value) src = reinterpret_cast<const double*>(v.f->p);
+                else {
+                    scratch_d.size_to(len, st);
+                    HIPCHK((launch_convert<F, double>(v.f->p, scratch_d.p, (long)len, st)));
+                    src = scratch_d.p;
+                }
+            }
+        }
+        if (n) *n = (long)len;
+        if (out && cap > 0 && len > 0) {
+            const size_t m = std::min((size_t)cap, len);
+            HIPCHK(hipMemcpyAsync(out, src, m * sizeof(double), hipMemcpyDeviceToHost, st));
+        }
+        HIPCHK(hipStreamSynchronize(st));
+    }
+    void set_array(const char* name, const double* in, long n) override
+    {
+        const std::string s(name);
+        hipStream_t st = stream;
+        if (n < 0) throw Error(SMX_EINVAL, "negative length");
+        Named v = find(s);
+        if ((!v.f && !v.d) || s == "H0_weights" || s == "M0_grad" || s == "M1_grad")
+            throw Error(SMX_EINVAL, "array '" + s + "' cannot be set");
+        if (v.d) { v.d->upload(in, (size_t)n, st); }
+        else if (std::is_same<F, double>::value) { reinterpret_cast<DVec<double>*>(v.f)->upload(in, (size_t)n, st); }
+        else {
+            scratch_d.upload(in, (size_t)n, st);
+            v.f->size_to((size_t)n, st);
+            HIPCHK((launch_convert<double, F>(scratch_d.p, v.f->p, n, st)));
+        }
+        HIPCHK(hipStreamSynchronize(st));
+    }
+
+    // ------------------------------------------------------------------
+    DVec<int> rf_send, rf_recv, rf_count, rf_sstart, rf_cursor, rf_slist, rf_rstart, rf_rlist;
+    DVec<double> rf_out;
+    void reduce_forces(int num_atoms, const int* sender_atom, const int* receiver_atom, double* atom_forces,
+                       double* virial) override
+    {
+        hipStream_t s = stream;
+        need(node_forces.p, "node_forces");
+        if (node_forces.n != (size_t)3 * E) throw Error(SMX_EINVAL, "node_forces does not match the current edge list");
+        if (atom_forces) {
+            if (num_atoms <= 0) throw Error(SMX_EINVAL, "num_atoms must be positive");
+            if (!sender_atom) throw Error(SMX_EINVAL, "sender_atom is required");
+            rf_send.upload(sender_atom, (size_t)E, s);
+            rf_count.size_to(num_atoms, s); rf_cursor.size_to(num_atoms, s);
+            rf_sstart.size_to((size_t)num_atoms + 1, s); rf_slist.size_to((size_t)E, s);
+            scan_tmp.size_to((size_t)num_atoms / 1024 + 2, s);
+            HIPCHK(hipMemsetAsync(flags.p, 0, sizeof(int), s));
+            HIPCHK(launch_check_range(rf_send.p, E, num_atoms, flags.p, s));
+            const int* rstart = nullptr;
+            const int* rlist = nullptr;
+            if (receiver_atom) {
+                // receiver_atom[i] = atom row of receiver block i -> expand to edges
+                std::vector<int> hn(N_geo), hr((size_t)E);
+                HIPCHK(hipMemcpyAsync(hn.data(), num_neigh, (size_t)N_geo * sizeof(int), hipMemcpyDeviceToHost, s));
+                HIPCHK(hipStreamSynchronize(s));
+                size_t e = 0;
+                for (int i = 0; i < N_geo; ++i) {
+                    if (receiver_atom[i] < 0 || receiver_atom[i] >= num_atoms) throw Error(SMX_EINVAL, "receiver_atom out of range");
+                    for (int j = 0; j < hn[i]; ++j) hr[e++] = receiver_atom[i];
+                }
+                rf_recv.upload(hr.data(), hr.size(), s);
+                HIPCHK(hipStreamSynchronize(s));
+                rf_rstart.size_to((size_t)num_atoms + 1, s); rf_rlist.size_to((size_t)E, s);
+                HIPCHK(launch_sender_lists(rf_recv.p, (int)E, num_atoms, rf_count.p, rf_rstart.p, rf_cursor.p, rf_rlist.p, scan_tmp.p, s));
+                rstart = rf_rstart.p; rlist = rf_rlist.p;
+            } else {
+                if (num_atoms < N_geo) throw Error(SMX_EINVAL, "num_atoms is smaller than the number of receivers");
+                // receiver block i is atom i: CSR offsets padded with E for atoms beyond the receivers
+                std::vector<int> h((size_t)num_atoms + 1);
+                HIPCHK(hipMemcpyAsync(h.data(), first_neigh.p, ((size_t)N_geo + 1) * sizeof(int), hipMemcpyDeviceToHost, s));
+                HIPCHK(hipStreamSynchronize(s));
+                for (int i = N_geo + 1; i <= num_atoms; ++i) h[i] = h[N_geo];
+                rf_rstart.upload(h.data(), h.size(), s);
+                HIPCHK(hipStreamSynchronize(s));
+                rstart = rf_rstart.p;
+            }
+            int f = 0;
+            HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, s));
+            HIPCHK(hipStreamSynchronize(s));
+            if (f) throw Error(SMX_EINVAL, "sender_atom out of range");
+            HIPCHK(launch_sender_lists(rf_send.p, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, s));
+            rf_out.size_to((size_t)3 * num_atoms, s);
+            HIPCHK(launch_force_scatter(num_atoms, rstart, rlist, rf_sstart.p, rf_slist.p, node_forces.p, rf_out.p, s));
+            HIPCHK(hipMemcpyAsync(atom_forces, rf_out.p, (size_t)3 * num_atoms * sizeof(double), hipMemcpyDeviceToHost, s));
+            HIPCHK(hipStreamSynchronize(s));
+        }
+        if (virial) {
+            const int nb = 64;
+            scratch_d.size_to((size_t)nb * 6, s);
+            HIPCHK(launch_virial(E, xyz, node_forces.p, scratch_d.p, nb, s));
+            std::vector<double> part((size_t)nb * 6);
+            HIPCHK(hipMemcpyAsync(part.data(), scratch_d.p, part.size() * sizeof(double), hipMemcpyDeviceToHost, s));
+            HIPCHK(hipStreamSynchronize(s));
+            for (int q = 0; q < 6; ++q) {
+                double v = 0;
+                for (int b = 0; b < nb; ++b) v += part[(size_t)b * 6 + q];
+                virial[q] = v;
+            }
+        }
+    }
+};
+
+}  // namespace smx
+
+// ===========================================================================
+struct smx_model {
+    std::unique_ptr<smx::EngineBase> eng;
+};
+
+namespace {
+
+template <typename Fn>
+int guarded(Fn&& fn)
+{
+    try {
+        fn();
+        return SMX_OK;
+    } catch (const smx::Error& e) {
+        smx::g_last_error = e.what();
+        return e.code;
+    } catch (const smx::JsonError& e) {
+        smx::g_last_error = e.what();
+        return SMX_EFILE;
+    } catch (const std::bad_alloc&) {
+        smx::g_last_error = "out of host memory";
+        return SMX_ENOMEM;
+    } catch (const std::exception& e) {
+        const std::string w = e.what();
+        smx::g_last_error = w;
+        return w.rfind("unsupported:", 0) == 0 ? SMX_EUNSUPPORTED : SMX_EINVAL;
+    }
+}
+
+void require_device()
+{
+    int n = 0;
+    hipError_t e = hipGetDeviceCount(&n);
+    if (e != hipSuccess || n <= 0)
+        throw smx::Error(SMX_ENODEVICE, "no HIP device available: this engine has no CPU path");
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess) throw smx::Error(SMX_ENODEVICE, "hipGetDevice failed");
+    hipDeviceProp_t prop;
+    if (hipGetDeviceProperties(&prop, dev) != hipSuccess) throw smx::Error(SMX_ENODEVICE, "hipGetDeviceProperties failed");
+    if (std::string(prop.gcnArchName).rfind("gfx950", 0) != 0)
+        throw smx::Error(SMX_ENODEVICE, std::string("kernels are built for gfx950 only; found ") + prop.gcnArchName);
+}
+
+smx::EngineBase& E(smx_model* m)
+{
+    if (!m || !m->eng) throw smx::Error(SMX_EINVAL, "null model");
+    return *m->eng;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char* smx_last_error(void) { return smx::g_last_error.c_str(); }
+
+int smx_model_load(const char* json_path, int flags, smx_model** out)
+{
+    return guarded([&] {
+        if (!json_path || !out) throw smx::Error(SMX_EINVAL, "null argument");
+        if (flags != SMX_FP64 && flags != SMX_FP32_FEATURES) throw smx::Error(SMX_EINVAL, "unknown precision flag");
+        *out = nullptr;
+        smx::HostModel hm = smx::load_host_model(json_path);
+        require_device();
+        std::unique_ptr<smx_model> m(new smx_model());
+        if (flags == SMX_FP64) m->eng.reset(new smx::Engine<double>(std::move(hm), flags));
+        else m->eng.reset(new smx::Engine<float>(std::move(hm), flags));
+        *out = m.release();
+    });
+}
+
+void smx_model_free(smx_model* m)
+{
+    if (!m) return;
+    (void)hipDeviceSynchronize();
+    delete m;
+}
+
+int smx_model_get_int(const smx_model* m, const char* key, int* out)
+{
+    return guarded([&] {
+        if (!m || !key || !out) throw smx::Error(SMX_EINVAL, "null argument");
+        const smx::HostModel& h = m->eng->hm;
+        const std::string k(key);
+        if (k == "num_elements") *out = h.T;
+        else if (k == "num_channels") *out = h.K;
+        else if (k == "l_max") *out = h.l_max;
+        else if (k == "num_lm") *out = h.num_lm;
+        else if (k == "L_max") *out = h.L_max;
+        else if (k == "num_LM") *out = h.num_LM;
+        else if (k == "has_zbl") *out = h.has_zbl ? 1 : 0;
+        else if (k == "num_lme") *out = h.num_lme;
+        else if (k == "num_lelm1lm2") *out = h.num_lelm1lm2;
+        else if (k == "precision") *out = m->eng->precision;
+        else if (k == "num_radial_tables_0") *out = (int)h.tables0.size();
+        else if (k == "num_radial_tables_1") *out = (int)h.tables1.size();
+        else throw smx::Error(SMX_EINVAL, "unknown integer key '" + k + "'");
+    });
+}
+
+int smx_model_get_double(const smx_model* m, const char* key, double* out)
+{
+    return guarded([&] {
+        if (!m || !key || !out) throw smx::Error(SMX_EINVAL, "null argument");
+        const std::string k(key);
+        if (k == "r_cut") *out = m->eng->hm.r_cut;
+        else throw smx::Error(SMX_EINVAL, "unknown double key '" + k + "'");
+    });
+}
+
+int smx_model_get_atomic_numbers(const smx_model* m, int* out, int cap, int* n)
+{
+    return guarded([&] {
+        if (!m) throw smx::Error(SMX_EINVAL, "null model");
+        const auto& v = m->eng->hm.atomic_numbers;
+        if (n) *n = (int)v.size();
+        for (int i = 0; out && i < cap && i < (int)v.size(); ++i) out[i] = v[i];
+    });
+}
+int smx_model_get_atomic_energies(const smx_model* m, double* out, int cap, int* n)
+{
+    return guarded([&] {
+        if (!m) throw smx::Error(SMX_EINVAL, "null model");
+        const auto& v = m->eng->hm.atomic_energies;
+        if (n) *n = (int)v.size();
+        for (int i = 0; out && i < cap && i < (int)v.size(); ++i) out[i] = v[i];
+    });
+}
+
+int smx_compute_node_energies_forces(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                                     const int* neigh_indices, const int* neigh_types, const double* xyz,
+                                     const double* r, long num_edges)
+{
+    return guarded([&] {
+        auto& e = E(m);
+        if (num_nodes > 0 && (!node_types || !num_neigh)) throw smx::Error(SMX_EINVAL, "null node array");
+        if (num_edges > 0 && (!neigh_indices || !neigh_types || !xyz || !r)) throw smx::Error(SMX_EINVAL, "null edge array");
+        e.stream = nullptr;
+        e.compute(num_nodes, node_types, num_neigh, neigh_indices, neigh_types, xyz, r, num_edges, false, nullptr, nullptr);
+        HIPCHK(hipStreamSynchronize(e.stream));
+    });
+}
+
+int smx_compute_device(smx_model* m, int num_nodes, const int* d_node_types, const int* d_num_neigh,
+                       const int* d_neigh_indices, const int* d_neigh_types, const double* d_xyz, const double* d_r,
+                       long num_edges, double* d_node_energies, double* d_node_forces, void* stream)
+{
+    return guarded([&] {
+        auto& e = E(m);
+        if (num_nodes > 0 && (!d_node_types || !d_num_neigh)) throw smx::Error(SMX_EINVAL, "null node array");
+        if (num_edges > 0 && (!d_neigh_indices || !d_neigh_types || !d_xyz || !d_r)) throw smx::Error(SMX_EINVAL, "null edge array");
+        e.stream = static_cast<hipStream_t>(stream);
+        e.compute(num_nodes, d_node_types, d_num_neigh, d_neigh_indices, d_neigh_types, d_xyz, d_r, num_edges, true,
+                  d_node_energies, d_node_forces);
+    });
+}
+
+int smx_set_num_H1_rows(smx_model* m, int rows)
+{
+    return guarded([&] { E(m).H1_rows_override = rows; });
+}
+
+#define SMX_STAGE(fn, name, NT, NN, NI, NTY, XYZ, R, EE, FA, FB) \
+    return guarded([&] { auto& e = E(m); e.stream = nullptr; e.stage(name, num_nodes, NT, NN, NI, NTY, XYZ, R, EE, FA, FB); HIPCHK(hipStreamSynchronize(e.stream)); })
+
+int smx_compute_Y(smx_model* m, const double* xyz, long n3)
+{
+    const int num_nodes = 0;
+    if (n3 % 3) { smx::g_last_error = "xyz length is not a multiple of 3"; return SMX_EINVAL; }
+    SMX_STAGE(smx_compute_Y, "Y", nullptr, nullptr, nullptr, nullptr, xyz, nullptr, n3 / 3, 0, 0);
+}
+int smx_compute_R0(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh, const int* neigh_types,
+                   const double* r, long num_edges)
+{
+    SMX_STAGE(smx_compute_R0, "R0", node_types, num_neigh, nullptr, neigh_types, nullptr, r, num_edges, 0, 0);
+}
+int smx_compute_R1(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh, const int* neigh_types,
+                   const double* r, long num_edges)
+{
+    SMX_STAGE(smx_compute_R1, "R1", node_types, num_neigh, nullptr, neigh_types, nullptr, r, num_edges, 0, 0);
+}
+int smx_compute_A0(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh, const int* neigh_types,
+                   long num_edges)
+{
+    SMX_STAGE(smx_compute_A0, "A0", node_types, num_neigh, nullptr, neigh_types, nullptr, nullptr, num_edges, 0, 0);
+}
+int smx_reverse_A0(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh, const int* neigh_types,
+                   const double* xyz, const double* r, long num_edges)
+{
+    SMX_STAGE(smx_reverse_A0, "reverse_A0", node_types, num_neigh, nullptr, neigh_types, xyz, r, num_edges, 0, 0);
+}
+int smx_compute_M0(smx_model* m, int num_nodes, const int* node_types)
+{
+    SMX_STAGE(smx_compute_M0, "M0", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_reverse_M0(smx_model* m, int num_nodes, const int* node_types)
+{
+    SMX_STAGE(smx_reverse_M0, "reverse_M0", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_compute_H1(smx_model* m, int num_nodes)
+{
+    SMX_STAGE(smx_compute_H1, "H1", nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_reverse_H1(smx_model* m, int num_nodes)
+{
+    SMX_STAGE(smx_reverse_H1, "reverse_H1", nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_compute_Phi1(smx_model* m, int num_nodes, const int* num_neigh, const int* neigh_indices, long num_edges)
+{
+    SMX_STAGE(smx_compute_Phi1, "Phi1", nullptr, num_neigh, neigh_indices, nullptr, nullptr, nullptr, num_edges, 0, 0);
+}
+int smx_reverse_Phi1(smx_model* m, int num_nodes, const int* num_neigh, const int* neigh_indices, const double* xyz,
+                     const double* r, long num_edges, int zero_dxyz, int zero_H1_adj)
+{
+    SMX_STAGE(smx_reverse_Phi1, "reverse_Phi1", nullptr, num_neigh, neigh_indices, nullptr, xyz, r, num_edges, zero_dxyz, zero_H1_adj);
+}
+int smx_compute_A1(smx_model* m, int num_nodes)
+{
+    SMX_STAGE(smx_compute_A1, "A1", nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_reverse_A1(smx_model* m, int num_nodes)
+{
+    SMX_STAGE(smx_reverse_A1, "reverse_A1", nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_compute_M1(smx_model* m, int num_nodes, const int* node_types)
+{
+    SMX_STAGE(smx_compute_M1, "M1", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_reverse_M1(smx_model* m, int num_nodes, const int* node_types)
+{
+    SMX_STAGE(smx_reverse_M1, "reverse_M1", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_compute_H2(smx_model* m, int num_nodes, const int* node_types)
+{
+    SMX_STAGE(smx_compute_H2, "H2", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+int smx_reverse_H2(smx_model* m, int num_nodes, const int* node_types, int zero_H1_adj)
+{
+    SMX_STAGE(smx_reverse_H2, "reverse_H2", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, zero_H1_adj, 0);
+}
+int smx_compute_readouts(smx_model* m, int num_nodes, const int* node_types)
+{
+    SMX_STAGE(smx_compute_readouts, "readouts", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
+}
+
+int smx_get_array(smx_model* m, const char* name, double* out, long cap, long* n)
+{
+    return guarded([&] {
+        if (!name) throw smx::Error(SMX_EINVAL, "null name");
+        E(m).get_array(name, out, cap, n);
+    });
+}
+int smx_set_array(smx_model* m, const char* name, const double* in, long n)
+{
+    return guarded([&] {
+        if (!name || (!in && n > 0)) throw smx::Error(SMX_EINVAL, "null argument");
+        E(m).set_array(name, in, n);
+    });
+}
+
+int smx_set_profiling(smx_model* m, int enabled)
+{
+    return guarded([&] {
+        auto& e = E(m);
+        e.profiling = enabled != 0;
+        for (int i = 0; i < smx::ST_COUNT; ++i) e.ev_used[i] = false;
+    });
+}
+const char* smx_stage_names(void) { return smx::kStageNames; }
+int smx_get_stage_times(smx_model* m, float* ms, int cap, int* n)
+{
+    return guarded([&] {
+        auto& e = E(m);
+        HIPCHK(hipStreamSynchronize(e.stream));
+        if (n) *n = smx::ST_COUNT;
+        for (int i = 0; ms && i < cap && i < smx::ST_COUNT; ++i) {
+            ms[i] = 0.f;
+            if (e.ev_used[i]) HIPCHK(hipEventElapsedTime(&ms[i], e.ev0[i], e.ev1[i]));
+        }
+    });
+}
+int smx_synchronize(smx_model* m)
+{
+    return guarded([&] { HIPCHK(hipStreamSynchronize(E(m).stream)); });
+}
+int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const int* receiver_atom,
+                      double* atom_forces, double* virial)
+{
+    return guarded([&] { E(m).reduce_forces(num_atoms, sender_atom, receiver_atom, atom_forces, virial); });
+}
+
+}  // extern "C"

@@ -1,0 +1,145 @@
+// Launch interface of the gfx950 kernels (definitions in smx_kernels_*.hip).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+namespace smx {
+
+// ---------------------------------------------------------------------------
+// Edge aggregation (forward) and its adjoint.  One templated pair of kernels
+// serves layer 0 (MACE::compute_A0 / reverse_A0 without the channel-mixing
+// linear, libsymmetrix/source/mace.cpp:158-178, 238-269) and layer 1
+// (compute_Phi1 / reverse_Phi1, mace.cpp:453-605): per edge
+//     out[i, lme, k] += R_path(lme)[k](r_ij) * sum_m2 B_ij[lme, m2] * H[g_ij, l2^2+m2, k]
+// with B_ij[.,.] = sum_m1 C * Y_m1(r_ij) the Clebsch-Gordan-contracted
+// harmonics of the edge, H the gathered sender row (H0_weights[type_j] for
+// layer 0, H1[neigh_index] for layer 1) and R the radial spline set of the
+// species pair.  Y, B and R are recomputed per edge inside the kernels and
+// never stored.
+template <typename F>
+struct AggParams {
+    int num_nodes;
+    int K;
+    const int* first_neigh;   // [num_nodes+1] CSR offsets of the receiver-sorted edge list
+    const int* node_types;    // [num_nodes]
+    const int* neigh_types;   // [E]
+    const int* gather;        // [E] row of Hsrc per edge
+    const double* xyz;        // [E][3]
+    const double* r;          // [E]
+    const F* Hsrc;            // [rows][NLM][K]
+    const F* tab;             // [table][nodes-1][4][P*K]
+    const int* pair_table;    // [T(T+1)/2] -> table
+    int T;
+    int spl_nodes;
+    double spl_h;
+    const int* B_start;       // [NB+1] rows of the coupling list
+    const int* B_lm1;
+    const double* B_c;
+    F* out;                   // fwd: [num_nodes][NE][K]
+    const F* d_out;           // bwd: adjoint of out
+    double* forces;           // bwd: [E][3]
+    int accumulate_forces;    // bwd: add to forces instead of overwriting
+    F* msg;                   // bwd: [E][NLM][K] adjoint message to the sender row, or null
+};
+
+template <typename F> hipError_t launch_agg_fwd(int L_max_H, const AggParams<F>& p, hipStream_t s);
+template <typename F> hipError_t launch_agg_bwd(int L_max_H, const AggParams<F>& p, hipStream_t s);
+
+// H1_adj[j] (+)= sum over edges with sender j of msg[e], in ascending edge order.
+template <typename F>
+hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg,
+                                F* H_adj, int zero_first, hipStream_t s);
+
+// ---------------------------------------------------------------------------
+// Integer list preparation
+hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums, hipStream_t s);  // out[n] = total
+hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
+                               int* slist, int* block_sums, hipStream_t s);
+hipError_t launch_type_groups(const int* node_types, int N, int T, int* tcount, int* tstart, int* cursor,
+                              int* perm, int* block_sums, hipStream_t s);
+// flags[0] |= 1 if any index is outside [0, limit)
+hipError_t launch_check_range(const int* v, long n, int limit, int* flags, hipStream_t s);
+hipError_t launch_check_r(const double* r, long n, double r_cut, int* flags, hipStream_t s);
+
+// ---------------------------------------------------------------------------
+// Symmetric contraction (MACE::compute_M0 / compute_M1, mace.cpp:348-370, 759-777):
+// value and gradient of NP polynomials of the 16 A_lm of one channel.
+template <typename F>
+struct PolyParams {
+    int num_nodes, K, NP;              // NP polynomials (num_LM for M0, 1 for M1)
+    const int* node_types;
+    const F* A;                        // [N][16][K]
+    F* M;                              // [N][NP][K]
+    F* M_grad;                         // [N][NP][16][K]
+    // per polynomial (device arrays of length NP)
+    const int* const* row_i0; const int* const* row_i1; const int* const* row_start;
+    const int* const* entry_var; const F* const* coef;   // coef[p]: [T][entries][K]
+    const int* num_rows; const int* num_entries;
+};
+template <typename F> hipError_t launch_poly(const PolyParams<F>& p, hipStream_t s);
+
+// A_adj[i,lm,k] = sum_LM M_grad[i,LM,lm,k] * M_adj[i,LM,k]   (reverse_M0 / reverse_M1)
+template <typename F>
+hipError_t launch_poly_reverse(int N, int NP, int K, const F* M_grad, const F* M_adj, F* A_adj, hipStream_t s);
+
+// ---------------------------------------------------------------------------
+// Dense channel mixing on the matrix cores.
+//   C[row(node,s)][n] (+)= sum_k A[row(node,s)][k] * W[type(node)][k][n]   (or W^T)
+// rows are (node, s) with s < sub; row (node,s) of A starts at
+// A + node*a_node_stride + a_off + s*a_sub_stride and is Kd long.
+struct GemmProb {
+    long a_off, a_sub_stride;   // row (node,s) of A starts at A + node*a_node_stride + a_off + s*a_sub_stride
+    long c_off, c_sub_stride;
+    long w_off;                 // offset of this problem's weight block inside W[type]
+    int Kd, Nn, sub;            // inner size, output columns, rows per node
+};
+template <typename TA, typename TC, typename CT>
+struct GemmParams {
+    const TA* A; long a_node_stride;
+    TC* C; long c_node_stride;
+    const CT* W; long w_type_stride;
+    int transW;              // 0: W block is [Kd][Nn]; 1: W block is [Nn][Kd]
+    int accumulate;          // 1: C += ...
+    int num_nodes;
+    const int* node_types;   // null -> single weight matrix
+    const int* perm;         // [num_nodes] nodes grouped by type (with node_types)
+    const int* tstart;       // [T+1]
+    int T;
+    int nprob;               // sub-problems selected by blockIdx.z (one per l)
+    GemmProb prob[4];
+};
+template <typename TA, typename TC, typename CT>
+hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p, hipStream_t s);
+
+// ---------------------------------------------------------------------------
+// Readout tail (MACE::compute_readouts, mace.cpp:876-903) after the two MFMA
+// products: hidden[N][16] = H2 . W1^T has been formed; this applies the scaled
+// SiLU, adds E0 + w1.H1[l=0] + w2.act to the node energy and leaves
+// g[N][16] = w2 * act' for the product g . W1 that yields H2_adj.
+template <typename F>
+hipError_t launch_readout(int N, int K, int num_LM, const int* node_types, const double* atomic_energies,
+                          const double* w1, const F* H1, double* hidden_g, const double* w2, double scale,
+                          double* node_energies, int zero_energies, hipStream_t s);
+// H1_adj: zero everywhere (rows x num_LM x K), l=0 block of the first N rows = readout_1 weights
+template <typename F>
+hipError_t launch_seed_H1_adj(int rows, int N, int num_LM, int K, const double* w1, F* H1_adj, hipStream_t s);
+
+template <typename T> hipError_t launch_fill(T* p, long n, T v, hipStream_t s);
+template <typename TS, typename TD> hipError_t launch_convert(const TS* src, TD* dst, long n, hipStream_t s);
+
+// Y[E][16], Y_grad[E][3][16] as the reference stores them (mace.cpp:118-148); inspection only
+hipError_t launch_sph_harm(const double* xyz, long E, double* Y, double* Y_grad, hipStream_t s);
+// R[E][nspl] spline values (mace.cpp:66-116); inspection only
+template <typename F>
+hipError_t launch_radial(int N, const int* first_neigh, const int* node_types, const int* neigh_types,
+                         const double* r, const F* tab, const int* pair_table, int T, int nodes, double h,
+                         int nspl, double* R, hipStream_t s);
+
+// atom_forces[j] += f_e, atom_forces[i] -= f_e in a fixed order per atom, virial sums
+hipError_t launch_force_scatter(int num_atoms, const int* recv_start, const int* recv_list,
+                                const int* send_start, const int* send_list, const double* forces,
+                                double* atom_forces, hipStream_t s);
+hipError_t launch_virial(long E, const double* xyz, const double* forces, double* partial, int nblocks,
+                         hipStream_t s);
+
+}  // namespace smx

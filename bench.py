@@ -1,0 +1,214 @@
+#!/usr/bin/env python3
+"""Benchmark of the MACE energy+forces hot path on one MI355X.
+
+One "step" = one evaluation of node energies and per-edge forces
+(MACE::compute_node_energies_forces, libsymmetrix/source/mace.cpp:17-64) for a
+fixed synthetic atomic configuration whose edge arrays are already resident in
+HBM.  Metric: atom-steps/s = atoms / seconds per step.
+
+Prints ONE JSON line.  Besides the driver's fields it carries
+  roofline      the dominant kernel of the step against the HBM roofline
+                (algorithmic bytes per launch / HIP-event duration of that stage)
+  cpu_baseline  the CPU oracle (serial fp64 restatement of the reference path)
+                timed on this host on the same workload
+  stages_ms     HIP-event time of every stage of the pipeline
+  fp32_features the same workload in the fp32-feature mode
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import tempfile
+import time
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, HERE)
+
+HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
+
+
+def algorithmic_bytes(stage, N, E, K, s, n_LM, n_e):
+    """Per-evaluation algorithmic HBM bytes of the edge kernels.
+
+    Spline, weight and coupling tables are cache resident and not counted;
+    every per-edge gather is.  36 = xyz 24 + r 8 + neighbour type 4; 40 adds the
+    neighbour index; 24 is the force write, 48 a force read-modify-write.
+    """
+    table = {
+        "agg0_fwd": 36 * E + (8 + 16 * K * s) * N,
+        "agg1_fwd": (40 + n_LM * K * s) * E + (8 + n_e * K * s) * N,
+        "agg1_bwd": (64 + 2 * n_LM * K * s) * E + n_e * K * s * N,
+        "sender_reduce": (4 + n_LM * K * s) * E + 2 * n_LM * K * s * N,
+        "agg0_bwd": 84 * E + 16 * K * s * N,
+    }
+    return table.get(stage)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="off_small", choices=["tiny", "off_small", "off_medium", "mp_medium"])
+    ap.add_argument("--scale", type=float, default=1.0, help="shrink the atom count (tests)")
+    ap.add_argument("--dtype", default="float64", choices=["float64", "float32"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-atoms", type=int, default=0, help="atoms in the CPU sample (0 = whole workload)")
+    ap.add_argument("--model-dir", default=tempfile.gettempdir())
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on exactly one GPU (no collectives exist in it); use --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+    from symmetrix_amd import modelgen, neighbors, systems
+    from symmetrix_amd.mace import MACE
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    dev = torch.device("cuda:0")
+
+    # ---- model file (seeded, random-init) and synthetic system
+    cfg = dict(modelgen.CONFIGS[args.workload])
+    # plain MACE has a species-independent radial network: every pair table of the file is equal
+    cfg["pair_dependent_radial"] = False
+    model_path = os.path.join(args.model_dir, f"smx_bench_{args.workload}.json")
+    if not os.path.exists(model_path):
+        modelgen.write_model(model_path, **cfg)
+    pos, cell, species = systems.config_system(args.workload, seed=0, scale=args.scale)
+    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"])
+    ea = neighbors.edge_arrays(nl, species)
+    N, E = int(ea["num_nodes"]), int(len(ea["r"]))
+
+    def to_dev(a, dt):
+        return torch.from_numpy(np.ascontiguousarray(a)).to(dev, dtype=dt)
+
+    d = dict(
+        node_types=to_dev(ea["node_types"], torch.int32), num_neigh=to_dev(ea["num_neigh"], torch.int32),
+        neigh_indices=to_dev(ea["neigh_indices"], torch.int32), neigh_types=to_dev(ea["neigh_types"], torch.int32),
+        xyz=to_dev(ea["xyz"], torch.float64), r=to_dev(ea["r"], torch.float64),
+    )
+    out_E = torch.zeros(N, dtype=torch.float64, device=dev)
+    out_F = torch.zeros(3 * E, dtype=torch.float64, device=dev)
+
+    def run_mode(dtype, steps, warmup):
+        eng = MACE(model_path, dtype)
+        stream = torch.cuda.current_stream().cuda_stream
+
+        def step():
+            eng.compute_device(N, d["node_types"].data_ptr(), d["num_neigh"].data_ptr(), d["neigh_indices"].data_ptr(),
+                               d["neigh_types"].data_ptr(), d["xyz"].data_ptr(), d["r"].data_ptr(), E,
+                               out_E.data_ptr(), out_F.data_ptr(), stream)
+
+        for _ in range(warmup):
+            step()
+        torch.cuda.synchronize()
+        # timed region: exactly `steps` evaluations; per-stage HIP events ride along on the same stream
+        eng.set_profiling(True)
+        acc = {}
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+            # stage events are per model and reused every step: read them back before the next step
+            for k, v in eng.stage_times().items():
+                acc[k] = acc.get(k, 0.0) + v
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        eng.set_profiling(False)
+        # the same number of steps without event read-back (pure asynchronous enqueue)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            step()
+        torch.cuda.synchronize()
+        dt_async = time.perf_counter() - t0
+        stages = {k: v / steps for k, v in acc.items()}
+        energy = float(out_E.sum().item())
+        fmax = float(out_F.abs().max().item()) if E else 0.0
+        del eng
+        return dict(ms_sync=1e3 * dt / steps, ms=1e3 * dt_async / steps, stages=stages, energy=energy, fmax=fmax,
+                    forces=out_F.cpu().numpy().copy())
+
+    res = run_mode(args.dtype, args.steps, args.warmup)
+    other = "float32" if args.dtype == "float64" else "float64"
+    res_other = run_mode(other, max(5, args.steps // 2), args.warmup)
+
+    K = cfg["num_channels"]
+    L_max = cfg["L_max"]
+    n_LM = (L_max + 1) ** 2
+    n_e = 16 if L_max == 0 else 40
+    s_bytes = 8 if args.dtype == "float64" else 4
+    edge_stages = ["agg0_fwd", "agg1_fwd", "agg1_bwd", "sender_reduce", "agg0_bwd"]
+    dom = max(edge_stages, key=lambda k: res["stages"].get(k, 0.0))
+    dom_bytes = algorithmic_bytes(dom, N, E, K, s_bytes, n_LM, n_e)
+    dom_s = res["stages"][dom] * 1e-3
+    achieved = dom_bytes / dom_s / 1e9 if dom_s > 0 else 0.0
+    total_bytes = sum(algorithmic_bytes(k, N, E, K, s_bytes, n_LM, n_e) for k in edge_stages) + (32 * E + 24 * N)
+
+    value = N / (res["ms"] * 1e-3)
+    line = {
+        "metric": "atom-steps/s per MI355X (energy+forces)",
+        "value": value,
+        "unit": "atom-steps/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": res["ms"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f64" if args.dtype == "float64" else "f32-features/f64-accumulation",
+        "data": "synthetic",
+        "config": {
+            "workload": f"{args.workload}: {N} atoms, {E} edges, K={K}, L_max={L_max}, r_cut={cfg['r_cut']}, "
+                        f"random-init symmetrix JSON model (seed 0), species-independent radial tables",
+            "atoms": N, "edges": E, "channels": K, "L_max": L_max, "scale": args.scale,
+        },
+        "roofline": {
+            "bound": "hbm", "kernel": dom, "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+            "frac": achieved / (HBM_PEAK / 1e9), "traffic": None,
+            "algorithmic_bytes_per_launch": dom_bytes,
+            "whole_step_algorithmic_bytes": total_bytes,
+            "whole_step_frac": (total_bytes / HBM_PEAK) / (res["ms"] * 1e-3),
+        },
+        "stages_ms": res["stages"],
+        "ms_per_step_with_event_readback": res["ms_sync"],
+        "energy": res["energy"],
+        "other_precision": {"dtype": other, "ms_per_step": res_other["ms"], "value": N / (res_other["ms"] * 1e-3),
+                            "energy": res_other["energy"], "stages_ms": res_other["stages"]},
+    }
+
+    # ---- CPU baseline: the oracle (serial fp64 port of the reference path) on this host
+    if not args.no_cpu:
+        from oracle.oracle import OracleMACE
+        orc = OracleMACE(model_path)
+        if args.cpu_atoms and args.cpu_atoms < N:
+            p2, c2, s2 = systems.config_system(args.workload, seed=0, scale=args.scale * args.cpu_atoms / N)
+            nl2 = neighbors.neighbor_list(p2, c2, cfg["r_cut"])
+            ea2 = neighbors.edge_arrays(nl2, s2)
+            sample = f"{ea2['num_nodes']} atoms / {len(ea2['r'])} edges sub-box of the workload (same density, same model), 1 evaluation"
+        else:
+            ea2 = ea
+            sample = f"the whole workload ({N} atoms, {E} edges), 1 evaluation"
+        t0 = time.perf_counter()
+        orc.compute_node_energies_forces(ea2["num_nodes"], ea2["node_types"], ea2["num_neigh"], ea2["neigh_indices"],
+                                         ea2["neigh_types"], ea2["xyz"], ea2["r"])
+        dt = time.perf_counter() - t0
+        cpu_value = ea2["num_nodes"] / dt
+        line["cpu_baseline"] = {"value": cpu_value, "unit": "atom-steps/s", "cores": 1, "kind": "port",
+                                "sample": sample, "seconds": dt, "host_cores": os.cpu_count(),
+                                "gpu_over_cpu_1core": value / cpu_value}
+        if ea2 is ea:
+            Ecpu = float(orc.node_energies.sum())
+            line["cpu_baseline"]["energy_rel_diff_vs_gpu"] = abs(Ecpu - res["energy"]) / abs(Ecpu)
+            line["cpu_baseline"]["force_max_abs_diff_vs_gpu"] = float(np.abs(orc.node_forces - res["forces"]).max())
+    print(json.dumps(line))
+
+
+if __name__ == "__main__":
+    main()

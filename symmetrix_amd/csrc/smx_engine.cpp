@@ -73,11 +73,11 @@ struct DVec {
         cap = newcap;
     }
     // size to m elements; previous contents are undefined afterwards
-    void size_to(size_t m, hipStream_t s) { reserve(m, s, false); n = m; }
+    void size_to(size_t m, hipStream_t s) { reserve(m ? m : 1, s, false); n = m; }
     // std::vector::resize
     void resize(size_t m, hipStream_t s)
     {
-        reserve(m, s, true);
+        reserve(m ? m : 1, s, true);
         if (m > n) HIPCHK(hipMemsetAsync(p + n, 0, (m - n) * sizeof(T), s));
         n = m;
     }
@@ -307,6 +307,24 @@ struct Engine : EngineBase {
         if (f & 1) throw Error(SMX_EINVAL, "node_types / neigh_types / neigh_indices hold an index outside the model or the node range");
         if (f & 2) throw Error(SMX_ERANGE, "an edge length lies outside (0, r_cut): the radial spline tables do not cover it");
     }
+    // stage-level calls: check whichever integer arrays this call brought
+    void validate_stage_inputs(int N, bool have_nt, bool have_ni, bool have_nty, bool have_r)
+    {
+        hipStream_t s = stream;
+        HIPCHK(hipMemsetAsync(flags.p, 0, sizeof(int), s));
+        if (have_nt) HIPCHK(launch_check_range(node_types, N, hm.T, flags.p, s));
+        if (have_nty) HIPCHK(launch_check_range(neigh_types, E, hm.T, flags.p, s));
+        if (have_ni) {
+            const size_t rows_now = H1.n / ((size_t)hm.num_LM * hm.K);
+            HIPCHK(launch_check_range(neigh_indices, E, (int)std::max<size_t>(rows_now, (size_t)N), flags.p, s));
+        }
+        if (have_r) HIPCHK(launch_check_r(r, E, hm.r_cut, flags.p, s));
+        int f = 0;
+        HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, s));
+        HIPCHK(hipStreamSynchronize(s));
+        if (f & 1) throw Error(SMX_EINVAL, "node_types / neigh_types / neigh_indices hold an index outside the model or the node range");
+        if (f & 2) throw Error(SMX_ERANGE, "an edge length lies outside (0, r_cut): the radial spline tables do not cover it");
+    }
     int edges_from_counts_check(int N, const int* host_num_neigh, long E_)
     {
         long tot = 0;
@@ -524,12 +542,19 @@ struct Engine : EngineBase {
         if (hm.has_zbl || hm.A0_scaled || hm.A1_scaled)
             throw Error(SMX_EUNSUPPORTED, "models with ZBL or density normalisation are not implemented on the device yet");
         if (!on_device) edges_from_counts_check(N, nn, E_);
+        if (N == 0) {
+            if (E_ != 0) throw Error(SMX_EINVAL, "edges without nodes");
+            E = 0; N_geo = 0;
+            node_energies.size_to(0, stream); node_forces.size_to(0, stream);
+            return;
+        }
         stage_begin(ST_PREP);
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, on_device);
         build_first_neigh(N);
+        // range checks come before any kernel that uses these integers as indices
+        if (!on_device) validate(N, N);
         build_type_groups(N);
         sender_rows = -1;
-        if (!on_device) validate(N, N);
         build_sender_lists(N);
         stage_end(ST_PREP);
 
@@ -570,6 +595,7 @@ struct Engine : EngineBase {
         if (nn && E_ >= 0) edges_from_counts_check(N, nn, E_);
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, false);
         if (nn) build_first_neigh(N);
+        validate_stage_inputs(N, nt != nullptr, ni != nullptr, nty != nullptr, rr != nullptr);
         if (s == "Y" || s == "R0" || s == "R1") return;  // geometry remembered; evaluated inside the fused kernels
         if (s == "A0") { build_type_groups(N); st_agg0_fwd(N); st_A0_lin(N, false); }
         else if (s == "reverse_A0") { build_type_groups(N); st_A0_lin(N, true); st_agg0_bwd(N); }
@@ -692,6 +718,12 @@ struct Engine : EngineBase {
             scan_tmp.size_to((size_t)num_atoms / 1024 + 2, s);
             HIPCHK(hipMemsetAsync(flags.p, 0, sizeof(int), s));
             HIPCHK(launch_check_range(rf_send.p, E, num_atoms, flags.p, s));
+            {
+                int f = 0;
+                HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, s));
+                HIPCHK(hipStreamSynchronize(s));
+                if (f) throw Error(SMX_EINVAL, "sender_atom out of range");
+            }
             const int* rstart = nullptr;
             const int* rlist = nullptr;
             if (receiver_atom) {
@@ -720,10 +752,6 @@ struct Engine : EngineBase {
                 HIPCHK(hipStreamSynchronize(s));
                 rstart = rf_rstart.p;
             }
-            int f = 0;
-            HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, s));
-            HIPCHK(hipStreamSynchronize(s));
-            if (f) throw Error(SMX_EINVAL, "sender_atom out of range");
             HIPCHK(launch_sender_lists(rf_send.p, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, s));
             rf_out.size_to((size_t)3 * num_atoms, s);
             HIPCHK(launch_force_scatter(num_atoms, rstart, rlist, rf_sstart.p, rf_slist.p, node_forces.p, rf_out.p, s));

@@ -68,17 +68,21 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_add(int* out, int n, const 
     if (i < n) out[i] += block_sums[blockIdx.x];
 }
 
-__global__ void k_count(const int* key, long n, int* count)
-{
-    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) atomicAdd(&count[key[i]], 1);
-}
-__global__ void k_place(const int* key, long n, const int* start, int* cursor, int* list)
+// keys outside [0, rows) are ignored (callers that hand over device arrays are not range-checked)
+__global__ void k_count(const int* key, long n, int rows, int* count)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) {
         const int j = key[i];
-        list[start[j] + atomicAdd(&cursor[j], 1)] = (int)i;
+        if (j >= 0 && j < rows) atomicAdd(&count[j], 1);
+    }
+}
+__global__ void k_place(const int* key, long n, int rows, const int* start, int* cursor, int* list)
+{
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const int j = key[i];
+        if (j >= 0 && j < rows) list[start[j] + atomicAdd(&cursor[j], 1)] = (int)i;
     }
 }
 // ascending order inside every bucket: the placement above is unordered
@@ -132,13 +136,14 @@ hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums
 hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
                                int* slist, int* block_sums, hipStream_t s)
 {
+    if (rows <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, count, (long)rows, 0);
     hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, cursor, (long)rows, 0);
-    if (E > 0) hipLaunchKernelGGL(k_count, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, count);
+    if (E > 0) hipLaunchKernelGGL(k_count, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, count);
     hipError_t err = launch_scan_exclusive(count, sstart, rows, block_sums, s);
     if (err != hipSuccess) return err;
     if (E > 0) {
-        hipLaunchKernelGGL(k_place, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, sstart, cursor, slist);
+        hipLaunchKernelGGL(k_place, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, sstart, cursor, slist);
         hipLaunchKernelGGL(k_sort_buckets, dim3(nblk(rows, 64)), dim3(64), 0, s, sstart, rows, slist);
     }
     return hipGetLastError();
@@ -147,15 +152,16 @@ hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, i
 hipError_t launch_type_groups(const int* node_types, int N, int T, int* tcount, int* tstart, int* cursor,
                               int* perm, int* block_sums, hipStream_t s)
 {
+    if (T <= 0) return hipSuccess;
     hipLaunchKernelGGL(k_fill<int>, dim3(nblk(T, 256)), dim3(256), 0, s, tcount, (long)T, 0);
     hipLaunchKernelGGL(k_fill<int>, dim3(nblk(T, 256)), dim3(256), 0, s, cursor, (long)T, 0);
-    if (N > 0) hipLaunchKernelGGL(k_count, dim3(nblk(N, 256)), dim3(256), 0, s, node_types, (long)N, tcount);
+    if (N > 0) hipLaunchKernelGGL(k_count, dim3(nblk(N, 256)), dim3(256), 0, s, node_types, (long)N, T, tcount);
     hipError_t err = launch_scan_exclusive(tcount, tstart, T, block_sums, s);
     if (err != hipSuccess) return err;
     if (N > 0) {
         // order inside a type group is left as placed: every output row of the
         // products that use this grouping is computed independently of its tile mates
-        hipLaunchKernelGGL(k_place, dim3(nblk(N, 256)), dim3(256), 0, s, node_types, (long)N, tstart, cursor, perm);
+        hipLaunchKernelGGL(k_place, dim3(nblk(N, 256)), dim3(256), 0, s, node_types, (long)N, T, tstart, cursor, perm);
     }
     return hipGetLastError();
 }

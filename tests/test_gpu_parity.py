@@ -1,0 +1,238 @@
+"""GPU parity tests proper (run on an MI355X with -m gpu).
+
+Every check goes through the C ABI (symmetrix_amd.mace.MACE is a ctypes face of
+include/symmetrix_amd.h) and compares the HIP engine with the CPU oracle on the
+same seeded inputs.  Tolerances are the ones the task states:
+  fp64 mode           energy rel <= 1e-10, forces max-abs <= 1e-8 eV/A
+  fp32-feature mode   energy rel <= 1e-5,  forces max-abs <= 1e-4 eV/A
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+TOL = {"float64": dict(E=1e-10, F=1e-8, inter=1e-11), "float32": dict(E=1e-5, F=1e-4, inter=2e-5)}
+INTERMEDIATES = ["Y", "Y_grad", "R0", "R1", "A0", "M0", "H1", "Phi1", "A1", "M1", "H2", "H2_adj", "M1_adj",
+                 "A1_adj", "Phi1_adj", "H1_adj", "M0_adj", "A0_adj"]
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    from symmetrix_amd.mace import MACE
+    return MACE
+
+
+def _oracle():
+    from oracle.oracle import OracleMACE
+    return OracleMACE
+
+
+def _compare(orc, eng, dtype, names=INTERMEDIATES):
+    tol = TOL[dtype]
+    for name in names:
+        a = getattr(orc, name); b = getattr(eng, name)
+        assert a.shape == b.shape, name
+        scale = max(1.0, np.abs(a).max()) if len(a) else 1.0
+        assert np.abs(a - b).max(initial=0.0) <= tol["inter"] * scale * 10, name
+    Eo, Eg = orc.node_energies.sum(), eng.node_energies.sum()
+    assert abs(Eo - Eg) <= tol["E"] * abs(Eo)
+    assert np.abs(orc.node_energies - eng.node_energies).max() <= tol["E"] * max(1.0, np.abs(orc.node_energies).max()) * 10
+    assert np.abs(orc.node_forces - eng.node_forces).max(initial=0.0) <= tol["F"]
+
+
+CASES = [
+    # K, L_max, atoms, pair-dependent radial
+    (32, 0, 40, True), (32, 1, 40, True), (96, 0, 48, False), (128, 1, 36, True), (48, 1, 24, True),
+    (20, 0, 17, True), (64, 1, 30, False), (128, 0, 30, True),
+]
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("K,L_max,natoms,pair", CASES)
+def test_pipeline_matches_oracle(gpu, tmp_models, K, L_max, natoms, pair, dtype):
+    model = H.tiny_model(K=K, L_max=L_max, n_pts=64, seed=K + L_max, pair=pair)
+    path = H.write_model(model, tmp_models / f"m_{K}_{L_max}_{int(pair)}.json")
+    orc = _oracle()(model)
+    eng = gpu(path, dtype)
+    pos, cell, sp = H.small_system(natoms, seed=natoms)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K={K} L_max={L_max} atoms={natoms} edges={len(ea['r'])} {dtype}", flush=True)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    _compare(orc, eng, dtype)
+    # bit-reproducible: no atomics on floats anywhere
+    f1, e1 = eng.node_forces, eng.node_energies
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    assert np.array_equal(f1, eng.node_forces) and np.array_equal(e1, eng.node_energies)
+    # caller-side reduction, symmetrix_calc.py:93-102 / pair_symmetrix_mace.cpp:334-368
+    F, V = eng.reduce_forces(len(pos), nl["j"], virial=True)
+    assert np.allclose(F, H.atom_forces(nl, orc.node_forces, len(pos)), atol=TOL[dtype]["F"] * 10)
+    f = orc.node_forces.reshape(-1, 3); x = ea["xyz"].reshape(-1, 3)
+    W = x.T @ f
+    Vref = np.array([W[0, 0], W[1, 1], W[2, 2], 0.5 * (W[0, 1] + W[1, 0]), 0.5 * (W[0, 2] + W[2, 0]), 0.5 * (W[1, 2] + W[2, 1])])
+    assert np.allclose(V, Vref, atol=TOL[dtype]["F"] * 100)
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+def test_golden_fixture(gpu, dtype):
+    z = np.load(os.path.join(GOLD, "tiny_case.npz"))
+    eng = gpu(os.path.join(GOLD, "tiny_model.json"), dtype)
+    eng.compute_node_energies_forces(len(z["node_types"]), z["node_types"], z["num_neigh"], z["neigh_indices"],
+                                     z["neigh_types"], z["xyz"], z["r"])
+    tol = TOL[dtype]
+    E = z["node_energies"].sum()
+    assert abs(eng.node_energies.sum() - E) <= tol["E"] * abs(E)
+    assert np.abs(eng.node_forces - z["node_forces"]).max() <= tol["F"]
+    for name in ("A0", "M0", "H1", "Phi1", "A1", "M1", "H2", "H1_adj", "A0_adj"):
+        assert np.abs(getattr(eng, name) - z[name]).max() <= tol["inter"] * 10 * max(1.0, np.abs(z[name]).max()), name
+
+
+def test_stage_level_calls_follow_the_reference_test_method(gpu, tmp_models):
+    """symmetrix/test/test_mace.py drives the evaluator stage by stage and overwrites
+    intermediates between calls (e.g. :246-249).  Same here, against the oracle."""
+    model = H.tiny_model(K=8, L_max=1, n_pts=40, seed=9)
+    path = H.write_model(model, tmp_models / "stage.json")
+    orc = _oracle()(model)
+    eng = gpu(path)
+    pos, cell, sp = H.small_system(10, seed=3)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    N, nt, nn, ni, nty, xyz, r = H.call_args(ea)
+    rng = np.random.default_rng(0)
+    for m in (orc, eng):
+        m.compute_Y(xyz)
+        m.compute_R0(N, nt, nn, nty, r)
+        m.compute_A0(N, nt, nn, nty)
+    assert np.allclose(orc.A0, eng.A0, atol=1e-12)
+    assert np.allclose(orc.R0, eng.R0, atol=1e-12) and np.allclose(orc.Y, eng.Y, atol=1e-13)
+    A0 = rng.normal(size=len(orc.A0))
+    for m in (orc, eng):
+        m.A0 = A0
+        m.compute_M0(N, nt)
+        m.M0_adj = np.ones(len(m.M0))
+        m.reverse_M0(N, nt)
+    assert np.allclose(orc.M0, eng.M0, atol=1e-11) and np.allclose(orc.A0_adj, eng.A0_adj, atol=1e-10)
+    for m in (orc, eng):
+        m.compute_H1(N)
+        m.H1_adj = np.ones(len(m.H1))
+        m.reverse_H1(N)
+    assert np.allclose(orc.H1, eng.H1, atol=1e-11) and np.allclose(orc.M0_adj, eng.M0_adj, atol=1e-11)
+    for m in (orc, eng):
+        m.compute_R1(N, nt, nn, nty, r)
+        m.compute_Phi1(N, nn, ni)
+        m.Phi1_adj = np.ones(len(m.Phi1))
+        m.reverse_Phi1(N, nn, ni, xyz, r, True, True)
+    assert np.allclose(orc.Phi1, eng.Phi1, atol=1e-11)
+    assert np.allclose(orc.node_forces, eng.node_forces, atol=1e-10)
+    assert np.allclose(orc.H1_adj, eng.H1_adj, atol=1e-10)
+    for m in (orc, eng):
+        m.compute_A1(N)
+        m.A1_adj = np.ones(len(m.A1))
+        m.reverse_A1(N)
+    assert np.allclose(orc.A1, eng.A1, atol=1e-12) and np.allclose(orc.Phi1_adj, eng.Phi1_adj, atol=1e-12)
+    for m in (orc, eng):
+        m.compute_M1(N, nt)
+        m.M1_adj = np.ones(len(m.M1))
+        m.reverse_M1(N, nt)
+    assert np.allclose(orc.M1, eng.M1, atol=1e-12) and np.allclose(orc.A1_adj, eng.A1_adj, atol=1e-11)
+    for m in (orc, eng):
+        m.compute_H2(N, nt)
+        m.H2_adj = np.ones(len(m.H2))
+        m.reverse_H2(N, nt, True)
+    assert np.allclose(orc.H2, eng.H2, atol=1e-12)
+    assert np.allclose(orc.M1_adj, eng.M1_adj, atol=1e-12) and np.allclose(orc.H1_adj, eng.H1_adj, atol=1e-12)
+    for m in (orc, eng):
+        m.node_energies = np.zeros(N)
+        m.compute_readouts(N, nt)
+    assert np.allclose(orc.node_energies, eng.node_energies, atol=1e-12)
+    assert np.allclose(orc.H2_adj, eng.H2_adj, atol=1e-12) and np.allclose(orc.H1_adj, eng.H1_adj, atol=1e-13)
+    # reverse_A0 accumulates into node_forces (mace.cpp:237)
+    for m in (orc, eng):
+        m.A0_adj = np.ones(len(m.A0))
+        m.node_forces = np.zeros(len(xyz))
+        m.reverse_A0(N, nt, nn, nty, xyz, r)
+    assert np.allclose(orc.node_forces, eng.node_forces, atol=1e-10)
+
+
+def test_edge_cases(gpu, tmp_models):
+    model = H.tiny_model(K=8, L_max=0, n_pts=32, seed=2)
+    path = H.write_model(model, tmp_models / "edge.json")
+    orc = _oracle()(model)
+    eng = gpu(path)
+    # no nodes at all
+    eng.compute_node_energies_forces(0, [], [], [], [], [], [])
+    assert len(eng.node_energies) == 0 and len(eng.node_forces) == 0
+    # isolated atoms only: E_i = E0[type]
+    eng.compute_node_energies_forces(3, [0, 2, 1], [0, 0, 0], [], [], [], [])
+    assert np.allclose(eng.node_energies, np.array(model["atomic_energies"])[[0, 2, 1]], atol=1e-14)
+    # ragged degrees, including zero-degree receivers in the middle
+    rng = np.random.default_rng(4)
+    nn = np.array([3, 0, 5, 1, 0, 2], dtype=np.int32)
+    E = int(nn.sum())
+    nt = rng.integers(0, 3, size=6).astype(np.int32)
+    ni = rng.integers(0, 6, size=E).astype(np.int32)
+    nty = nt[ni]
+    xyz = rng.normal(size=(E, 3)); xyz *= (rng.uniform(0.8, 3.9, size=(E, 1)) / np.linalg.norm(xyz, axis=1, keepdims=True))
+    r = np.linalg.norm(xyz, axis=1)
+    args = (6, nt, nn, ni, nty, xyz.reshape(-1), r)
+    orc.compute_node_energies_forces(*args); eng.compute_node_energies_forces(*args)
+    _compare(orc, eng, "float64")
+    # a receiver with more edges than one LDS chunk, several times over
+    nn = np.array([70, 1], dtype=np.int32); E = 71
+    ni = rng.integers(0, 2, size=E).astype(np.int32); nt = np.array([0, 1], dtype=np.int32); nty = nt[ni]
+    xyz = rng.normal(size=(E, 3)); xyz *= (rng.uniform(0.8, 3.9, size=(E, 1)) / np.linalg.norm(xyz, axis=1, keepdims=True))
+    args = (2, nt, nn, ni, nty, xyz.reshape(-1), np.linalg.norm(xyz, axis=1))
+    orc.compute_node_energies_forces(*args); eng.compute_node_energies_forces(*args)
+    _compare(orc, eng, "float64")
+
+
+def test_invalid_inputs_raise(gpu, tmp_models):
+    model = H.tiny_model(K=8, L_max=0, n_pts=32, seed=2)
+    eng = gpu(H.write_model(model, tmp_models / "inv.json"))
+    xyz = np.array([[1.0, 0, 0], [-1.0, 0, 0]]).reshape(-1)
+    ok = (2, [0, 1], [1, 1], [1, 0], [1, 0], xyz, [1.0, 1.0])
+    eng.compute_node_energies_forces(*ok)
+    with pytest.raises(ValueError):      # beyond the spline table (cubic_spline_set.cpp:54 would read past it)
+        eng.compute_node_energies_forces(2, [0, 1], [1, 1], [1, 0], [1, 0], xyz * 5, [5.0, 5.0])
+    with pytest.raises(ValueError):      # species index outside the model
+        eng.compute_node_energies_forces(2, [0, 7], [1, 1], [1, 0], [1, 0], xyz, [1.0, 1.0])
+    with pytest.raises(ValueError):      # sender outside the node range
+        eng.compute_node_energies_forces(2, [0, 1], [1, 1], [5, 0], [1, 0], xyz, [1.0, 1.0])
+    with pytest.raises(ValueError):      # counts do not add up
+        eng.compute_node_energies_forces(2, [0, 1], [2, 1], [1, 0], [1, 0], xyz, [1.0, 1.0])
+    eng.compute_node_energies_forces(*ok)   # still usable afterwards
+
+
+@pytest.mark.parametrize("workload", ["off_small"])
+def test_full_size_properties(gpu, tmp_models, workload):
+    """At the benchmark's full size: properties that do not need the oracle."""
+    from symmetrix_amd import modelgen, neighbors, systems
+    cfg = dict(modelgen.CONFIGS[workload]); cfg["pair_dependent_radial"] = False
+    path = str(tmp_models / f"{workload}.json")
+    modelgen.write_model(path, **cfg)
+    pos, cell, sp = systems.config_system(workload)
+    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"]); ea = neighbors.edge_arrays(nl, sp)
+    e64 = gpu(path, "float64")
+    e64.compute_node_energies_forces(*H.call_args(ea))
+    E64, f64 = e64.node_energies.sum(), e64.node_forces
+    F = e64.reduce_forces(len(pos), nl["j"])
+    assert np.abs(F.sum(0)).max() < 1e-9                       # Newton's third law
+    assert np.allclose(F, H.atom_forces(nl, f64, len(pos)), atol=1e-10)
+    # relabelling the atoms permutes the answers
+    perm = np.random.default_rng(0).permutation(len(pos))
+    nl2 = neighbors.neighbor_list(pos[perm], cell, cfg["r_cut"]); ea2 = neighbors.edge_arrays(nl2, sp[perm])
+    e64.compute_node_energies_forces(*H.call_args(ea2))
+    assert abs(e64.node_energies.sum() - E64) <= 1e-10 * abs(E64)
+    assert np.allclose(e64.reduce_forces(len(pos), nl2["j"]), F[perm], atol=1e-9)
+    # fp32-feature mode against fp64 mode
+    e32 = gpu(path, "float32")
+    e32.compute_node_energies_forces(*H.call_args(ea))
+    assert abs(e32.node_energies.sum() - E64) <= 1e-5 * abs(E64)
+    assert np.abs(e32.node_forces - f64).max() <= 1e-4

@@ -1,0 +1,129 @@
+"""Host-side logic that needs no GPU: neighbour lists, the model generator's
+structure, and that the C-ABI library loads and exports every declared symbol."""
+import ctypes as C
+import json
+import os
+import re
+
+import numpy as np
+import pytest
+
+from symmetrix_amd import _lib, cg, modelgen, neighbors, systems
+from tests import helpers as H
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+@pytest.mark.parametrize("L,N,rc", [(6.0, 30, 5.0), (12.0, 100, 4.5), (4.0, 5, 5.0), (3.0, 1, 4.0)])
+def test_neighbor_list_matches_brute_force(L, N, rc):
+    rng = np.random.default_rng(int(L * 10 + N))
+    pos = rng.uniform(0, L, size=(N, 3))
+    cell = [L, L * 1.1, L * 0.9]
+    a = neighbors.neighbor_list(pos, cell, rc)
+    b = neighbors.brute_force_neighbor_list(pos, cell, rc)
+    for k in ("i", "j", "S", "xyz", "r"):
+        assert np.array_equal(a[k], b[k]), k          # integers and floats bit-exact
+    # canonical order: (i, j, Sx, Sy, Sz) ascending, no duplicates
+    key = np.stack([a["i"], a["j"], a["S"][:, 0], a["S"][:, 1], a["S"][:, 2]], axis=1)
+    assert all(tuple(key[q]) < tuple(key[q + 1]) for q in range(len(key) - 1))
+    assert np.all(a["r"] < rc)
+
+
+def test_neighbor_list_symmetric_full_list():
+    pos, cell, sp = systems.random_box(60, 0.1, [0.5, 0.5], seed=2)
+    nl = neighbors.neighbor_list(pos, cell, 4.0)
+    fwd = set(zip(nl["i"].tolist(), nl["j"].tolist(), map(tuple, nl["S"].tolist())))
+    for i, j, S in fwd:
+        assert (j, i, (-S[0], -S[1], -S[2])) in fwd
+    ea = neighbors.edge_arrays(nl, sp)
+    # the ASE caller counts neighbours over j (symmetrix_calc.py:80): same thing for a full list
+    assert np.array_equal(ea["num_neigh"], np.bincount(nl["j"], minlength=len(pos)))
+
+
+def test_empty_and_open_boundaries():
+    pos = np.array([[0.0, 0.0, 0.0], [10.0, 0.0, 0.0]])
+    nl = neighbors.neighbor_list(pos, [30.0, 30.0, 30.0], 3.0)
+    assert len(nl["i"]) == 0 and nl["first_neigh"].tolist() == [0, 0, 0]
+    nl = neighbors.neighbor_list(np.array([[0.5, 0.5, 0.5], [2.5, 0.5, 0.5]]), [3.0, 30.0, 30.0], 2.5, pbc=(False, True, True))
+    assert len(nl["i"]) == 2                          # no image across the open direction
+
+
+def test_real_cg_couples_harmonics():
+    rng = np.random.default_rng(0)
+    u = rng.normal(size=(6, 3))
+    Y = cg.real_sph_harm(u)
+    for (l, l1, l2) in cg.tensor_product_paths(3, 1):
+        Cg = cg.real_cg(l1, l2, l)
+        out = np.einsum("na,nb,abc->nc", Y[:, l1 * l1:(l1 + 1) ** 2], Y[:, l2 * l2:(l2 + 1) ** 2], Cg)
+        ratio = out / Y[:, l * l:(l + 1) ** 2]
+        assert np.allclose(ratio, ratio.flat[0], rtol=1e-9)
+        assert np.allclose((Cg ** 2).sum(axis=(0, 1)), 1.0)
+
+
+def test_generator_emits_every_key_the_loader_reads():
+    m = json.loads(json.dumps(H.tiny_model(K=3, L_max=1, n_pts=12)))
+    keys = ["num_elements", "num_channels", "r_cut", "l_max", "L_max", "atomic_numbers", "atomic_energies", "has_zbl",
+            "radial_spline_h", "radial_spline_values_0", "radial_spline_derivs_0", "radial_spline_values_1",
+            "radial_spline_derivs_1", "H0_weights", "A0_weights", "A0_scaled", "M0_weights", "M0_monomials",
+            "H1_weights", "Phi1_l", "Phi1_l1", "Phi1_l2", "Phi1_lme", "Phi1_clebsch_gordan", "Phi1_lelm1lm2",
+            "A1_weights", "A1_scaled", "M1_weights", "M1_monomials", "H2_weights_for_H1", "H2_weights_for_M1",
+            "readout_1_weights", "readout_2_weights_1", "readout_2_weights_2", "readout_2_scale_factor"]
+    for k in keys:                                     # mace.cpp:912-1029
+        assert k in m, k
+    T, K = 3, 3
+    assert np.array(m["radial_spline_values_0"]).shape == (T * (T + 1) // 2, 4 * K, 12)
+    P = len(m["Phi1_l"])
+    assert P == 10 and m["Phi1_l"] == sorted(m["Phi1_l"])          # non-decreasing, mace.cpp:619-640
+    assert np.array(m["radial_spline_values_1"]).shape == (6, P * K, 12)
+    assert [len(w) for w in m["A1_weights"]] == [n * K * K for n in (2, 3, 3, 2)]
+    assert sorted(m["M0_monomials"].keys()) == ["0", "1", "2", "3"]
+    assert len(m["M0_weights"]["2"]["3"]["1"]) == len(m["M0_monomials"]["3"])
+    assert max(len(t) for t in m["M1_monomials"]) == 3
+    assert max(m["Phi1_lme"]) == 39 and max(m["Phi1_lelm1lm2"]) == 87    # n_e = 40, n_r = 88
+    # spline grid as the extractor's: knots on linspace(1e-12, r_cut, n)
+    assert m["radial_spline_h"] == pytest.approx((m["r_cut"] - 1e-12) / 11)
+
+
+def test_capi_library_exports_declared_symbols():
+    """Every function declared in include/symmetrix_amd.h is exported by the built library."""
+    header = open(os.path.join(ROOT, "include", "symmetrix_amd.h")).read()
+    declared = set(re.findall(r"\b(smx_[a-zA-Z0-9_]+)\s*\(", header))
+    declared.discard("smx_model")
+    assert declared == set(_lib.EXPORTS)
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libsymmetrix_amd.so not built yet (python -c 'import __graft_entry__ as g; g.build()')")
+    L = C.CDLL(_lib.LIB_PATH)
+    for name in sorted(declared):
+        assert hasattr(L, name), name
+    L.smx_stage_names.restype = C.c_char_p
+    assert L.smx_stage_names().decode().split(";")[0] == "prep"
+
+
+def test_capi_error_paths_without_gpu(tmp_path):
+    """File errors are reported before any device is touched."""
+    if not os.path.exists(_lib.LIB_PATH):
+        pytest.skip("libsymmetrix_amd.so not built yet")
+    L = _lib.lib()
+    h = C.c_void_p()
+    assert L.smx_model_load(str(tmp_path / "missing.json").encode(), 0, C.byref(h)) == -2
+    assert b"cannot open" in L.smx_last_error()
+    bad = tmp_path / "bad.json"
+    bad.write_text('{"num_elements": 2, ')
+    assert L.smx_model_load(str(bad).encode(), 0, C.byref(h)) == -2
+    nokey = tmp_path / "nokey.json"
+    nokey.write_text('{"num_elements": 2}')
+    assert L.smx_model_load(str(nokey).encode(), 0, C.byref(h)) == -2
+    assert b"missing key" in L.smx_last_error()
+    assert L.smx_model_load(None, 0, C.byref(h)) == -1
+    m = H.tiny_model(K=2, L_max=0, n_pts=8)
+    m["M1_monomials"][0] = [0, 1, 2, 3]                      # degree 4: outside the device kernels
+    p = H.write_model(m, tmp_path / "deg4.json")
+    assert L.smx_model_load(p.encode(), 0, C.byref(h)) == -3
+    assert b"degree 4" in L.smx_last_error()
+    import torch
+    if not torch.cuda.is_available():
+        good = H.write_model(H.tiny_model(K=2, L_max=0, n_pts=8), tmp_path / "good.json")
+        assert L.smx_model_load(good.encode(), 0, C.byref(h)) == -4   # no device: fails loudly, no CPU path
+        with pytest.raises(RuntimeError):
+            from symmetrix_amd.mace import MACE
+            MACE(good)

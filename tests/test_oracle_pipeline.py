@@ -1,0 +1,219 @@
+"""The oracle's pipeline pinned with the reference's own test method (CPU only).
+
+symmetrix/test/test_mace.py checks every stage two ways: a stored sum (needs
+model files that cannot be fetched here) and the analytic adjoint against
+central finite differences (h = 1e-4, rtol 1e-4 / atol 1e-6, test_mace.py:73-84,
+145-159).  The second half is reproduced here stage by stage, plus what the
+mathematics fixes for the whole path: per-edge forces are the derivative of the
+total energy (test_mace.py:682-704), Newton's third law, and invariance of the
+energy under rotation, translation and relabelling of the atoms.
+"""
+import json
+import os
+
+import numpy as np
+import pytest
+from scipy.spatial.transform import Rotation
+
+from oracle.oracle import OracleMACE
+from tests import helpers as H
+
+GOLD = os.path.join(os.path.dirname(__file__), "golden")
+
+
+def numerical_gradient(f, x, h=1e-4):
+    g = np.zeros(len(x))
+    for i in range(len(x)):
+        x[i] += h; fp = f(x)
+        x[i] -= 2 * h; fm = f(x)
+        x[i] += h
+        g[i] = (fp - fm) / (2 * h)
+    f(x)
+    return g
+
+
+@pytest.fixture(scope="module", params=[0, 1], ids=["Lmax0", "Lmax1"])
+def setup(request):
+    model = H.tiny_model(K=3, L_max=request.param, n_pts=40)
+    orc = OracleMACE(model)
+    pos, cell, sp = H.small_system(7, seed=4)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    return model, orc, nl, ea
+
+
+def _r_of(xyz):
+    x = xyz.reshape(-1, 3)
+    return np.sqrt((x * x).sum(1))
+
+
+def test_A0_adjoint(setup):
+    model, orc, nl, ea = setup
+    N = ea["num_nodes"]
+    geo = (N, ea["node_types"], ea["num_neigh"], ea["neigh_types"])
+
+    def f(xyz):
+        r = _r_of(xyz)
+        orc.compute_Y(xyz); orc.compute_R0(*geo, r); orc.compute_A0(*geo)
+        return orc.A0.sum()
+    xyz = ea["xyz"].copy()
+    g = numerical_gradient(f, xyz)
+    orc.A0_adj = np.ones(len(orc.A0))
+    orc.node_forces = np.zeros(len(xyz))
+    orc.reverse_A0(*geo, xyz, _r_of(xyz))
+    assert np.allclose(-orc.node_forces, g, rtol=1e-4, atol=1e-6)
+
+
+def test_M0_H1_adjoints(setup):
+    model, orc, nl, ea = setup
+    N, nt = ea["num_nodes"], ea["node_types"]
+    A0 = orc.A0.copy()
+
+    def f(a):
+        orc.A0 = a; orc.compute_M0(N, nt)
+        return orc.M0.sum()
+    g = numerical_gradient(f, A0.copy())
+    orc.M0_adj = np.ones(len(orc.M0)); orc.reverse_M0(N, nt)
+    assert np.allclose(orc.A0_adj, g, rtol=1e-4, atol=1e-6)
+    M0 = orc.M0.copy()
+
+    def f2(m):
+        orc.M0 = m; orc.compute_H1(N)
+        return orc.H1.sum()
+    g = numerical_gradient(f2, M0.copy())
+    orc.H1_adj = np.ones(len(orc.H1)); orc.reverse_H1(N)
+    assert np.allclose(orc.M0_adj, g, rtol=1e-4, atol=1e-6)
+    orc.A0 = A0; orc.compute_M0(N, nt); orc.compute_H1(N)
+
+
+def test_Phi1_adjoint(setup):
+    model, orc, nl, ea = setup
+    N = ea["num_nodes"]
+    geo = (N, ea["node_types"], ea["num_neigh"], ea["neigh_types"])
+    H1 = orc.H1.copy()
+
+    def f(xyz):
+        r = _r_of(xyz)
+        orc.compute_Y(xyz); orc.compute_R1(*geo, r); orc.compute_Phi1(N, ea["num_neigh"], ea["neigh_indices"])
+        return orc.Phi1.sum()
+    xyz = ea["xyz"].copy()
+    g = numerical_gradient(f, xyz)
+    orc.Phi1_adj = np.ones(len(orc.Phi1))
+    orc.reverse_Phi1(N, ea["num_neigh"], ea["neigh_indices"], xyz, _r_of(xyz), True, True)
+    assert np.allclose(-orc.node_forces, g, rtol=1e-4, atol=1e-6)
+    H1_adj = orc.H1_adj.copy()
+
+    def f2(h):
+        orc.H1 = h; orc.compute_Phi1(N, ea["num_neigh"], ea["neigh_indices"])
+        return orc.Phi1.sum()
+    g = numerical_gradient(f2, H1.copy())
+    assert np.allclose(H1_adj, g, rtol=1e-4, atol=1e-6)
+    orc.H1 = H1
+
+
+def test_A1_M1_H2_readout_adjoints(setup):
+    model, orc, nl, ea = setup
+    N, nt = ea["num_nodes"], ea["node_types"]
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    Phi1 = orc.Phi1.copy()
+
+    def f(p):
+        orc.Phi1 = p; orc.compute_A1(N)
+        return orc.A1.sum()
+    g = numerical_gradient(f, Phi1.copy())
+    orc.A1_adj = np.ones(len(orc.A1)); orc.reverse_A1(N)
+    assert np.allclose(orc.Phi1_adj, g, rtol=1e-4, atol=1e-6)
+    A1 = orc.A1.copy()
+
+    def f2(a):
+        orc.A1 = a; orc.compute_M1(N, nt)
+        return orc.M1.sum()
+    g = numerical_gradient(f2, A1.copy())
+    orc.M1_adj = np.ones(len(orc.M1)); orc.reverse_M1(N, nt)
+    assert np.allclose(orc.A1_adj, g, rtol=1e-4, atol=1e-6)
+    M1 = orc.M1.copy(); H1 = orc.H1.copy()
+
+    def f3(m):
+        orc.M1 = m; orc.compute_H2(N, nt)
+        return orc.H2.sum()
+    g = numerical_gradient(f3, M1.copy())
+    orc.H2_adj = np.ones(len(orc.H2)); orc.reverse_H2(N, nt, True)
+    assert np.allclose(orc.M1_adj, g, rtol=1e-4, atol=1e-6)
+    H1_adj = orc.H1_adj.copy()
+
+    def f4(h):
+        orc.H1 = h; orc.compute_H2(N, nt)
+        return orc.H2.sum()
+    g = numerical_gradient(f4, H1.copy())
+    assert np.allclose(H1_adj, g, rtol=1e-4, atol=1e-6)
+    orc.H1 = H1
+    H2 = orc.H2.copy()
+
+    def f5(h2):
+        orc.H2 = h2
+        orc.node_energies = np.zeros(N)
+        orc.compute_readouts(N, nt)
+        return orc.node_energies.sum()
+    g = numerical_gradient(f5, H2.copy())
+    assert np.allclose(orc.H2_adj, g, rtol=1e-4, atol=1e-6)
+
+
+def test_total_energy_per_edge_forces(setup):
+    """test_mace.py:682-704: node_forces[ij] = -dE/dxyz_ij with every edge varied independently."""
+    model, orc, nl, ea = setup
+    args = list(H.call_args(ea))
+
+    def f(xyz):
+        a = list(args); a[5] = xyz; a[6] = _r_of(xyz)
+        orc.compute_node_energies_forces(*a)
+        return orc.node_energies.sum()
+    xyz = ea["xyz"].copy()
+    g = numerical_gradient(f, xyz)
+    assert np.allclose(-orc.node_forces, g, rtol=1e-4, atol=1e-6)
+
+
+def test_invariances():
+    model = H.tiny_model(K=4, L_max=1, n_pts=40)
+    orc = OracleMACE(model)
+    rng = np.random.default_rng(0)
+    big = np.array([60.0, 60.0, 60.0])
+    pos = rng.uniform(0, 4.5, size=(9, 3)) + 25.0
+    sp = rng.integers(0, 3, size=9).astype(np.int32)
+
+    def run(p, s):
+        nl, ea = H.edges_of(p, big, s, model["r_cut"])
+        orc.compute_node_energies_forces(*H.call_args(ea))
+        return orc.node_energies.sum(), H.atom_forces(nl, orc.node_forces, len(p)), orc.node_energies.copy()
+    E0, F0, e0 = run(pos, sp)
+    assert np.abs(F0.sum(0)).max() < 1e-12                      # Newton's third law
+    R = Rotation.random(random_state=3).as_matrix()
+    E1, F1, _ = run((pos - 27.0) @ R.T + 27.0, sp)
+    assert abs(E1 - E0) <= 1e-12 * abs(E0)                      # rotation
+    assert np.allclose(F0 @ R.T, F1, atol=1e-12)
+    E2, F2, _ = run(pos + np.array([1.3, -0.7, 2.1]), sp)        # translation
+    assert abs(E2 - E0) <= 1e-12 * abs(E0)
+    perm = rng.permutation(9)
+    E3, F3, e3 = run(pos[perm], sp[perm])                        # relabelling
+    assert abs(E3 - E0) <= 1e-12 * abs(E0)
+    assert np.allclose(e3, e0[perm], atol=1e-12)
+    assert np.allclose(F3, F0[perm], atol=1e-12)
+
+
+def test_isolated_and_empty():
+    model = H.tiny_model(K=2, L_max=0, n_pts=24)
+    orc = OracleMACE(model)
+    # an atom with no neighbours: E = E0 + MLP(0) = E0, and no force entries
+    orc.compute_node_energies_forces(1, [1], [0], [], [], [], [])
+    assert orc.node_energies[0] == pytest.approx(model["atomic_energies"][1], abs=1e-14)
+    assert len(orc.node_forces) == 0
+
+
+def test_golden_fixture_reproduced():
+    with open(os.path.join(GOLD, "tiny_model.json")) as f:
+        model = json.load(f)
+    z = np.load(os.path.join(GOLD, "tiny_case.npz"))
+    orc = OracleMACE(model)
+    orc.compute_node_energies_forces(len(z["node_types"]), z["node_types"], z["num_neigh"], z["neigh_indices"],
+                                     z["neigh_types"], z["xyz"], z["r"])
+    for name in ["Y", "A0", "M0", "H1", "Phi1", "A1", "M1", "H2", "H1_adj", "A0_adj", "node_energies", "node_forces"]:
+        assert np.allclose(getattr(orc, name), z[name], rtol=1e-13, atol=1e-15), name

@@ -1,0 +1,70 @@
+"""Calculator face: energy, per-atom energies, forces and stress of an atomic
+configuration, the work of `Symmetrix.calculate`
+(symmetrix/source/symmetrix/symmetrix_calc.py:72-102), without requiring ASE.
+
+`SymmetrixCalculator.compute(positions, cell, atomic_numbers)` builds the
+canonical neighbour list, calls the engine and reduces per-edge forces to atoms
+on the device.  When ASE is importable, `Symmetrix` is an
+`ase.calculators.calculator.Calculator` with the reference's constructor
+signature and `implemented_properties`.
+"""
+from __future__ import annotations
+
+import numpy as np
+
+from . import neighbors
+from .mace import MACE
+
+
+class SymmetrixCalculator:
+    implemented_properties = ["energy", "free_energy", "energies", "forces", "stress"]
+
+    def __init__(self, model_file, dtype="float64"):
+        if dtype not in ("float32", "float64"):
+            raise ValueError(f"Unsupported dtype '{dtype}'. Supported dtypes are 'float64' and 'float32'.")
+        self.evaluator = MACE(str(model_file), dtype)
+        self.cutoff = self.evaluator.r_cut
+        self.results = {}
+
+    def compute(self, positions, cell, atomic_numbers, pbc=(True, True, True)):
+        Z = [int(z) for z in atomic_numbers]
+        table = self.evaluator.atomic_numbers
+        try:
+            species = np.array([table.index(z) for z in Z], dtype=np.int32)
+        except ValueError as exc:
+            raise ValueError("an atom's element is not in the model") from exc
+        nl = neighbors.neighbor_list(positions, cell, self.cutoff, pbc)
+        ea = neighbors.edge_arrays(nl, species)
+        ev = self.evaluator
+        ev.compute_node_energies_forces(ea["num_nodes"], ea["node_types"], ea["num_neigh"], ea["neigh_indices"],
+                                        ea["neigh_types"], ea["xyz"], ea["r"])
+        energies = ev.node_energies
+        n_atoms = len(Z)
+        forces, virial = ev.reduce_forces(n_atoms, nl["j"], virial=True)
+        cell = np.asarray(cell, dtype=np.float64)
+        volume = abs(np.linalg.det(np.diag(cell) if cell.shape == (3,) else cell))
+        # symmetrix_calc.py:102: stress = -(pair_forces^T xyz)/V in Voigt order xx,yy,zz,yz,xz,xy
+        stress = -np.array([virial[0], virial[1], virial[2], virial[5], virial[4], virial[3]]) / volume
+        self.results = {"energy": float(energies.sum()), "free_energy": float(energies.sum()),
+                        "energies": energies, "forces": forces, "stress": stress}
+        return self.results
+
+
+try:  # pragma: no cover - ase is not installed in the build image
+    from ase.calculators.calculator import Calculator, all_changes
+
+    class Symmetrix(Calculator):
+        implemented_properties = SymmetrixCalculator.implemented_properties
+
+        def __init__(self, model_file, dtype="float64", use_kokkos=False, **kwargs):
+            Calculator.__init__(self, **kwargs)
+            self._impl = SymmetrixCalculator(model_file, dtype)
+            self.evaluator = self._impl.evaluator
+            self.cutoff = self._impl.cutoff
+
+        def calculate(self, atoms=None, properties=("energy",), system_changes=all_changes):
+            Calculator.calculate(self, atoms, properties, system_changes)
+            self.results = dict(self._impl.compute(self.atoms.get_positions(), self.atoms.get_cell().array,
+                                                   self.atoms.get_atomic_numbers(), self.atoms.get_pbc()))
+except ImportError:
+    Symmetrix = SymmetrixCalculator

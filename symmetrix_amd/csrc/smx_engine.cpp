@@ -20,6 +20,7 @@
 
 #include <cmath>
 #include <cstdio>
+#include <cstdlib>
 #include <cstring>
 #include <memory>
 #include <stdexcept>
@@ -145,18 +146,24 @@ struct Engine : EngineBase {
     DVec<int> B0_start, B0_lm1, B1_start, B1_lm1;
     DVec<double> B0_c, B1_c;
     std::vector<long> A1w_off;   // per l
+    // channel-slice tables (see smx_kernels_slice.hip); CH = 0 disables the path for that layer
+    DVec<F> tabS0, tabS1;
+    int slice_CH0 = 0, slice_CH1 = 0, slice_W = 0, slice_U0 = 0, slice_U1 = 0, num_cus = 0;
+    double cdiag1[16] = {};
+    DVec<double> fpart;
     DVec<double> H2w_H1, H2w_M1, ro1, ro2_w1, ro2_w2, E0;
     struct DevPoly {
-        DVec<int> row_i0, row_i1, row_start, entry_var;
+        DVec<int> packed, chunks;
         DVec<F> coef;
-        int num_rows = 0, num_entries = 0;
+        int num_entries = 0;
     };
     std::vector<std::unique_ptr<DevPoly>> P0;
     DevPoly P1;
     // pointer tables for the polynomial kernel: [0..num_LM) = P0, then P1
-    DVec<const int*> pp_i0, pp_i1, pp_start, pp_var;
+    DVec<const int4*> pp_packed;
+    DVec<const int*> pp_chunks;
     DVec<const F*> pp_coef;
-    DVec<int> pp_nrows, pp_nent;
+    DVec<int> pp_nent;
 
     // ---- geometry of the current edge list (device)
     DVec<int> g_node_types, g_num_neigh, g_neigh_indices, g_neigh_types;
@@ -198,6 +205,7 @@ struct Engine : EngineBase {
             for (auto& w : hm.A1_weights) { A1w_off.push_back((long)all.size()); all.insert(all.end(), w.begin(), w.end()); }
             upload_as(A1w, all, s);
         }
+        build_slices(s);
         // layer 0 couples Y_lm straight into output slot lm
         {
             std::vector<int> st(17), lm(16);
@@ -216,17 +224,17 @@ struct Engine : EngineBase {
         upload_as(ro2_w2, hm.readout_2_w2, s);
         upload_as(E0, hm.atomic_energies, s);
         auto up_poly = [&](DevPoly& d, const PolySpec& p) {
-            upload_as(d.row_i0, p.row_i0, s); upload_as(d.row_i1, p.row_i1, s);
-            upload_as(d.row_start, p.row_start, s); upload_as(d.entry_var, p.entry_var, s);
+            upload_as(d.packed, p.packed, s); upload_as(d.chunks, p.chunks, s);
             upload_as(d.coef, p.coef, s);
-            d.num_rows = (int)p.row_i0.size(); d.num_entries = p.num_entries;
+            d.num_entries = p.num_entries;
         };
-        std::vector<const int*> vi0, vi1, vst, vvar;
+        std::vector<const int4*> vpk;
+        std::vector<const int*> vch;
         std::vector<const F*> vco;
-        std::vector<int> vnr, vne;
+        std::vector<int> vne;
         auto reg = [&](DevPoly& d) {
-            vi0.push_back(d.row_i0.p); vi1.push_back(d.row_i1.p); vst.push_back(d.row_start.p);
-            vvar.push_back(d.entry_var.p); vco.push_back(d.coef.p); vnr.push_back(d.num_rows); vne.push_back(d.num_entries);
+            vpk.push_back(reinterpret_cast<const int4*>(d.packed.p)); vch.push_back(d.chunks.p);
+            vco.push_back(d.coef.p); vne.push_back(d.num_entries);
         };
         for (int LM = 0; LM < hm.num_LM; ++LM) {
             P0.emplace_back(new DevPoly());
@@ -235,12 +243,88 @@ struct Engine : EngineBase {
         }
         up_poly(P1, hm.P1);
         reg(P1);
-        pp_i0.upload(vi0.data(), vi0.size(), s); pp_i1.upload(vi1.data(), vi1.size(), s);
-        pp_start.upload(vst.data(), vst.size(), s); pp_var.upload(vvar.data(), vvar.size(), s);
+        pp_packed.upload(vpk.data(), vpk.size(), s); pp_chunks.upload(vch.data(), vch.size(), s);
         pp_coef.upload(vco.data(), vco.size(), s);
-        pp_nrows.upload(vnr.data(), vnr.size(), s); pp_nent.upload(vne.data(), vne.size(), s);
+        pp_nent.upload(vne.data(), vne.size(), s);
         flags.resize(4, s);
         HIPCHK(hipStreamSynchronize(s));
+    }
+
+    // Regroup a radial table per channel slice, or return 0 when the slice path does not apply.
+    int build_slice_table(const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst, hipStream_t s)
+    {
+        const int R = hm.spl_nodes - 1, Kc = hm.K, U = (int)tables.size();
+        if (nspl != 4 * Kc || U > 4) return 0;
+        hipDeviceProp_t prop;
+        int dev = 0;
+        HIPCHK(hipGetDevice(&dev));
+        HIPCHK(hipGetDeviceProperties(&prop, dev));
+        num_cus = prop.multiProcessorCount;
+        // LDS a single workgroup may use (opt-in limit where the runtime reports one)
+        size_t lds_cap = prop.sharedMemPerBlock;
+        if ((size_t)prop.sharedMemPerBlockOptin > lds_cap) lds_cap = prop.sharedMemPerBlockOptin;
+        if (lds_cap > 160 * 1024) lds_cap = 160 * 1024;
+        for (int CH = sizeof(F) == 8 ? 4 : 8; CH >= 2; CH /= 2) {
+            int W = 16 * CH;
+            const int step = 16 / (int)sizeof(F);
+            while (((W * (int)sizeof(F) / 4) / 4) % 2 == 0) W += step;   // rows land on different LDS bank groups
+            if ((size_t)R * W * sizeof(F) > lds_cap) continue;
+            const int S = (Kc + CH - 1) / CH;
+            std::vector<F> buf((size_t)S * U * R * W, F(0));
+            for (int sl = 0; sl < S; ++sl)
+                for (int u = 0; u < U; ++u)
+                    for (int n = 0; n < R; ++n)
+                        for (int q = 0; q < 4; ++q)
+                            for (int pth = 0; pth < 4; ++pth)
+                                for (int c = 0; c < CH; ++c) {
+                                    const int k = sl * CH + c;
+                                    if (k < Kc)
+                                        buf[(((size_t)sl * U + u) * R + n) * W + (q * 4 + pth) * CH + c] =
+                                            (F)tables[u][((size_t)n * 4 + q) * nspl + pth * Kc + k];
+                                }
+            dst.upload(buf.data(), buf.size(), s);
+            HIPCHK(hipStreamSynchronize(s));
+            slice_W = W;
+            return CH;
+        }
+        return 0;
+    }
+    void build_slices(hipStream_t s)
+    {
+        slice_CH0 = build_slice_table(hm.tables0, hm.nspl0, tabS0, s);
+        slice_U0 = (int)hm.tables0.size();
+        if (hm.L_max == 0) {
+            // layer 1 qualifies when every output slot lm is fed by harmonic lm alone
+            bool diag = hm.num_B == 16;
+            for (int b = 0; diag && b < 16; ++b) {
+                cdiag1[b] = 0.0;
+                for (int t = hm.B_start[b]; t < hm.B_start[b + 1]; ++t) {
+                    if (hm.B_lm1[t] != b) diag = false;
+                    else cdiag1[b] += hm.B_c[t];
+                }
+            }
+            if (diag) {
+                slice_CH1 = build_slice_table(hm.tables1, hm.nspl1, tabS1, s);
+                slice_U1 = (int)hm.tables1.size();
+            }
+        }
+    }
+    SliceParams<F> slice_params(int layer, int N)
+    {
+        SliceParams<F> p{};
+        p.a = agg_params(layer, N);
+        p.tabS = layer == 0 ? tabS0.p : tabS1.p;
+        p.U = layer == 0 ? slice_U0 : slice_U1;
+        p.W = slice_W;
+        p.CH = layer == 0 ? slice_CH0 : slice_CH1;
+        for (int q = 0; q < 16; ++q) p.cdiag[q] = layer == 0 ? 1.0 : cdiag1[q];
+        p.E = E;
+        p.num_cus = num_cus;
+        {
+            const char* ov = getenv(layer == 0 ? "SMX_SPLIT0" : "SMX_SPLIT1");
+            p.split_override = ov ? atoi(ov) : 0;
+        }
+        return p;
     }
 
     // ------------------------------------------------------------------
@@ -285,10 +369,10 @@ struct Engine : EngineBase {
     void build_sender_lists(int rows)
     {
         hipStream_t s = stream;
-        s_count.size_to(rows, s); s_start.size_to((size_t)rows + 1, s); s_cursor.size_to(rows, s);
+        s_count.size_to((size_t)2 * rows, s); s_start.size_to((size_t)rows + 1, s);
         s_list.size_to((size_t)E, s);
         scan_tmp.size_to((size_t)rows / 1024 + 2, s);
-        HIPCHK(launch_sender_lists(neigh_indices, (int)E, rows, s_count.p, s_start.p, s_cursor.p, s_list.p, scan_tmp.p, s));
+        HIPCHK(launch_sender_lists(neigh_indices, (int)E, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p, s));
         sender_rows = rows;
     }
     // Host-path validation of what the reference leaves unchecked (mace.cpp:17-64 trusts
@@ -362,6 +446,12 @@ struct Engine : EngineBase {
     {
         need(xyz, "xyz (compute_Y)"); need(r, "r (compute_R0)"); need(first_neigh.p, "num_neigh");
         Phi0.size_to((size_t)N * 16 * K(), stream);
+        if (slice_CH0) {
+            auto sp = slice_params(0, N);
+            sp.a.out = Phi0.p;
+            HIPCHK(launch_slice_fwd<F>(sp, stream));
+            return;
+        }
         auto p = agg_params(0, N);
         p.out = Phi0.p;
         HIPCHK(launch_agg_fwd<F>(0, p, stream));
@@ -392,7 +482,7 @@ struct Engine : EngineBase {
     void st_poly(int N, bool layer1)
     {
         PolyParams<F> p{};
-        p.num_nodes = N; p.K = K(); p.node_types = node_types;
+        p.num_nodes = N; p.K = K();
         const int off = layer1 ? NLM() : 0;
         p.NP = layer1 ? 1 : NLM();
         if (layer1) {
@@ -402,8 +492,9 @@ struct Engine : EngineBase {
             M0.size_to((size_t)N * NLM() * K(), stream); M0_grad.size_to((size_t)N * NLM() * 16 * K(), stream);
             p.A = A0.p; p.M = M0.p; p.M_grad = M0_grad.p;
         }
-        p.row_i0 = pp_i0.p + off; p.row_i1 = pp_i1.p + off; p.row_start = pp_start.p + off;
-        p.entry_var = pp_var.p + off; p.coef = pp_coef.p + off; p.num_rows = pp_nrows.p + off; p.num_entries = pp_nent.p + off;
+        p.packed = pp_packed.p + off; p.chunks = pp_chunks.p + off; p.coef = pp_coef.p + off; p.num_entries = pp_nent.p + off;
+        need(t_perm.p, "species groups");
+        p.perm = t_perm.p; p.tstart = t_start.p; p.T = hm.T;
         HIPCHK(launch_poly<F>(p, stream));
     }
     void st_H1(int N, bool reverse)
@@ -422,6 +513,12 @@ struct Engine : EngineBase {
     {
         need(xyz, "xyz (compute_Y)"); need(r, "r (compute_R1)"); need(neigh_indices, "neigh_indices");
         Phi1.size_to((size_t)N * NE() * K(), stream);
+        if (slice_CH1) {
+            auto sp = slice_params(1, N);
+            sp.a.out = Phi1.p;
+            HIPCHK(launch_slice_fwd<F>(sp, stream));
+            return;
+        }
         auto p = agg_params(1, N);
         p.out = Phi1.p;
         HIPCHK(launch_agg_fwd<F>(hm.L_max, p, stream));
@@ -510,10 +607,19 @@ struct Engine : EngineBase {
         const int k = K(), nlm = NLM();
         node_forces.resize((size_t)3 * E, stream);
         msg.size_to((size_t)E * nlm * k, stream);
-        auto p = agg_params(1, N);
-        p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
         stage_begin(ST_AGG1B);
-        HIPCHK(launch_agg_bwd<F>(hm.L_max, p, stream));
+        if (slice_CH1) {
+            auto sp = slice_params(1, N);
+            const int S = (k + sp.CH - 1) / sp.CH;
+            fpart.size_to((size_t)S * 3 * E, stream);
+            sp.a.d_out = dPhi1.p; sp.a.msg = msg.p; sp.fpart = fpart.p;
+            HIPCHK(launch_slice_bwd<F>(sp, stream));
+            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, stream));
+        } else {
+            auto p = agg_params(1, N);
+            p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
+            HIPCHK(launch_agg_bwd<F>(hm.L_max, p, stream));
+        }
         stage_end(ST_AGG1B);
         // edges beyond the first N receivers carry no layer-1 adjoint
         const long EN = E;  // first_neigh[N] == E whenever the list covers exactly N receivers
@@ -529,6 +635,15 @@ struct Engine : EngineBase {
     {
         need(xyz, "xyz"); need(r, "r");
         node_forces.resize((size_t)3 * E, stream);
+        if (slice_CH0) {
+            auto sp = slice_params(0, N);
+            const int S = (K() + sp.CH - 1) / sp.CH;
+            fpart.size_to((size_t)S * 3 * E, stream);
+            sp.a.d_out = Phi0.p; sp.a.msg = nullptr; sp.fpart = fpart.p;
+            HIPCHK(launch_slice_bwd<F>(sp, stream));
+            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, 1, stream));
+            return;
+        }
         auto p = agg_params(0, N);
         p.d_out = Phi0.p; p.forces = node_forces.p; p.accumulate_forces = 1; p.msg = nullptr;
         HIPCHK(launch_agg_bwd<F>(0, p, stream));
@@ -599,7 +714,7 @@ struct Engine : EngineBase {
         if (s == "Y" || s == "R0" || s == "R1") return;  // geometry remembered; evaluated inside the fused kernels
         if (s == "A0") { build_type_groups(N); st_agg0_fwd(N); st_A0_lin(N, false); }
         else if (s == "reverse_A0") { build_type_groups(N); st_A0_lin(N, true); st_agg0_bwd(N); }
-        else if (s == "M0") st_poly(N, false);
+        else if (s == "M0") { build_type_groups(N); st_poly(N, false); }
         else if (s == "reverse_M0") st_reverse_M0(N);
         else if (s == "H1") st_H1(N, false);
         else if (s == "reverse_H1") st_H1(N, true);
@@ -607,7 +722,7 @@ struct Engine : EngineBase {
         else if (s == "reverse_Phi1") { sender_rows = -1; st_agg1_bwd(N, fa != 0, fb != 0); }
         else if (s == "A1") st_A1(N, false);
         else if (s == "reverse_A1") st_A1(N, true);
-        else if (s == "M1") st_poly(N, true);
+        else if (s == "M1") { build_type_groups(N); st_poly(N, true); }
         else if (s == "reverse_M1") st_reverse_M1(N);
         else if (s == "H2") { build_type_groups(N); st_H2(N); }
         else if (s == "reverse_H2") { build_type_groups(N); st_reverse_H2(N, fa != 0); }

@@ -126,13 +126,54 @@ PolySpec build_poly(int num_lm, int T, int K, const std::vector<std::vector<int>
         P.entry_var.push_back(ents[i].c);
     }
     P.row_start.push_back((int)ents.size());
-    P.coef.assign((size_t)T * ents.size() * K, 0.0);
+    {
+        struct LE { int fa, fb, mono, first; };
+        std::vector<std::vector<LE>> lists(16);
+        for (size_t i = 0; i < ents.size(); ++i) {
+            const int f[3] = {ents[i].i0, ents[i].i1, ents[i].c};   // padded with ONE in front
+            bool first_done = false;
+            for (int pos = 0; pos < 3; ++pos) {
+                if (f[pos] == ONE) continue;
+                const int fa = f[(pos + 1) % 3], fb = f[(pos + 2) % 3];
+                const int is_first = first_done ? 0 : 1;
+                first_done = true;
+                lists[f[pos]].push_back(LE{fa, fb, (int)i, is_first});
+            }
+        }
+        P.list_start.assign(1, 0);
+        for (int v = 0; v < 16; ++v) {
+            std::stable_sort(lists[v].begin(), lists[v].end(), [](const LE& a, const LE& b) { return a.first > b.first; });
+            int nf = 0;
+            for (auto& e : lists[v]) {
+                nf += e.first;
+                P.list_fa.push_back(e.fa); P.list_fb.push_back(e.fb); P.list_mono.push_back(e.mono);
+            }
+            P.list_nfirst.push_back(nf);
+            P.list_start.push_back((int)P.list_fa.size());
+        }
+        if (ents.size() >= 65535) unsupported("more than 65534 monomials in one symmetric-contraction polynomial");
+        const int dummy = (int)ents.size() | (ONE << 16) | (ONE << 24);
+        for (int v = 0; v < 16; ++v) {
+            const int s0 = P.list_start[v], sf = s0 + P.list_nfirst[v], s1 = P.list_start[v + 1];
+            const int bounds[3] = {s0, sf, s1};
+            for (int part = 0; part < 2; ++part) {
+                int n = 0;
+                for (int e = bounds[part]; e < bounds[part + 1]; ++e, ++n)
+                    P.packed.push_back(P.list_mono[e] | (P.list_fa[e] << 16) | (P.list_fb[e] << 24));
+                while (n % 4) { P.packed.push_back(dummy); ++n; }
+                P.chunks.push_back(n / 4);
+            }
+        }
+        for (int q = 0; q < 4; ++q) P.packed.push_back(dummy);
+    }
+    // one extra all-zero coefficient row per species for the padding entries
+    P.coef.assign((size_t)T * (ents.size() + 1) * K, 0.0);
     for (int a = 0; a < T; ++a)
         for (int k = 0; k < K; ++k) {
             const std::vector<double>& w = coef_of(a, k);
             if (w.size() != monomials.size()) throw JsonError("model file: polynomial weights and monomials differ in length");
             for (size_t i = 0; i < ents.size(); ++i)
-                P.coef[((size_t)a * ents.size() + i) * K + k] = w[ents[i].src];
+                P.coef[((size_t)a * (ents.size() + 1) + i) * K + k] = w[ents[i].src];
         }
     return P;
 }

@@ -21,10 +21,23 @@ namespace smx {
 // share their first two factors.  Index 16 denotes the constant 1, so that a
 // monomial (a) is stored as (16,16,a) and (a,b) as (16,a,b).
 struct PolySpec {
-    int num_entries = 0;
+    int num_entries = 0;                         // distinct monomials
     std::vector<int> row_i0, row_i1, row_start;  // row_start has num_rows+1 entries
     std::vector<int> entry_var;                  // third factor of each entry
     std::vector<double> coef;                    // [T][num_entries][K]
+    // The same polynomial seen from each variable v: dP/dx_v = sum over the
+    // entries of list v of coef[mono] * x[fa] * x[fb] (a monomial appears once per
+    // occurrence of v in it).  The first list_nfirst[v] entries of list v are the
+    // monomials whose first factor is v, so P = sum_v x_v * (their partial sum).
+    std::vector<int> list_start;                 // [17]
+    std::vector<int> list_nfirst;                // [16]
+    std::vector<int> list_fa, list_fb, list_mono;
+    // Device form of the lists: entries packed as mono | fa << 16 | fb << 24, each
+    // half-list (first-factor entries of v, then the rest of v) padded to a
+    // multiple of four with entries that point at an all-zero coefficient row
+    // (index num_entries), plus one spare chunk at the end for the prefetch.
+    std::vector<int> packed;                     // [4 * (total chunks + 1)]
+    std::vector<int> chunks;                     // [32]: chunks of (v, first part), (v, rest)
 };
 
 struct HostModel {

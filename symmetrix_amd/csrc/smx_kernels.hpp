@@ -45,6 +45,29 @@ struct AggParams {
 template <typename F> hipError_t launch_agg_fwd(int L_max_H, const AggParams<F>& p, hipStream_t s);
 template <typename F> hipError_t launch_agg_bwd(int L_max_H, const AggParams<F>& p, hipStream_t s);
 
+// Channel-slice variant of the same two stages for scalar hidden features
+// (L_max = 0 path structure: output slot lm is fed by path l(lm) and harmonic lm
+// only, with a per-slot coupling constant cdiag[lm]).  tabS is the radial table
+// regrouped per slice: [slice][table][interval][W] with row content
+// [4 coefficients][4 paths][CH channels] padded to W elements.
+template <typename F>
+struct SliceParams {
+    AggParams<F> a;
+    const F* tabS;
+    int U;             // unique radial tables (one pass over the edges per table)
+    int W;             // padded row length in elements
+    int CH;            // channels per slice
+    double cdiag[16];
+    double* fpart;     // bwd: [slices][E][3] partial forces
+    long E;
+    int num_cus;
+    int split_override;   // lanes per receiver, 0 = choose from the average degree
+};
+template <typename F> hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s);
+template <typename F> hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s);
+// forces (+)= sum over slices of fpart, slices added in ascending order
+hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, hipStream_t s);
+
 // H1_adj[j] (+)= sum over edges with sender j of msg[e], in ascending edge order.
 template <typename F>
 hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg,
@@ -67,14 +90,17 @@ hipError_t launch_check_r(const double* r, long n, double r_cut, int* flags, hip
 template <typename F>
 struct PolyParams {
     int num_nodes, K, NP;              // NP polynomials (num_LM for M0, 1 for M1)
-    const int* node_types;
     const F* A;                        // [N][16][K]
     F* M;                              // [N][NP][K]
     F* M_grad;                         // [N][NP][16][K]
-    // per polynomial (device arrays of length NP)
-    const int* const* row_i0; const int* const* row_i1; const int* const* row_start;
-    const int* const* entry_var; const F* const* coef;   // coef[p]: [T][entries][K]
-    const int* num_rows; const int* num_entries;
+    // per polynomial (device arrays of length NP): per-variable entry lists, packed
+    // mono | fa << 16 | fb << 24 in chunks of four (padding entries address the
+    // all-zero row `num_entries`), and the chunk counts [32] = (v, first part), (v, rest)
+    const int4* const* packed;
+    const int* const* chunks;
+    const F* const* coef;              // coef[p]: [T][num_entries + 1][K]
+    const int* num_entries;            // monomials per polynomial
+    const int* perm; const int* tstart; int T;   // atoms grouped by species
 };
 template <typename F> hipError_t launch_poly(const PolyParams<F>& p, hipStream_t s);
 

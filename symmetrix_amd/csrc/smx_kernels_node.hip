@@ -85,17 +85,57 @@ __global__ void k_place(const int* key, long n, int rows, const int* start, int*
         if (j >= 0 && j < rows) list[start[j] + atomicAdd(&cursor[j], 1)] = (int)i;
     }
 }
-// ascending order inside every bucket: the placement above is unordered
-__global__ void k_sort_buckets(const int* start, int rows, int* list)
+// Ascending order inside every bucket (the atomic placement above is unordered).
+// One wavefront per bucket; entries are distinct, so the rank of an entry is the
+// number of smaller ones: bucket staged in LDS, every lane counts for its entries.
+constexpr int SORT_LDS = 1024;
+__global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows, int* list)
 {
-    const int j = blockIdx.x * blockDim.x + threadIdx.x;
-    if (j >= rows) return;
-    const int s0 = start[j], s1 = start[j + 1];
-    for (int a = s0 + 1; a < s1; ++a) {
-        const int v = list[a];
-        int b = a - 1;
-        while (b >= s0 && list[b] > v) { list[b + 1] = list[b]; --b; }
-        list[b + 1] = v;
+    __shared__ int buf[SORT_LDS];
+    const int j = blockIdx.x;
+    const int s0 = start[j], n = start[j + 1] - s0;
+    if (n <= 1) return;
+    if (n <= SORT_LDS) {
+        for (int t = threadIdx.x; t < n; t += 64) buf[t] = list[s0 + t];
+        __syncthreads();
+        for (int t = threadIdx.x; t < n; t += 64) {
+            const int v = buf[t];
+            int rank = 0;
+            for (int q = 0; q < n; ++q) rank += buf[q] < v;
+            list[s0 + rank] = v;
+        }
+    } else if (threadIdx.x == 0) {
+        // very long bucket: in-place insertion sort by one lane (correct, slow, not expected in practice)
+        for (int a = s0 + 1; a < s0 + n; ++a) {
+            const int v = list[a];
+            int b = a - 1;
+            while (b >= s0 && list[b] > v) { list[b + 1] = list[b]; --b; }
+            list[b + 1] = v;
+        }
+    }
+}
+// species groups in one block: LDS histogram, scan over the (few) species, placement
+__global__ __launch_bounds__(1024) void k_type_groups(const int* node_types, int N, int T, int* tstart, int* perm)
+{
+    extern __shared__ int sh[];   // [T] counts, [T] cursors
+    int* cnt = sh;
+    int* cur = sh + T;
+    for (int t = threadIdx.x; t < T; t += blockDim.x) { cnt[t] = 0; cur[t] = 0; }
+    __syncthreads();
+    for (int i = threadIdx.x; i < N; i += blockDim.x) {
+        const int t = node_types[i];
+        if (t >= 0 && t < T) atomicAdd(&cnt[t], 1);
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int acc = 0;
+        for (int t = 0; t < T; ++t) { const int c = cnt[t]; cnt[t] = acc; tstart[t] = acc; acc += c; }
+        tstart[T] = acc;
+    }
+    __syncthreads();
+    for (int i = threadIdx.x; i < N; i += blockDim.x) {
+        const int t = node_types[i];
+        if (t >= 0 && t < T) perm[cnt[t] + atomicAdd(&cur[t], 1)] = i;
     }
 }
 __global__ void k_check_range(const int* v, long n, int limit, int* flags)
@@ -122,14 +162,33 @@ __global__ void k_convert(const TS* s, TD* d, long n)
 }
 inline unsigned nblk(long n, int bs) { return (unsigned)((n + bs - 1) / bs); }
 
+// whole scan in one block (tiles visited in order with a running carry): one launch
+// instead of three while the array is short
+__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_single(const int* in, int* out, int n)
+{
+    int carry = 0;
+    for (int b0 = 0; b0 < n; b0 += SCAN_BLOCK) {
+        const int i = b0 + threadIdx.x;
+        const int v = i < n ? in[i] : 0;
+        int total;
+        const int ex = block_scan_exclusive(v, &total);
+        if (i < n) out[i] = carry + ex;
+        carry += total;
+    }
+    if (threadIdx.x == 0) out[n] = carry;
+}
 }  // namespace
 
 hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums, hipStream_t s)
 {
+    if (n <= 64 * SCAN_BLOCK) {
+        hipLaunchKernelGGL(k_scan_single, dim3(1), dim3(SCAN_BLOCK), 0, s, in, out, n);
+        return hipGetLastError();
+    }
     const int nb = (n + SCAN_BLOCK - 1) / SCAN_BLOCK;
-    if (nb > 0) hipLaunchKernelGGL(k_scan_tiles, dim3(nb), dim3(SCAN_BLOCK), 0, s, in, out, n, block_sums);
+    hipLaunchKernelGGL(k_scan_tiles, dim3(nb), dim3(SCAN_BLOCK), 0, s, in, out, n, block_sums);
     hipLaunchKernelGGL(k_scan_sums, dim3(1), dim3(SCAN_BLOCK), 0, s, block_sums, nb, out, n);
-    if (nb > 1) hipLaunchKernelGGL(k_scan_add, dim3(nb), dim3(SCAN_BLOCK), 0, s, out, n, block_sums);
+    hipLaunchKernelGGL(k_scan_add, dim3(nb), dim3(SCAN_BLOCK), 0, s, out, n, block_sums);
     return hipGetLastError();
 }
 
@@ -137,14 +196,18 @@ hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, i
                                int* slist, int* block_sums, hipStream_t s)
 {
     if (rows <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, count, (long)rows, 0);
-    hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, cursor, (long)rows, 0);
+    if (cursor == count + rows) {
+        hipLaunchKernelGGL(k_fill<int>, dim3(nblk(2L * rows, 256)), dim3(256), 0, s, count, 2L * rows, 0);
+    } else {
+        hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, count, (long)rows, 0);
+        hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, cursor, (long)rows, 0);
+    }
     if (E > 0) hipLaunchKernelGGL(k_count, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, count);
     hipError_t err = launch_scan_exclusive(count, sstart, rows, block_sums, s);
     if (err != hipSuccess) return err;
     if (E > 0) {
         hipLaunchKernelGGL(k_place, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, sstart, cursor, slist);
-        hipLaunchKernelGGL(k_sort_buckets, dim3(nblk(rows, 64)), dim3(64), 0, s, sstart, rows, slist);
+        hipLaunchKernelGGL(k_sort_buckets, dim3(rows), dim3(64), 0, s, sstart, rows, slist);
     }
     return hipGetLastError();
 }
@@ -152,17 +215,11 @@ hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, i
 hipError_t launch_type_groups(const int* node_types, int N, int T, int* tcount, int* tstart, int* cursor,
                               int* perm, int* block_sums, hipStream_t s)
 {
+    (void)tcount; (void)cursor; (void)block_sums;
     if (T <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_fill<int>, dim3(nblk(T, 256)), dim3(256), 0, s, tcount, (long)T, 0);
-    hipLaunchKernelGGL(k_fill<int>, dim3(nblk(T, 256)), dim3(256), 0, s, cursor, (long)T, 0);
-    if (N > 0) hipLaunchKernelGGL(k_count, dim3(nblk(N, 256)), dim3(256), 0, s, node_types, (long)N, T, tcount);
-    hipError_t err = launch_scan_exclusive(tcount, tstart, T, block_sums, s);
-    if (err != hipSuccess) return err;
-    if (N > 0) {
-        // order inside a type group is left as placed: every output row of the
-        // products that use this grouping is computed independently of its tile mates
-        hipLaunchKernelGGL(k_place, dim3(nblk(N, 256)), dim3(256), 0, s, node_types, (long)N, T, tstart, cursor, perm);
-    }
+    // order inside a species group is left as placed: every output row of the products
+    // that use this grouping is computed independently of its tile mates
+    hipLaunchKernelGGL(k_type_groups, dim3(1), dim3(1024), 2 * T * sizeof(int), s, node_types, N, T, tstart, perm);
     return hipGetLastError();
 }
 
@@ -197,62 +254,91 @@ template hipError_t launch_convert<double, double>(const double*, double*, long,
 template hipError_t launch_convert<float, float>(const float*, float*, long, hipStream_t);
 
 // ===========================================================================
-// Symmetric contraction.  One thread per (node, channel).  The 16 variables
-// and the 16 gradient accumulators of a thread live in LDS columns
-// ([17][blockDim], slot 16 = the constant 1) because the monomial indices come
-// from the model file and are wavefront-uniform but not compile-time.  Rows
-// share their first two factors, so one product p = x_i0 x_i1 serves a run of
-// entries: G[c] += w p, s += w x_c; then f += s p, G[i0] += s x_i1,
-// G[i1] += s x_i0.
+// Symmetric contraction.  Atoms are grouped by species (list preparation); a
+// thread owns one channel of two atoms of the same species, so every coefficient
+// it loads (coalesced over channels, [species][monomial][K]) serves two
+// evaluations.  The monomial indices come from the model file: the same for
+// every lane, but not compile-time, so the 16 variables of each atom live in an
+// LDS column ([17][block], slot 16 = the constant 1) that is only ever read in
+// the loops.  The polynomial is walked once per variable v: the entries of list
+// v give dP/dx_v = sum w x_fa x_fb in a register, written straight to M_grad;
+// the monomials that start with v come first in the list, and
+// P = sum_v x_v * (their partial sum).
 namespace {
 constexpr int POLY_BLOCK = 128;
+constexpr int POLY_NB = 2;       // atoms per thread
 
 template <typename F>
 __global__ __launch_bounds__(POLY_BLOCK) void k_poly(const PolyParams<F> a)
 {
-    __shared__ F X[17][POLY_BLOCK];
-    __shared__ F G[17][POLY_BLOCK];
+    __shared__ F X[POLY_NB][17][POLY_BLOCK];
     const int tid = threadIdx.x;
+    // species segment and pair of atoms of this block row
     const int kblocks = (a.K + POLY_BLOCK - 1) / POLY_BLOCK;
-    const int i = blockIdx.x / kblocks;
+    int type = -1, grp = blockIdx.x / kblocks, seg0 = 0, seg_n = 0;
+    for (int t = 0; t < a.T; ++t) {
+        const int n_t = a.tstart[t + 1] - a.tstart[t];
+        const int groups = (n_t + POLY_NB - 1) / POLY_NB;
+        if (grp < groups) { type = t; seg0 = a.tstart[t]; seg_n = n_t; break; }
+        grp -= groups;
+    }
+    if (type < 0) return;
     const int k = (blockIdx.x % kblocks) * POLY_BLOCK + tid;
-    const bool live = k < a.K;
-    const int type = a.node_types[i];
-    const int kk = live ? k : 0;
+    const bool klive = k < a.K;
+    const int kk = klive ? k : a.K - 1;
+    int node[POLY_NB];
+    bool nlive[POLY_NB];
 #pragma unroll
-    for (int q = 0; q < 16; ++q) X[q][tid] = a.A[((size_t)i * 16 + q) * a.K + kk];
-    X[16][tid] = F(1);
+    for (int b = 0; b < POLY_NB; ++b) {
+        const int j = grp * POLY_NB + b;
+        nlive[b] = j < seg_n;
+        node[b] = a.perm[seg0 + (nlive[b] ? j : seg_n - 1)];
+#pragma unroll
+        for (int q = 0; q < 16; ++q) X[b][q][tid] = a.A[((size_t)node[b] * 16 + q) * a.K + kk];
+        X[b][16][tid] = F(1);
+    }
+    // a thread reads back only its own columns: no barrier needed
     for (int pl = 0; pl < a.NP; ++pl) {
+        const int4* pk = a.packed[pl];
+        const int* nch = a.chunks[pl];
+        const F* coef = a.coef[pl] + (size_t)type * (a.num_entries[pl] + 1) * a.K + kk;
+        F f[POLY_NB];
 #pragma unroll
-        for (int q = 0; q < 17; ++q) G[q][tid] = F(0);
-        const int* ri0 = a.row_i0[pl];
-        const int* ri1 = a.row_i1[pl];
-        const int* rs = a.row_start[pl];
-        const int* ev = a.entry_var[pl];
-        const int nrows = a.num_rows[pl], nent = a.num_entries[pl];
-        const F* coef = a.coef[pl] + (size_t)type * nent * a.K + kk;
-        F f = F(0);
-        for (int rw = 0; rw < nrows; ++rw) {
-            const int i0 = ri0[rw], i1 = ri1[rw];
-            const F xa = X[i0][tid], xb = X[i1][tid];
-            const F p = xa * xb;
-            F s = F(0);
-            const int t1 = rs[rw + 1];
-            for (int t = rs[rw]; t < t1; ++t) {
-                const F w = coef[(size_t)t * a.K];
-                const int c = ev[t];
-                G[c][tid] += w * p;
-                s += w * X[c][tid];
+        for (int b = 0; b < POLY_NB; ++b) f[b] = F(0);
+        int4 cur = pk[0];
+        int c = 0;
+        for (int v = 0; v < 16; ++v) {
+            F g[POLY_NB];
+#pragma unroll
+            for (int b = 0; b < POLY_NB; ++b) g[b] = F(0);
+#pragma unroll
+            for (int part = 0; part < 2; ++part) {
+                const int n = nch[2 * v + part];
+                for (int j = 0; j < n; ++j) {
+                    const int4 nxt = pk[c + 1];   // next chunk's indices are in flight while this one is used
+                    const int e4[4] = {cur.x, cur.y, cur.z, cur.w};
+#pragma unroll
+                    for (int q = 0; q < 4; ++q) {
+                        const int mono = e4[q] & 0xffff, ia = (e4[q] >> 16) & 0xff, ib = (e4[q] >> 24) & 0xff;
+                        const F w = coef[(size_t)mono * a.K];
+#pragma unroll
+                        for (int b = 0; b < POLY_NB; ++b) g[b] += w * (X[b][ia][tid] * X[b][ib][tid]);
+                    }
+                    cur = nxt;
+                    ++c;
+                }
+                if (part == 0) {
+#pragma unroll
+                    for (int b = 0; b < POLY_NB; ++b) f[b] += X[b][v][tid] * g[b];
+                }
             }
-            f += s * p;
-            G[i0][tid] += s * xb;
-            G[i1][tid] += s * xa;
-        }
-        if (live) {
-            a.M[((size_t)i * a.NP + pl) * a.K + k] = f;
 #pragma unroll
-            for (int q = 0; q < 16; ++q) a.M_grad[(((size_t)i * a.NP + pl) * 16 + q) * a.K + k] = G[q][tid];
+            for (int b = 0; b < POLY_NB; ++b)
+                if (klive && nlive[b]) a.M_grad[(((size_t)node[b] * a.NP + pl) * 16 + v) * a.K + k] = g[b];
         }
+#pragma unroll
+        for (int b = 0; b < POLY_NB; ++b)
+            if (klive && nlive[b]) a.M[((size_t)node[b] * a.NP + pl) * a.K + k] = f[b];
     }
 }
 
@@ -277,7 +363,8 @@ hipError_t launch_poly(const PolyParams<F>& p, hipStream_t s)
 {
     if (p.num_nodes <= 0) return hipSuccess;
     const int kblocks = (p.K + POLY_BLOCK - 1) / POLY_BLOCK;
-    hipLaunchKernelGGL(k_poly<F>, dim3((unsigned)p.num_nodes * kblocks), dim3(POLY_BLOCK), 0, s, p);
+    const unsigned groups = (unsigned)((p.num_nodes + POLY_NB - 1) / POLY_NB + p.T);
+    hipLaunchKernelGGL(k_poly<F>, dim3(groups * kblocks), dim3(POLY_BLOCK), 0, s, p);
     return hipGetLastError();
 }
 template hipError_t launch_poly<double>(const PolyParams<double>&, hipStream_t);

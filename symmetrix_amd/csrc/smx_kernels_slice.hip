@@ -1,0 +1,369 @@
+// Channel-slice edge kernels for gfx950 (scalar hidden features, P = 4 paths).
+//
+// The radial spline table is the hot operand of the edge stages: every edge
+// needs 4 coefficient rows x 4 paths x K channels (12 KB at K = 96 in double),
+// far more than its geometry or its sender row.  These kernels cut the channel
+// axis into slices of CH channels, small enough that the whole table slice
+// ([intervals][4][4][CH], about 130 KB) stays resident in the 160 KB LDS of a
+// CU.  A block owns one slice; its lanes own receivers (SPLIT lanes share one
+// receiver and take alternate edges) and walk the receiver's edge list, so that
+//   - spline coefficients come from LDS, never from L2/HBM, after one
+//     contiguous copy of the slice per block,
+//   - harmonics are evaluated by the lane that uses them (no staging),
+//   - accumulators (16 x CH per lane) stay in registers, sums run in edge
+//     order, no atomics: results are bit-reproducible.
+// The adjoint kernel writes, per slice, a partial force per edge; a last kernel
+// adds the partials over slices in a fixed order.
+#include "smx_kernels.hpp"
+
+namespace smx {
+
+namespace {
+
+__device__ __forceinline__ void sph_l3_s(double x, double y, double z, double* Y)
+{
+    const double s3 = 1.7320508075688772, s15 = 3.872983346207417, s5h = 1.118033988749895;
+    const double s15h = 1.9364916731037085, c3a = 2.091650066335189, s105 = 10.246950765959598;
+    const double c3c = 1.620185174601965, c3d = 1.3228756555322954, c3e = 5.123475382979799;
+    const double xx = x * x, yy = y * y, zz = z * z;
+    Y[0] = 1.0;
+    Y[1] = s3 * y; Y[2] = s3 * z; Y[3] = s3 * x;
+    Y[4] = s15 * x * y; Y[5] = s15 * y * z; Y[6] = s5h * (2 * zz - xx - yy);
+    Y[7] = s15 * x * z; Y[8] = s15h * (xx - yy);
+    Y[9] = c3a * y * (3 * xx - yy); Y[10] = s105 * x * y * z;
+    Y[11] = c3c * y * (4 * zz - xx - yy); Y[12] = c3d * z * (2 * zz - 3 * xx - 3 * yy);
+    Y[13] = c3c * x * (4 * zz - xx - yy); Y[14] = c3e * (xx - yy) * z; Y[15] = c3a * x * (xx - 3 * yy);
+}
+
+// harmonics Y[16] and the derivative of their homogeneous forms along the permuted axes, g[3][16]
+__device__ __forceinline__ void sph_l3_g(double x, double y, double z, double* Y, double (*g)[16])
+{
+    const double s3 = 1.7320508075688772, s15 = 3.872983346207417, s5h = 1.118033988749895;
+    const double s15h = 1.9364916731037085, c3a = 2.091650066335189, s105 = 10.246950765959598;
+    const double c3c = 1.620185174601965, c3d = 1.3228756555322954, c3e = 5.123475382979799;
+    const double xx = x * x, yy = y * y, zz = z * z;
+    Y[0] = 1.0;                              g[0][0] = 0;               g[1][0] = 0;                g[2][0] = 0;
+    Y[1] = s3 * y;                           g[0][1] = 0;               g[1][1] = s3;               g[2][1] = 0;
+    Y[2] = s3 * z;                           g[0][2] = 0;               g[1][2] = 0;                g[2][2] = s3;
+    Y[3] = s3 * x;                           g[0][3] = s3;              g[1][3] = 0;                g[2][3] = 0;
+    Y[4] = s15 * x * y;                      g[0][4] = s15 * y;         g[1][4] = s15 * x;          g[2][4] = 0;
+    Y[5] = s15 * y * z;                      g[0][5] = 0;               g[1][5] = s15 * z;          g[2][5] = s15 * y;
+    Y[6] = s5h * (2 * zz - xx - yy);         g[0][6] = -2 * s5h * x;    g[1][6] = -2 * s5h * y;     g[2][6] = 4 * s5h * z;
+    Y[7] = s15 * x * z;                      g[0][7] = s15 * z;         g[1][7] = 0;                g[2][7] = s15 * x;
+    Y[8] = s15h * (xx - yy);                 g[0][8] = 2 * s15h * x;    g[1][8] = -2 * s15h * y;    g[2][8] = 0;
+    Y[9] = c3a * y * (3 * xx - yy);          g[0][9] = 6 * c3a * x * y; g[1][9] = 3 * c3a * (xx - yy); g[2][9] = 0;
+    Y[10] = s105 * x * y * z;                g[0][10] = s105 * y * z;   g[1][10] = s105 * x * z;    g[2][10] = s105 * x * y;
+    Y[11] = c3c * y * (4 * zz - xx - yy);    g[0][11] = -2 * c3c * x * y; g[1][11] = c3c * (4 * zz - xx - 3 * yy); g[2][11] = 8 * c3c * y * z;
+    Y[12] = c3d * z * (2 * zz - 3 * xx - 3 * yy); g[0][12] = -6 * c3d * x * z; g[1][12] = -6 * c3d * y * z; g[2][12] = 3 * c3d * (2 * zz - xx - yy);
+    Y[13] = c3c * x * (4 * zz - xx - yy);    g[0][13] = c3c * (4 * zz - 3 * xx - yy); g[1][13] = -2 * c3c * x * y; g[2][13] = 8 * c3c * x * z;
+    Y[14] = c3e * (xx - yy) * z;             g[0][14] = 2 * c3e * x * z; g[1][14] = -2 * c3e * y * z; g[2][14] = c3e * (xx - yy);
+    Y[15] = c3a * x * (xx - 3 * yy);         g[0][15] = 3 * c3a * (xx - yy); g[1][15] = -6 * c3a * x * y; g[2][15] = 0;
+}
+
+__device__ __forceinline__ int pair_index_s(int T, int a, int b)
+{
+    return (a <= b) ? a * (2 * T - a - 1) / 2 + b : b * (2 * T - b - 1) / 2 + a;
+}
+
+__device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, size_t bytes)
+{
+    // both sides 16-byte aligned, size a multiple of 16
+    const uint4* s = reinterpret_cast<const uint4*>(src);
+    uint4* d = reinterpret_cast<uint4*>(dst);
+    const size_t n = bytes / 16;
+    for (size_t q = threadIdx.x; q < n; q += blockDim.x) d[q] = s[q];
+}
+
+constexpr int lm_l(int lm) { return lm < 1 ? 0 : (lm < 4 ? 1 : (lm < 9 ? 2 : 3)); }
+
+// value of the lane ROT places further round its 16-lane row (DPP row_ror: a VALU move, no LDS traffic)
+template <int ROT>
+__device__ __forceinline__ float row_rotate(float v)
+{
+    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + ROT, 0xf, 0xf, false));
+}
+template <int ROT>
+__device__ __forceinline__ double row_rotate(double v)
+{
+    const long long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), 0x120 + ROT, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), 0x120 + ROT, 0xf, 0xf, false);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
+// sum over the lanes of a 16-lane row whose index agrees modulo CL (CL = 1, 2, 4 or 8)
+template <int CL, typename T>
+__device__ __forceinline__ T row_sum_strided(T v)
+{
+    if constexpr (CL <= 8) v += row_rotate<8>(v);
+    if constexpr (CL <= 4) v += row_rotate<4>(v);
+    if constexpr (CL <= 2) v += row_rotate<2>(v);
+    if constexpr (CL <= 1) v += row_rotate<1>(v);
+    return v;
+}
+
+// ---------------------------------------------------------------------------
+// Lane mapping of both kernels.  A wavefront works on four receivers at a time,
+// one per 16-lane row.  Inside a row, CL lanes share an edge and split the CH
+// channels of the slice between them (CPLN = CH/CL consecutive channels per
+// lane, one 16-byte LDS read per coefficient), and 16/CL edges are in flight.
+// The LDS unit serves a 16-byte read 8 lanes per cycle, i.e. 8/CL edges whose
+// lanes read adjacent bytes: far fewer distinct rows per cycle than with one
+// edge per lane, hence far fewer bank conflicts.
+template <typename F, int CH, int CL, int BT>
+__global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const F* lds = reinterpret_cast<const F*>(smem);
+    const AggParams<F>& a = p.a;
+    constexpr int CPLN = CH / CL, EPR = 16 / CL;
+    const int slice = blockIdx.x, K = a.K;
+    const int W = p.W, R = a.spl_nodes - 1;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int sub = lane & 15, e_sub = sub / CL, cs = sub % CL;
+    const int kc = slice * CH + cs * CPLN;                 // first channel of this lane
+    const int wave_tasks = (a.num_nodes + 3) / 4;
+    const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
+
+    for (int u = 0; u < p.U; ++u) {
+        __syncthreads();
+        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
+        __syncthreads();
+        for (int task = wave_id; task < wave_tasks; task += wave_stride) {
+            const int i = task * 4 + (lane >> 4);
+            const bool live = i < a.num_nodes;
+            int e0 = 0, e1 = 0, ti = 0;
+            if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
+            F acc[16][CPLN];
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c) acc[q][c] = F(0);
+            for (int e = e0 + e_sub; e < e1; e += EPR) {
+                const int tj = a.neigh_types[e];
+                if (p.U > 1 && a.pair_table[pair_index_s(a.T, ti, tj)] != u) continue;
+                const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
+                const double r = a.r[e];
+                const int g = a.gather[e];
+                const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
+                double Yd[16];
+                sph_l3_s(dz * inv, dx * inv, dy * inv, Yd);
+                int n = (int)(r / a.spl_h);
+                n = min(max(n, 0), R - 1);
+                const F x = (F)(r - a.spl_h * n);
+                const F* row = lds + (size_t)n * W + cs * CPLN;
+                F t[4][CPLN];
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c) {
+                    const F h = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)];
+#pragma unroll
+                    for (int l = 0; l < 4; ++l) {
+                        const F c0 = row[(0 * 4 + l) * CH + c], c1 = row[(1 * 4 + l) * CH + c];
+                        const F c2 = row[(2 * 4 + l) * CH + c], c3 = row[(3 * 4 + l) * CH + c];
+                        t[l][c] = (c0 + x * (c1 + x * (c2 + x * c3))) * h;
+                    }
+                }
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                    const F y = (F)Yd[q];
+#pragma unroll
+                    for (int c = 0; c < CPLN; ++c) acc[q][c] += t[lm_l(q)][c] * y;
+                }
+            }
+            // add up the lanes of the row that hold the same channels (they took alternate edges)
+#pragma unroll
+            for (int q = 0; q < 16; ++q)
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c) acc[q][c] = row_sum_strided<CL>(acc[q][c]);
+            if (live && e_sub == 0) {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) {
+                    const F cd = (F)p.cdiag[q];
+#pragma unroll
+                    for (int c = 0; c < CPLN; ++c)
+                        if (kc + c < K) {
+                            F* o = a.out + ((size_t)i * 16 + q) * K + kc + c;
+                            *o = (u == 0) ? acc[q][c] * cd : *o + acc[q][c] * cd;
+                        }
+                }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
+template <typename F, int CH, int CL, int BT>
+__global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
+{
+    extern __shared__ __align__(16) unsigned char smem[];
+    const F* lds = reinterpret_cast<const F*>(smem);
+    const AggParams<F>& a = p.a;
+    constexpr int CPLN = CH / CL, EPR = 16 / CL;
+    const int slice = blockIdx.x, K = a.K;
+    const int W = p.W, R = a.spl_nodes - 1;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int sub = lane & 15, e_sub = sub / CL, cs = sub % CL;
+    const int kc = slice * CH + cs * CPLN;
+    const int wave_tasks = (a.num_nodes + 3) / 4;
+    const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
+    double* fpart = p.fpart + (size_t)slice * p.E * 3;
+
+    for (int u = 0; u < p.U; ++u) {
+        __syncthreads();
+        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
+        __syncthreads();
+        for (int task = wave_id; task < wave_tasks; task += wave_stride) {
+            const int i = task * 4 + (lane >> 4);
+            const bool live = i < a.num_nodes;
+            int e0 = 0, e1 = 0, ti = 0;
+            if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
+            F d[16][CPLN];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const F cd = (F)p.cdiag[q];
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c)
+                    d[q][c] = (live && kc + c < K) ? a.d_out[((size_t)i * 16 + q) * K + kc + c] * cd : F(0);
+            }
+            // the lanes of a row iterate together so that the cross-lane sums below see all CL partners
+            const int iters = (e1 - e0 + EPR - 1) / EPR;
+            for (int it = 0; it < iters; ++it) {
+                const int e = e0 + it * EPR + e_sub;
+                bool on = e < e1;
+                int tj = 0;
+                if (on) {
+                    tj = a.neigh_types[e];
+                    if (p.U > 1 && a.pair_table[pair_index_s(a.T, ti, tj)] != u) on = false;
+                }
+                double fx = 0.0, fy = 0.0, fz = 0.0;
+                if (on) {
+                    const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
+                    const double r = a.r[e];
+                    const int g = a.gather[e];
+                    const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
+                    const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
+                    double Yd[16], gd[3][16];
+                    sph_l3_g(ux, uy, uz, Yd, gd);
+                    int n = (int)(r / a.spl_h);
+                    n = min(max(n, 0), R - 1);
+                    const F x = (F)(r - a.spl_h * n);
+                    const F* row = lds + (size_t)n * W + cs * CPLN;
+                    F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
+#pragma unroll
+                    for (int c = 0; c < CPLN; ++c) {
+                        const F h = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)];
+                        F mg = F(0);
+#pragma unroll
+                        for (int l = 0; l < 4; ++l) {
+                            const F c0 = row[(0 * 4 + l) * CH + c], c1 = row[(1 * 4 + l) * CH + c];
+                            const F c2 = row[(2 * 4 + l) * CH + c], c3 = row[(3 * 4 + l) * CH + c];
+                            const F Rv = c0 + x * (c1 + x * (c2 + x * c3));
+                            const F Rd = c1 + x * (F(2) * c2 + F(3) * x * c3);
+                            F ul = F(0), v0 = F(0), v1 = F(0), v2 = F(0);
+#pragma unroll
+                            for (int m = 0; m < 2 * l + 1; ++m) {
+                                const int q = l * l + m;
+                                const F dd = d[q][c];
+                                ul += dd * (F)Yd[q];
+                                v0 += dd * (F)gd[0][q]; v1 += dd * (F)gd[1][q]; v2 += dd * (F)gd[2][q];
+                            }
+                            const F Rh = Rv * h;
+                            srad += Rd * h * ul;
+                            wx += Rh * v0; wy += Rh * v1; wz += Rh * v2;
+                            lterm += Rh * ul * F(l);
+                            mg += Rv * ul;
+                        }
+                        if (a.msg && kc + c < K) a.msg[(size_t)e * K + kc + c] = mg;
+                    }
+                    // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
+                    // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
+                    const double sr = (double)srad, lt = (double)lterm;
+                    const double ir = 1.0 / r;
+                    fx = -(dx * ir * sr + ((double)wy - uy * lt) * inv);   // original x is permuted axis 1
+                    fy = -(dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
+                    fz = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
+                }
+                // channels of the slice are spread over CL adjacent lanes: add their partial forces
+#pragma unroll
+                for (int off = 1; off < CL; off <<= 1) {
+                    fx += __shfl_xor(fx, off, 64); fy += __shfl_xor(fy, off, 64); fz += __shfl_xor(fz, off, 64);
+                }
+                if (on && cs == 0) {
+                    fpart[3 * (size_t)e] = fx; fpart[3 * (size_t)e + 1] = fy; fpart[3 * (size_t)e + 2] = fz;
+                }
+            }
+        }
+    }
+}
+
+__global__ void k_fpart_reduce(long n3, int nslices, const double* fpart, double* forces, int accumulate)
+{
+    const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (t >= n3) return;
+    double s = accumulate ? forces[t] : 0.0;
+    for (int q = 0; q < nslices; ++q) s += fpart[(size_t)q * n3 + t];
+    forces[t] = s;
+}
+
+template <typename F, int CH, bool BWD>
+hipError_t launch_slice_t(const SliceParams<F>& p, hipStream_t s)
+{
+    constexpr int BT = 512;
+    constexpr int CL = 2;
+    const int S = (p.a.K + CH - 1) / CH;
+    const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F);
+    const int waves_per_block = BT / 64;
+    // one block per CU (the slice fills most of its LDS); receiver groups share a slice
+    int RG = p.num_cus / S;
+    if (RG < 1) RG = 1;
+    const long tasks_per_slice = ((long)p.a.num_nodes + 3) / 4;
+    if ((long)RG * waves_per_block > tasks_per_slice) RG = (int)((tasks_per_slice + waves_per_block - 1) / waves_per_block);
+    dim3 grid(S, RG);
+    void (*kern)(const SliceParams<F>) = nullptr;
+    if constexpr (BWD) kern = k_slice_bwd<F, CH, CL, BT>;
+    else kern = k_slice_fwd<F, CH, CL, BT>;
+    if (lds > 64 * 1024) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+    }
+    hipLaunchKernelGGL(kern, grid, dim3(BT), lds, s, p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+template <typename F>
+hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s)
+{
+    if (p.a.num_nodes <= 0) return hipSuccess;
+    switch (p.CH) {
+    case 2: return launch_slice_t<F, 2, false>(p, s);
+    case 4: return launch_slice_t<F, 4, false>(p, s);
+    case 8: return launch_slice_t<F, 8, false>(p, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+template <typename F>
+hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s)
+{
+    if (p.a.num_nodes <= 0) return hipSuccess;
+    switch (p.CH) {
+    case 2: return launch_slice_t<F, 2, true>(p, s);
+    case 4: return launch_slice_t<F, 4, true>(p, s);
+    case 8: return launch_slice_t<F, 8, true>(p, s);
+    default: return hipErrorInvalidValue;
+    }
+}
+template hipError_t launch_slice_fwd<double>(const SliceParams<double>&, hipStream_t);
+template hipError_t launch_slice_fwd<float>(const SliceParams<float>&, hipStream_t);
+template hipError_t launch_slice_bwd<double>(const SliceParams<double>&, hipStream_t);
+template hipError_t launch_slice_bwd<float>(const SliceParams<float>&, hipStream_t);
+
+hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, hipStream_t s)
+{
+    const long n3 = 3 * E;
+    if (n3 <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_fpart_reduce, dim3((unsigned)((n3 + 255) / 256)), dim3(256), 0, s, n3, nslices, fpart, forces, accumulate);
+    return hipGetLastError();
+}
+
+}  // namespace smx

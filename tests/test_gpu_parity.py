@@ -82,6 +82,23 @@ def test_pipeline_matches_oracle(gpu, tmp_models, K, L_max, natoms, pair, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("K,natoms", [(20, 70), (96, 200), (33, 9)])
+def test_two_species_three_radial_tables(gpu, tmp_models, K, natoms, dtype):
+    """Scalar hidden features with a few distinct pair tables: the channel-slice
+    kernels make one pass over the edges per table."""
+    model = H.tiny_model(K=K, L_max=0, T=(1, 8), n_pts=50, seed=K, pair=True)
+    path = H.write_model(model, tmp_models / f"two_{K}.json")
+    orc = _oracle()(model)
+    eng = gpu(path, dtype)
+    pos, cell, sp = H.small_system(natoms, probs=(0.6, 0.4), seed=natoms)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K={K} atoms={natoms} edges={len(ea['r'])} {dtype}", flush=True)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    _compare(orc, eng, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
 def test_golden_fixture(gpu, dtype):
     z = np.load(os.path.join(GOLD, "tiny_case.npz"))
     eng = gpu(os.path.join(GOLD, "tiny_model.json"), dtype)
@@ -236,3 +253,35 @@ def test_full_size_properties(gpu, tmp_models, workload):
     e32.compute_node_energies_forces(*H.call_args(ea))
     assert abs(e32.node_energies.sum() - E64) <= 1e-5 * abs(E64)
     assert np.abs(e32.node_forces - f64).max() <= 1e-4
+
+
+def test_calculator_energy_forces_stress(gpu, tmp_models):
+    """The calculator face (symmetrix_calc.py:72-102): forces are -dE/dx and the
+    stress is dE/d(strain)/V, both checked by central differences of the engine's own energy."""
+    from symmetrix_amd.calc import SymmetrixCalculator
+    model = H.tiny_model(K=16, L_max=1, n_pts=64, seed=21)
+    path = H.write_model(model, tmp_models / "calc.json")
+    calc = SymmetrixCalculator(path)
+    pos, cell, sp = H.small_system(14, density=0.09, seed=8)
+    Z = np.array(model["atomic_numbers"])[sp]
+    res = calc.compute(pos, cell, Z)
+    orc = _oracle()(model)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    assert res["energy"] == pytest.approx(orc.node_energies.sum(), rel=1e-10)
+    assert np.allclose(res["forces"], H.atom_forces(nl, orc.node_forces, len(pos)), atol=1e-8)
+    F, e0 = res["forces"].copy(), res["energy"]
+    h = 1e-5
+    for a, c in ((0, 0), (3, 1), (7, 2)):
+        p = pos.copy(); p[a, c] += h; ep = calc.compute(p, cell, Z)["energy"]
+        p[a, c] -= 2 * h; em = calc.compute(p, cell, Z)["energy"]
+        assert -(ep - em) / (2 * h) == pytest.approx(F[a, c], abs=1e-6)
+    stress = calc.compute(pos, cell, Z)["stress"]
+    V = float(np.prod(cell))
+    voigt = [(0, 0), (1, 1), (2, 2), (1, 2), (0, 2), (0, 1)]
+    for q, (a, b) in enumerate(voigt):
+        def strained(eps):
+            S = np.eye(3); S[a, b] += eps / 2; S[b, a] += eps / 2
+            return calc.compute(pos @ S.T, np.diag(cell) @ S.T, Z)["energy"]
+        d = (strained(h) - strained(-h)) / (2 * h) / V
+        assert d == pytest.approx(stress[q], abs=1e-6)

@@ -127,3 +127,12 @@ def test_capi_error_paths_without_gpu(tmp_path):
         with pytest.raises(RuntimeError):
             from symmetrix_amd.mace import MACE
             MACE(good)
+
+
+def test_cpp_class_header_compiles():
+    """include/symmetrix_amd/mace.hpp is a drop-in for libsymmetrix's mace.hpp for a C++20 caller."""
+    import subprocess
+    src = '#include "mace.hpp"\n#include <memory>\nint f(){ std::unique_ptr<MACE> m; return m ? m->num_channels : 0; }\n'
+    r = subprocess.run(["g++", "-std=c++20", "-fsyntax-only", "-I", os.path.join(ROOT, "include", "symmetrix_amd"),
+                        "-x", "c++", "-"], input=src.encode(), capture_output=True)
+    assert r.returncode == 0, r.stderr.decode()

@@ -76,6 +76,21 @@ __device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, si
 
 constexpr int lm_l(int lm) { return lm < 1 ? 0 : (lm < 4 ? 1 : (lm < 9 ? 2 : 3)); }
 
+struct EdgeGeo {
+    double dx, dy, dz, r;
+    int g, tj;
+};
+template <typename F>
+__device__ __forceinline__ EdgeGeo load_edge(const AggParams<F>& a, int e)
+{
+    EdgeGeo q;
+    q.dx = a.xyz[3 * (size_t)e]; q.dy = a.xyz[3 * (size_t)e + 1]; q.dz = a.xyz[3 * (size_t)e + 2];
+    q.r = a.r[e];
+    q.g = a.gather[e];
+    q.tj = a.neigh_types[e];
+    return q;
+}
+
 // value of the lane ROT places further round its 16-lane row (DPP row_ror: a VALU move, no LDS traffic)
 template <int ROT>
 __device__ __forceinline__ float row_rotate(float v)
@@ -138,12 +153,20 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
             for (int q = 0; q < 16; ++q)
 #pragma unroll
                 for (int c = 0; c < CPLN; ++c) acc[q][c] = F(0);
+            // the geometry of the next edge of this lane is loaded while the current one is processed
+            EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0, 0};
+            {
+                const int ef = e0 + e_sub;
+                if (ef < e1) nx = load_edge(a, ef);
+            }
             for (int e = e0 + e_sub; e < e1; e += EPR) {
-                const int tj = a.neigh_types[e];
+                const EdgeGeo cu = nx;
+                if (e + EPR < e1) nx = load_edge(a, e + EPR);
+                const int tj = cu.tj;
                 if (p.U > 1 && a.pair_table[pair_index_s(a.T, ti, tj)] != u) continue;
-                const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
-                const double r = a.r[e];
-                const int g = a.gather[e];
+                const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
+                const double r = cu.r;
+                const int g = cu.g;
                 const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
                 double Yd[16];
                 sph_l3_s(dz * inv, dx * inv, dy * inv, Yd);
@@ -226,19 +249,22 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
             }
             // the lanes of a row iterate together so that the cross-lane sums below see all CL partners
             const int iters = (e1 - e0 + EPR - 1) / EPR;
+            EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0, 0};
+            {
+                const int ef = e0 + e_sub;
+                if (ef < e1) nx = load_edge(a, ef);
+            }
             for (int it = 0; it < iters; ++it) {
                 const int e = e0 + it * EPR + e_sub;
                 bool on = e < e1;
-                int tj = 0;
-                if (on) {
-                    tj = a.neigh_types[e];
-                    if (p.U > 1 && a.pair_table[pair_index_s(a.T, ti, tj)] != u) on = false;
-                }
+                const EdgeGeo cu = nx;
+                if (e + EPR < e1) nx = load_edge(a, e + EPR);
+                if (on && p.U > 1 && a.pair_table[pair_index_s(a.T, ti, cu.tj)] != u) on = false;
                 double fx = 0.0, fy = 0.0, fz = 0.0;
                 if (on) {
-                    const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
-                    const double r = a.r[e];
-                    const int g = a.gather[e];
+                    const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
+                    const double r = cu.r;
+                    const int g = cu.g;
                     const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
                     const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
                     double Yd[16], gd[3][16];

@@ -141,7 +141,7 @@ struct EngineBase {
 template <typename F>
 struct Engine : EngineBase {
     // ---- model on device
-    DVec<F> tab0, tab1, H0, A0w, H1w, A1w;
+    DVec<F> tab0, tab1, tabK0, tabK1, H0, A0w, H1w, A1w;
     DVec<int> pair_table0, pair_table1;
     DVec<int> B0_start, B0_lm1, B1_start, B1_lm1;
     DVec<double> B0_c, B1_c;
@@ -206,6 +206,20 @@ struct Engine : EngineBase {
             upload_as(A1w, all, s);
         }
         build_slices(s);
+        // the general edge kernels read the tables channel-major; layers served by the slice kernels need no copy
+        auto kmajor = [&](const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst) {
+            const int R = hm.spl_nodes - 1, Kc = hm.K, Pn = nspl / Kc;
+            std::vector<double> out((size_t)tables.size() * R * nspl * 4);
+            size_t o = 0;
+            for (auto& t : tables)
+                for (int n = 0; n < R; ++n)
+                    for (int k = 0; k < Kc; ++k)
+                        for (int pth = 0; pth < Pn; ++pth)
+                            for (int q = 0; q < 4; ++q) out[o++] = t[((size_t)n * 4 + q) * nspl + pth * Kc + k];
+            upload_as(dst, out, s);
+        };
+        if (!slice_CH0) kmajor(hm.tables0, hm.nspl0, tabK0);
+        if (!slice_CH1) kmajor(hm.tables1, hm.nspl1, tabK1);
         // layer 0 couples Y_lm straight into output slot lm
         {
             std::vector<int> st(17), lm(16);
@@ -427,12 +441,13 @@ struct Engine : EngineBase {
         p.num_nodes = N; p.K = hm.K;
         p.first_neigh = first_neigh.p; p.node_types = node_types; p.neigh_types = neigh_types;
         p.xyz = xyz; p.r = r; p.T = hm.T; p.spl_nodes = hm.spl_nodes; p.spl_h = hm.spl_h;
+        p.num_edges = E;
         if (layer == 0) {
-            p.gather = neigh_types; p.Hsrc = H0.p; p.tab = tab0.p; p.pair_table = pair_table0.p;
-            p.B_start = B0_start.p; p.B_lm1 = B0_lm1.p; p.B_c = B0_c.p;
+            p.gather = neigh_types; p.Hsrc = H0.p; p.tab = tab0.p; p.tabK = tabK0.p; p.pair_table = pair_table0.p;
+            p.B_start = B0_start.p; p.B_lm1 = B0_lm1.p; p.B_c = B0_c.p; p.num_terms = (int)B0_c.n;
         } else {
-            p.gather = neigh_indices; p.Hsrc = H1.p; p.tab = tab1.p; p.pair_table = pair_table1.p;
-            p.B_start = B1_start.p; p.B_lm1 = B1_lm1.p; p.B_c = B1_c.p;
+            p.gather = neigh_indices; p.Hsrc = H1.p; p.tab = tab1.p; p.tabK = tabK1.p; p.pair_table = pair_table1.p;
+            p.B_start = B1_start.p; p.B_lm1 = B1_lm1.p; p.B_c = B1_c.p; p.num_terms = (int)B1_c.n;
         }
         return p;
     }
@@ -618,7 +633,7 @@ struct Engine : EngineBase {
         } else {
             auto p = agg_params(1, N);
             p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
-            HIPCHK(launch_agg_bwd<F>(hm.L_max, p, stream));
+            agg_bwd_general(hm.L_max, p);
         }
         stage_end(ST_AGG1B);
         // edges beyond the first N receivers carry no layer-1 adjoint
@@ -646,7 +661,18 @@ struct Engine : EngineBase {
         }
         auto p = agg_params(0, N);
         p.d_out = Phi0.p; p.forces = node_forces.p; p.accumulate_forces = 1; p.msg = nullptr;
-        HIPCHK(launch_agg_bwd<F>(0, p, stream));
+        agg_bwd_general(0, p);
+    }
+    // general adjoint kernel; wide models are cut into channel groups whose partial forces are added in order
+    void agg_bwd_general(int L_max_H, AggParams<F>& p)
+    {
+        const int groups = agg_bwd_groups<F>(L_max_H, K());
+        if (groups > 1) {
+            fpart.size_to((size_t)groups * 3 * E, stream);
+            p.fpart = fpart.p;
+        }
+        HIPCHK(launch_agg_bwd<F>(L_max_H, p, stream));
+        if (groups > 1) HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, p.accumulate_forces, stream));
     }
 
     // ------------------------------------------------------------------

@@ -28,6 +28,7 @@ struct AggParams {
     const double* r;          // [E]
     const F* Hsrc;            // [rows][NLM][K]
     const F* tab;             // [table][nodes-1][4][P*K]
+    const F* tabK;            // the same numbers channel-major, [table][nodes-1][K][P][4] (general edge kernels)
     const int* pair_table;    // [T(T+1)/2] -> table
     int T;
     int spl_nodes;
@@ -40,10 +41,16 @@ struct AggParams {
     double* forces;           // bwd: [E][3]
     int accumulate_forces;    // bwd: add to forces instead of overwriting
     F* msg;                   // bwd: [E][NLM][K] adjoint message to the sender row, or null
+    double* fpart;            // bwd: [channel groups][E][3] partial forces, needed when agg_bwd_groups() > 1
+    long num_edges;
+    int num_terms;            // entries of B_lm1 / B_c
 };
 
 template <typename F> hipError_t launch_agg_fwd(int L_max_H, const AggParams<F>& p, hipStream_t s);
 template <typename F> hipError_t launch_agg_bwd(int L_max_H, const AggParams<F>& p, hipStream_t s);
+// number of channel groups launch_agg_bwd splits K into; with more than one, the forces come out as
+// fpart[group][E][3] and launch_fpart_reduce adds them up
+template <typename F> int agg_bwd_groups(int L_max_H, int K);
 
 // Channel-slice variant of the same two stages for scalar hidden features
 // (L_max = 0 path structure: output slot lm is fed by path l(lm) and harmonic lm

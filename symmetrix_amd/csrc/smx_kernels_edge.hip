@@ -1,143 +1,79 @@
-// Edge kernels for gfx950: fused harmonics + radial splines + receiver-segmented
-// aggregation, and the analytic edge-force adjoint.
+// Edge kernels for gfx950, general form: fused harmonics + radial splines +
+// receiver-segmented aggregation, and the analytic edge-force adjoint, for any
+// path list (scalar or l <= 1 hidden features) and any number of radial tables.
 //
-// Work decomposition.  The edge list is receiver-sorted (CSR).  A "team" of LPR
-// lanes (half a wavefront or a whole one) owns one receiver; lane j of the team
-// owns channels j, j+LPR, ... (CPL of them), so every table or feature load of a
-// team is one contiguous run of LPR elements.  Accumulators (NE per channel)
-// live in registers for the whole neighbour loop, so sums run in edge order with
-// no atomics and are bit-reproducible.  Per chunk of EC edges the first EC lanes
-// of the team evaluate the per-edge quantities that do not depend on the channel
-// (direction, harmonics, Clebsch-Gordan-contracted harmonics B, spline interval)
-// into LDS, from where the channel loop reads them as broadcasts.
+// Work decomposition.  The edge list is receiver-sorted (CSR).  One wavefront
+// owns one receiver; lane j owns CPL consecutive channels, so every table or
+// feature load of the wavefront is one contiguous run.  Accumulators (NE per
+// channel) live in registers for the whole neighbour loop, so sums run in edge
+// order with no atomics and are bit-reproducible.  Edges are taken in chunks of
+// EC.  Per chunk, the first EC lanes evaluate direction, harmonics and spline
+// interval of one edge each; then all 64 lanes share the EC x NB entries of the
+// Clebsch-Gordan-contracted harmonics B (and their gradients in the adjoint);
+// both go through LDS, from where the channel loop reads them as broadcasts.
+// The four wavefronts of a block share nothing but the coupling list, so the
+// only block-wide barrier is the one after that list is copied to LDS.
+#include "smx_device.hpp"
 #include "smx_kernels.hpp"
 #include "smx_paths.hpp"
-
-#include <type_traits>
 
 namespace smx {
 
 namespace {
 
-// compile-time loop: f(std::integral_constant<int, I>) for I in [I0, N)
-template <int I0, int N, typename Fn>
-__device__ __forceinline__ void static_for(Fn&& f)
-{
-    if constexpr (I0 < N) {
-        f(std::integral_constant<int, I0>{});
-        static_for<I0 + 1, N>(f);
-    }
-}
-
-// Real harmonics l<=3 in the engine convention (mace.cpp:118-148): orthonormal
-// real harmonics of the direction, evaluated at the permuted vector
-// (x',y',z') = (z,x,y) and multiplied by 2 sqrt(pi).  Arguments are the
-// permuted unit vector.  Y[16].
-__device__ __forceinline__ void sph_l3(double x, double y, double z, double* Y)
-{
-    const double s3 = 1.7320508075688772, s15 = 3.872983346207417, s5h = 1.118033988749895;
-    const double s15h = 1.9364916731037085, c3a = 2.091650066335189, s105 = 10.246950765959598;
-    const double c3c = 1.620185174601965, c3d = 1.3228756555322954, c3e = 5.123475382979799;
-    const double xx = x * x, yy = y * y, zz = z * z;
-    Y[0] = 1.0;
-    Y[1] = s3 * y; Y[2] = s3 * z; Y[3] = s3 * x;
-    Y[4] = s15 * x * y; Y[5] = s15 * y * z; Y[6] = s5h * (2 * zz - xx - yy);
-    Y[7] = s15 * x * z; Y[8] = s15h * (xx - yy);
-    Y[9] = c3a * y * (3 * xx - yy); Y[10] = s105 * x * y * z;
-    Y[11] = c3c * y * (4 * zz - xx - yy); Y[12] = c3d * z * (2 * zz - 3 * xx - 3 * yy);
-    Y[13] = c3c * x * (4 * zz - xx - yy); Y[14] = c3e * (xx - yy) * z; Y[15] = c3a * x * (xx - 3 * yy);
-}
-
-// Harmonics and their gradient with respect to the (unpermuted) edge vector.
-// (x,y,z) is the permuted unit vector, inv_r = 1/|v|.  G[a][lm] with a = 0,1,2
-// the derivative along the original x, y, z axes.
-__device__ __forceinline__ void sph_l3_grad(double x, double y, double z, double inv_r, double* Y, double (*G)[16])
-{
-    const double s3 = 1.7320508075688772, s15 = 3.872983346207417, s5h = 1.118033988749895;
-    const double s15h = 1.9364916731037085, c3a = 2.091650066335189, s105 = 10.246950765959598;
-    const double c3c = 1.620185174601965, c3d = 1.3228756555322954, c3e = 5.123475382979799;
-    const double xx = x * x, yy = y * y, zz = z * z;
-    double g[3][16];  // derivative of the homogeneous forms along x', y', z'
-    Y[0] = 1.0;                              g[0][0] = 0;               g[1][0] = 0;                g[2][0] = 0;
-    Y[1] = s3 * y;                           g[0][1] = 0;               g[1][1] = s3;               g[2][1] = 0;
-    Y[2] = s3 * z;                           g[0][2] = 0;               g[1][2] = 0;                g[2][2] = s3;
-    Y[3] = s3 * x;                           g[0][3] = s3;              g[1][3] = 0;                g[2][3] = 0;
-    Y[4] = s15 * x * y;                      g[0][4] = s15 * y;         g[1][4] = s15 * x;          g[2][4] = 0;
-    Y[5] = s15 * y * z;                      g[0][5] = 0;               g[1][5] = s15 * z;          g[2][5] = s15 * y;
-    Y[6] = s5h * (2 * zz - xx - yy);         g[0][6] = -2 * s5h * x;    g[1][6] = -2 * s5h * y;     g[2][6] = 4 * s5h * z;
-    Y[7] = s15 * x * z;                      g[0][7] = s15 * z;         g[1][7] = 0;                g[2][7] = s15 * x;
-    Y[8] = s15h * (xx - yy);                 g[0][8] = 2 * s15h * x;    g[1][8] = -2 * s15h * y;    g[2][8] = 0;
-    Y[9] = c3a * y * (3 * xx - yy);          g[0][9] = 6 * c3a * x * y; g[1][9] = 3 * c3a * (xx - yy); g[2][9] = 0;
-    Y[10] = s105 * x * y * z;                g[0][10] = s105 * y * z;   g[1][10] = s105 * x * z;    g[2][10] = s105 * x * y;
-    Y[11] = c3c * y * (4 * zz - xx - yy);    g[0][11] = -2 * c3c * x * y; g[1][11] = c3c * (4 * zz - xx - 3 * yy); g[2][11] = 8 * c3c * y * z;
-    Y[12] = c3d * z * (2 * zz - 3 * xx - 3 * yy); g[0][12] = -6 * c3d * x * z; g[1][12] = -6 * c3d * y * z; g[2][12] = 3 * c3d * (2 * zz - xx - yy);
-    Y[13] = c3c * x * (4 * zz - xx - yy);    g[0][13] = c3c * (4 * zz - 3 * xx - yy); g[1][13] = -2 * c3c * x * y; g[2][13] = 8 * c3c * x * z;
-    Y[14] = c3e * (xx - yy) * z;             g[0][14] = 2 * c3e * x * z; g[1][14] = -2 * c3e * y * z; g[2][14] = c3e * (xx - yy);
-    Y[15] = c3a * x * (xx - 3 * yy);         g[0][15] = 3 * c3a * (xx - yy); g[1][15] = -6 * c3a * x * y; g[2][15] = 0;
-    // chain rule through u = v/|v| (u.grad_u of a degree-l form is l times the form), then
-    // undo the permutation: original x is x' index 1, y is index 2, z is index 0
-    const double u[3] = {x, y, z};
-#pragma unroll
-    for (int lm = 0; lm < 16; ++lm) {
-        const int l = lm < 1 ? 0 : (lm < 4 ? 1 : (lm < 9 ? 2 : 3));
-        const double ly = l * Y[lm];
-        G[0][lm] = (g[1][lm] - u[1] * ly) * inv_r;
-        G[1][lm] = (g[2][lm] - u[2] * ly) * inv_r;
-        G[2][lm] = (g[0][lm] - u[0] * ly) * inv_r;
-    }
-}
-
-__device__ __forceinline__ int pair_index(int T, int a, int b)
-{
-    return (a <= b) ? a * (2 * T - a - 1) / 2 + b : b * (2 * T - b - 1) / 2 + a;
-}
-
-// sum over the LPR lanes of a team; every lane of the team gets the result
-template <int LPR>
-__device__ __forceinline__ double team_sum(double v)
-{
-#pragma unroll
-    for (int off = LPR / 2; off >= 1; off >>= 1) v += __shfl_xor(v, off, 64);
-    return v;
-}
-
-template <typename F, int NB, bool BWD>
-struct TeamLds {
-    static constexpr int NY = BWD ? 64 : 16;
-    static constexpr int NBT = BWD ? 4 * NB : NB;
-    __host__ __device__ static constexpr size_t bytes(int EC)
+template <typename F, int LMAXH, bool BWD>
+struct WaveLds {
+    using PT = Paths<LMAXH>;
+    static constexpr int NBP = (PT::NB + 3) / 4 * 4;          // B row padded for 16-byte reads
+    static constexpr int NY = BWD ? 64 : 16;                  // Y (and dY/dx, dY/dy, dY/dz)
+    static constexpr int NBT = BWD ? 4 * NBP : NBP;
+    __host__ __device__ static constexpr size_t per_wave(int EC)
     {
-        return (size_t)EC * (NY * sizeof(double) + NBT * sizeof(F) + sizeof(F) + (BWD ? 3 * sizeof(double) : 0) + 2 * sizeof(int)) + 16;
+        size_t b = (size_t)EC * (NY * sizeof(double) + (BWD ? 4 * sizeof(double) : 0) + NBT * sizeof(F));
+        b += (size_t)EC * (sizeof(double) + 2 * sizeof(int));   // x (held as double-sized slot), rows, gather rows
+        return (b + 15) / 16 * 16;
+    }
+    __host__ __device__ static constexpr size_t lists(int num_terms)
+    {
+        return ((size_t)num_terms * (sizeof(double) + sizeof(int)) + (PT::NB + 1) * sizeof(int) + 15) / 16 * 16;
     }
 };
 
+template <typename F, int CPL>
+__device__ __forceinline__ Vec<F, CPL> ldv(const F* p)
+{
+    return *reinterpret_cast<const Vec<F, CPL>*>(p);
+}
+
 // ---------------------------------------------------------------------------
-template <typename F, int LMAXH, int LPR, int CPL, int EC>
-__global__ __launch_bounds__(256) void k_agg_fwd(const AggParams<F> a)
+template <typename F, int LMAXH, int CPL, int EC>
+__global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const int num_terms)
 {
     using PT = Paths<LMAXH>;
-    constexpr int RPB = 256 / LPR, NB = PT::NB, NE = PT::NE, P = PT::P, NLM = PT::NLM;
+    using WL = WaveLds<F, LMAXH, false>;
+    constexpr int NB = PT::NB, NBP = WL::NBP, NE = PT::NE, P = PT::P, NLM = PT::NLM;
     extern __shared__ __align__(16) unsigned char smem[];
-    const int team = threadIdx.x / LPR, lane = threadIdx.x % LPR;
-    unsigned char* base = smem + (size_t)team * ((TeamLds<F, NB, false>::bytes(EC) + 15) / 16 * 16);
-    double* Yt = reinterpret_cast<double*>(base);                 // [EC][16]
-    F* Bs = reinterpret_cast<F*>(Yt + EC * 16);                   // [EC][NB]
-    F* xs = Bs + EC * NB;                                         // [EC]
-    int* rows = reinterpret_cast<int*>(xs + EC + (EC & 1));       // [EC]
-    int* grows = rows + EC;                                       // [EC]
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    double* cg_c = reinterpret_cast<double*>(smem);                               // [num_terms]
+    int* cg_lm1 = reinterpret_cast<int*>(cg_c + num_terms);                       // [num_terms]
+    int* cg_start = cg_lm1 + num_terms;                                           // [NB+1]
+    unsigned char* base = smem + WL::lists(num_terms) + (size_t)wave * WL::per_wave(EC);
+    double* Yt = reinterpret_cast<double*>(base);                                 // [EC][16]
+    double* xs = Yt + EC * 16;                                                    // [EC]
+    F* Bs = reinterpret_cast<F*>(xs + EC);                                        // [EC][NBP]
+    int* rows = reinterpret_cast<int*>(Bs + EC * NBP);                            // [EC]
+    int* grows = rows + EC;                                                       // [EC]
 
-    const int K = a.K, NSPL = P * K;
-    const int i = blockIdx.x * RPB + team;
-    const int kbase = blockIdx.y * (LPR * CPL);
-    int e0 = 0, e1 = 0, ti = 0;
-    if (i < a.num_nodes) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
-    int maxdeg = 0;
-#pragma unroll
-    for (int t = 0; t < RPB; ++t) {
-        const int ii = blockIdx.x * RPB + t;
-        if (ii < a.num_nodes) maxdeg = max(maxdeg, a.first_neigh[ii + 1] - a.first_neigh[ii]);
-    }
-    const int nchunks = (maxdeg + EC - 1) / EC;
+    for (int t = threadIdx.x; t < num_terms; t += 256) { cg_c[t] = a.B_c[t]; cg_lm1[t] = a.B_lm1[t]; }
+    for (int t = threadIdx.x; t <= NB; t += 256) cg_start[t] = a.B_start[t];
+    __syncthreads();
+
+    const int K = a.K;
+    const int i = blockIdx.x * 4 + wave;
+    if (i >= a.num_nodes) return;
+    const int k0 = (blockIdx.y * 64 + lane) * CPL;
+    const bool active = k0 < K;
+    const int e0 = a.first_neigh[i], e1 = a.first_neigh[i + 1], ti = a.node_types[i];
 
     F acc[CPL][NE];
 #pragma unroll
@@ -145,10 +81,10 @@ __global__ __launch_bounds__(256) void k_agg_fwd(const AggParams<F> a)
 #pragma unroll
         for (int q = 0; q < NE; ++q) acc[c][q] = F(0);
 
-    for (int ch = 0; ch < nchunks; ++ch) {
-        __syncthreads();
-        const int eb = e0 + ch * EC;
-        if (lane < EC && eb + lane < e1) {
+    for (int eb = e0; eb < e1; eb += EC) {
+        const int nE = min(EC, e1 - eb);
+        wave_lds_sync();
+        if (lane < nE) {
             const int e = eb + lane;
             const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
             const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
@@ -156,61 +92,67 @@ __global__ __launch_bounds__(256) void k_agg_fwd(const AggParams<F> a)
             sph_l3(dz * inv, dx * inv, dy * inv, Y);
 #pragma unroll
             for (int q = 0; q < 16; ++q) Yt[lane * 16 + q] = Y[q];
-            for (int b = 0; b < NB; ++b) {
-                double s = 0.0;
-                for (int t = a.B_start[b]; t < a.B_start[b + 1]; ++t) s += a.B_c[t] * Yt[lane * 16 + a.B_lm1[t]];
-                Bs[lane * NB + b] = (F)s;
-            }
             const double r = a.r[e];
             int n = (int)(r / a.spl_h);
             n = min(max(n, 0), a.spl_nodes - 2);
-            xs[lane] = (F)(r - a.spl_h * n);
+            xs[lane] = r - a.spl_h * n;
             const int tbl = a.pair_table[pair_index(a.T, ti, a.neigh_types[e])];
             rows[lane] = tbl * (a.spl_nodes - 1) + n;
             grows[lane] = a.gather[e];
         }
-        __syncthreads();
-        const int nE = min(EC, e1 - eb);
+        wave_lds_sync();
+        for (int it = lane; it < nE * NB; it += 64) {
+            const int le = it / NB, b = it - le * NB;
+            double s = 0.0;
+            for (int t = cg_start[b]; t < cg_start[b + 1]; ++t) s += cg_c[t] * Yt[le * 16 + cg_lm1[t]];
+            Bs[le * NBP + b] = (F)s;
+        }
+        wave_lds_sync();
+        if (!active) continue;
         for (int le = 0; le < nE; ++le) {
-            const F x = xs[le];
-            const F* row = a.tab + (size_t)rows[le] * 4 * NSPL;
-            const F* Hrow = a.Hsrc + (size_t)grows[le] * NLM * K;
-            const F* B = Bs + le * NB;
+            const F x = (F)xs[le];
+            const int row = __builtin_amdgcn_readfirstlane(rows[le]);
+            const int grow = __builtin_amdgcn_readfirstlane(grows[le]);
+            const F* rowp = a.tabK + ((size_t)row * K + k0) * (4 * P);
+            const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
+            const F* B = Bs + le * NBP;
+            Vec<F, CPL> H[NLM];
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) {
-                const int k = kbase + lane + c * LPR;
-                if (k < K) {
-                    F H[NLM];
+            for (int q = 0; q < NLM; ++q) H[q] = ldv<F, CPL>(Hp + q * K);
+            static_for<0, P>([&](auto pc) {
+                constexpr int p = decltype(pc)::value;
+                constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
+                constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1;
+                Vec<F, 4> cf[CPL];
 #pragma unroll
-                    for (int q = 0; q < NLM; ++q) H[q] = Hrow[q * K + k];
-                    static_for<0, P>([&](auto pc) {
-                        constexpr int p = decltype(pc)::value;
-                        constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
-                        constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l);
-                        const F c0 = row[p * K + k], c1 = row[NSPL + p * K + k];
-                        const F c2 = row[2 * NSPL + p * K + k], c3 = row[3 * NSPL + p * K + k];
-                        const F R = c0 + x * (c1 + x * (c2 + x * c3));
+                for (int c = 0; c < CPL; ++c) cf[c] = ldv<F, 4>(rowp + (c * P + p) * 4);
+                F Bv[(2 * l + 1) * n2];
 #pragma unroll
-                        for (int m = 0; m < 2 * l + 1; ++m) {
-                            F z = F(0);
+                for (int q = 0; q < (2 * l + 1) * n2; ++q) Bv[q] = B[bo + q];
 #pragma unroll
-                            for (int m2 = 0; m2 < 2 * l2 + 1; ++m2)
-                                z += B[bo + m * (2 * l2 + 1) + m2] * H[l2 * l2 + m2];
-                            acc[c][lme0 + m * es] += R * z;
-                        }
-                    });
+                for (int c = 0; c < CPL; ++c) {
+                    const F R = cf[c].v[0] + x * (cf[c].v[1] + x * (cf[c].v[2] + x * cf[c].v[3]));
+                    F w[n2];
+#pragma unroll
+                    for (int m2 = 0; m2 < n2; ++m2) w[m2] = R * H[l2 * l2 + m2].v[c];
+#pragma unroll
+                    for (int m = 0; m < 2 * l + 1; ++m) {
+                        F z = acc[c][lme0 + m * es];
+#pragma unroll
+                        for (int m2 = 0; m2 < n2; ++m2) z += Bv[m * n2 + m2] * w[m2];
+                        acc[c][lme0 + m * es] = z;
+                    }
                 }
-            }
+            });
         }
     }
-    if (i < a.num_nodes) {
+    if (active) {
 #pragma unroll
-        for (int c = 0; c < CPL; ++c) {
-            const int k = kbase + lane + c * LPR;
-            if (k < K) {
+        for (int q = 0; q < NE; ++q) {
+            Vec<F, CPL> o;
 #pragma unroll
-                for (int q = 0; q < NE; ++q) a.out[((size_t)i * NE + q) * K + k] = acc[c][q];
-            }
+            for (int c = 0; c < CPL; ++c) o.v[c] = acc[c][q];
+            *reinterpret_cast<Vec<F, CPL>*>(a.out + ((size_t)i * NE + q) * K + k0) = o;
         }
     }
 }
@@ -219,189 +161,210 @@ __global__ __launch_bounds__(256) void k_agg_fwd(const AggParams<F> a)
 // Adjoint: per edge force -dE/dxyz_ij (MACE::reverse_A0, mace.cpp:238-269;
 // MACE::reverse_Phi1, mace.cpp:531-574) and the adjoint message to the sender
 // row (mace.cpp:579-604), staged per edge for the deterministic sender-side sum.
-template <typename F, int LMAXH, int LPR, int CPL, int EC>
-__global__ __launch_bounds__(256) void k_agg_bwd(const AggParams<F> a)
+// With more than one channel group (gridDim.y > 1) each group writes its share
+// of the force to fpart[group][edge][3]; the caller adds the groups up.
+#ifndef EXP_WPE
+#define EXP_WPE 2
+#endif
+template <typename F, int LMAXH, int CPL, int EC>
+__global__ __launch_bounds__(256, EXP_WPE) void k_agg_bwd(const AggParams<F> a, const int num_terms)
 {
     using PT = Paths<LMAXH>;
-    constexpr int RPB = 256 / LPR, NB = PT::NB, NE = PT::NE, P = PT::P, NLM = PT::NLM;
+    using WL = WaveLds<F, LMAXH, true>;
+    constexpr int NB = PT::NB, NBP = WL::NBP, NE = PT::NE, P = PT::P, NLM = PT::NLM;
     extern __shared__ __align__(16) unsigned char smem[];
-    const int team = threadIdx.x / LPR, lane = threadIdx.x % LPR;
-    unsigned char* base = smem + (size_t)team * ((TeamLds<F, NB, true>::bytes(EC) + 15) / 16 * 16);
-    double* Yt = reinterpret_cast<double*>(base);                 // [EC][4][16]: Y, dY/dx, dY/dy, dY/dz
-    double* us = Yt + EC * 64;                                    // [EC][3] unit vector xyz/r
-    F* Bs = reinterpret_cast<F*>(us + EC * 3);                    // [EC][4][NB]
-    F* xs = Bs + EC * 4 * NB;                                     // [EC]
-    int* rows = reinterpret_cast<int*>(xs + EC + (EC & 1));
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    double* cg_c = reinterpret_cast<double*>(smem);
+    int* cg_lm1 = reinterpret_cast<int*>(cg_c + num_terms);
+    int* cg_start = cg_lm1 + num_terms;
+    unsigned char* base = smem + WL::lists(num_terms) + (size_t)wave * WL::per_wave(EC);
+    double* Yt = reinterpret_cast<double*>(base);                                 // [EC][4][16]: Y, dY/dx, dY/dy, dY/dz
+    double* us = Yt + EC * 64;                                                    // [EC][4] unit vector xyz/r
+    double* xs = us + EC * 4;                                                     // [EC]
+    F* Bs = reinterpret_cast<F*>(xs + EC);                                        // [EC][4][NBP]
+    int* rows = reinterpret_cast<int*>(Bs + EC * 4 * NBP);
     int* grows = rows + EC;
 
-    const int K = a.K, NSPL = P * K;
-    const int i = blockIdx.x * RPB + team;
-    const int kbase = blockIdx.y * (LPR * CPL);
-    int e0 = 0, e1 = 0, ti = 0;
-    if (i < a.num_nodes) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
-    int maxdeg = 0;
-#pragma unroll
-    for (int t = 0; t < RPB; ++t) {
-        const int ii = blockIdx.x * RPB + t;
-        if (ii < a.num_nodes) maxdeg = max(maxdeg, a.first_neigh[ii + 1] - a.first_neigh[ii]);
-    }
-    const int nchunks = (maxdeg + EC - 1) / EC;
+    for (int t = threadIdx.x; t < num_terms; t += 256) { cg_c[t] = a.B_c[t]; cg_lm1[t] = a.B_lm1[t]; }
+    for (int t = threadIdx.x; t <= NB; t += 256) cg_start[t] = a.B_start[t];
+    __syncthreads();
+
+    const int K = a.K;
+    const int i = blockIdx.x * 4 + wave;
+    if (i >= a.num_nodes) return;
+    const int k0 = (blockIdx.y * 64 + lane) * CPL;
+    const bool active = k0 < K;
+    const int e0 = a.first_neigh[i], e1 = a.first_neigh[i + 1], ti = a.node_types[i];
+    double* fout = gridDim.y > 1 ? a.fpart + (size_t)blockIdx.y * 3 * a.num_edges : a.forces;
+    const bool add_forces = gridDim.y == 1 && a.accumulate_forces;
 
     F d[CPL][NE];
 #pragma unroll
-    for (int c = 0; c < CPL; ++c) {
-        const int k = kbase + lane + c * LPR;
+    for (int q = 0; q < NE; ++q) {
+        // lanes beyond K read channel 0 and discard it
+        const Vec<F, CPL> v = ldv<F, CPL>(a.d_out + ((size_t)i * NE + q) * K + (active ? k0 : 0));
 #pragma unroll
-        for (int q = 0; q < NE; ++q)
-            d[c][q] = (i < a.num_nodes && k < K) ? a.d_out[((size_t)i * NE + q) * K + k] : F(0);
+        for (int c = 0; c < CPL; ++c) d[c][q] = active ? v.v[c] : F(0);
     }
 
-    for (int ch = 0; ch < nchunks; ++ch) {
-        __syncthreads();
-        const int eb = e0 + ch * EC;
-        if (lane < EC && eb + lane < e1) {
+    for (int eb = e0; eb < e1; eb += EC) {
+        const int nE = min(EC, e1 - eb);
+        wave_lds_sync();
+        if (lane < nE) {
             const int e = eb + lane;
             const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
             const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
-            double Y[16], G[3][16];
-            sph_l3_grad(dz * inv, dx * inv, dy * inv, inv, Y, G);
-#pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                Yt[lane * 64 + q] = Y[q];
-                Yt[lane * 64 + 16 + q] = G[0][q];
-                Yt[lane * 64 + 32 + q] = G[1][q];
-                Yt[lane * 64 + 48 + q] = G[2][q];
-            }
-            for (int b = 0; b < NB; ++b) {
-                double s = 0.0, sx = 0.0, sy = 0.0, sz = 0.0;
-                for (int t = a.B_start[b]; t < a.B_start[b + 1]; ++t) {
-                    const double cc = a.B_c[t];
-                    const int lm1 = a.B_lm1[t];
-                    s += cc * Yt[lane * 64 + lm1];
-                    sx += cc * Yt[lane * 64 + 16 + lm1];
-                    sy += cc * Yt[lane * 64 + 32 + lm1];
-                    sz += cc * Yt[lane * 64 + 48 + lm1];
-                }
-                Bs[(lane * 4 + 0) * NB + b] = (F)s;
-                Bs[(lane * 4 + 1) * NB + b] = (F)sx;
-                Bs[(lane * 4 + 2) * NB + b] = (F)sy;
-                Bs[(lane * 4 + 3) * NB + b] = (F)sz;
-            }
+            sph_l3_grad_store<16>(dz * inv, dx * inv, dy * inv, inv, Yt + lane * 64);
             const double r = a.r[e];
             // radial direction as the reference forms it: xyz / r with the caller's r
-            us[lane * 3] = dx / r; us[lane * 3 + 1] = dy / r; us[lane * 3 + 2] = dz / r;
+            us[lane * 4] = dx / r; us[lane * 4 + 1] = dy / r; us[lane * 4 + 2] = dz / r;
             int n = (int)(r / a.spl_h);
             n = min(max(n, 0), a.spl_nodes - 2);
-            xs[lane] = (F)(r - a.spl_h * n);
+            xs[lane] = r - a.spl_h * n;
             const int tbl = a.pair_table[pair_index(a.T, ti, a.neigh_types[e])];
             rows[lane] = tbl * (a.spl_nodes - 1) + n;
             grows[lane] = a.gather[e];
         }
-        __syncthreads();
-        const int nE = min(EC, e1 - eb);
+        wave_lds_sync();
+        for (int it = lane; it < nE * NB; it += 64) {
+            const int le = it / NB, b = it - le * NB;
+            double s = 0.0, sx = 0.0, sy = 0.0, sz = 0.0;
+            for (int t = cg_start[b]; t < cg_start[b + 1]; ++t) {
+                const double cc = cg_c[t];
+                const double* y = Yt + le * 64 + cg_lm1[t];
+                s += cc * y[0]; sx += cc * y[16]; sy += cc * y[32]; sz += cc * y[48];
+            }
+            F* o = Bs + (size_t)le * 4 * NBP + b;
+            o[0] = (F)s; o[NBP] = (F)sx; o[2 * NBP] = (F)sy; o[3 * NBP] = (F)sz;
+        }
+        wave_lds_sync();
         for (int le = 0; le < nE; ++le) {
-            const F x = xs[le];
-            const F* row = a.tab + (size_t)rows[le] * 4 * NSPL;
-            const F* Hrow = a.Hsrc + (size_t)grows[le] * NLM * K;
-            const F* B = Bs + (le * 4) * NB;
-            const F* Bx = B + NB;
-            const F* By = B + 2 * NB;
-            const F* Bz = B + 3 * NB;
-            double srad = 0.0, gx = 0.0, gy = 0.0, gz = 0.0;
+            F srad = F(0), gx = F(0), gy = F(0), gz = F(0);
+            if (active) {
+                const F x = (F)xs[le];
+                const int row = __builtin_amdgcn_readfirstlane(rows[le]);
+                const int grow = __builtin_amdgcn_readfirstlane(grows[le]);
+                // element offsets of this edge's table row and of its B block; they pass through the
+                // fence at the end of every path, which keeps the loads of a path behind the arithmetic
+                // of the path before it (all loads at once would need several hundred registers)
+                size_t roff = ((size_t)row * K + k0) * (4 * P);
+                int boffs = le * 4 * NBP;
+                const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
+                Vec<F, CPL> H[NLM], mg[NLM];
 #pragma unroll
-            for (int c = 0; c < CPL; ++c) {
-                const int k = kbase + lane + c * LPR;
-                if (k < K) {
-                    F H[NLM], mg[NLM];
+                for (int q = 0; q < NLM; ++q) {
+                    H[q] = ldv<F, CPL>(Hp + q * K);
 #pragma unroll
-                    for (int q = 0; q < NLM; ++q) { H[q] = Hrow[q * K + k]; mg[q] = F(0); }
-                    F s_c = F(0), gx_c = F(0), gy_c = F(0), gz_c = F(0);
-                    static_for<0, P>([&](auto pc) {
-                        constexpr int p = decltype(pc)::value;
-                        constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
-                        constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l);
-                        const F c0 = row[p * K + k], c1 = row[NSPL + p * K + k];
-                        const F c2 = row[2 * NSPL + p * K + k], c3 = row[3 * NSPL + p * K + k];
-                        const F R = c0 + x * (c1 + x * (c2 + x * c3));
-                        const F Rd = c1 + x * (F(2) * c2 + F(3) * x * c3);
+                    for (int c = 0; c < CPL; ++c) mg[q].v[c] = F(0);
+                }
+                static_for<0, P>([&](auto pc) {
+                    constexpr int p = decltype(pc)::value;
+                    constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
+                    constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1, nb = (2 * l + 1) * n2;
+                    const F* rowp = a.tabK + roff;
+                    const F* B = Bs + boffs;
+                    Vec<F, 4> cf[CPL];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) cf[c] = ldv<F, 4>(rowp + (c * P + p) * 4);
+                    F Bv[nb], uu[nb];
+#pragma unroll
+                    for (int q = 0; q < nb; ++q) { Bv[q] = B[bo + q]; uu[q] = F(0); }
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) {
+                        const F R = cf[c].v[0] + x * (cf[c].v[1] + x * (cf[c].v[2] + x * cf[c].v[3]));
+                        const F Rd = cf[c].v[1] + x * (F(2) * cf[c].v[2] + F(3) * x * cf[c].v[3]);
 #pragma unroll
                         for (int m = 0; m < 2 * l + 1; ++m) {
                             const F dd = d[c][lme0 + m * es];
-                            const F t = dd * R;
-                            F z = F(0), zx = F(0), zy = F(0), zz = F(0);
+                            const F t = dd * R, td = dd * Rd;
+                            F z = F(0);
 #pragma unroll
-                            for (int m2 = 0; m2 < 2 * l2 + 1; ++m2) {
-                                const int b = bo + m * (2 * l2 + 1) + m2;
-                                const F h = H[l2 * l2 + m2];
-                                z += B[b] * h; zx += Bx[b] * h; zy += By[b] * h; zz += Bz[b] * h;
-                                mg[l2 * l2 + m2] += t * B[b];
+                            for (int m2 = 0; m2 < n2; ++m2) {
+                                const F h = H[l2 * l2 + m2].v[c];
+                                z += Bv[m * n2 + m2] * h;
+                                mg[l2 * l2 + m2].v[c] += t * Bv[m * n2 + m2];
+                                uu[m * n2 + m2] += t * h;
                             }
-                            s_c += dd * Rd * z;
-                            gx_c += t * zx; gy_c += t * zy; gz_c += t * zz;
+                            srad += td * z;
                         }
-                    });
-                    srad += (double)s_c; gx += (double)gx_c; gy += (double)gy_c; gz += (double)gz_c;
-                    if (a.msg) {
-                        F* mrow = a.msg + (size_t)(eb + le) * NLM * K;
-#pragma unroll
-                        for (int q = 0; q < NLM; ++q) mrow[q * K + k] = mg[q];
                     }
+                    // the channels of this lane share the gradient of B; one component at a time (fenced like the paths)
+                    asm volatile("" : "+v"(uu[0]), "+v"(srad), "+v"(boffs));
+                    {
+                        const F* Bg = Bs + boffs + NBP + bo;
+#pragma unroll
+                        for (int q = 0; q < nb; ++q) gx += uu[q] * Bg[q];
+                    }
+                    asm volatile("" : "+v"(gx), "+v"(boffs));
+                    {
+                        const F* Bg = Bs + boffs + 2 * NBP + bo;
+#pragma unroll
+                        for (int q = 0; q < nb; ++q) gy += uu[q] * Bg[q];
+                    }
+                    asm volatile("" : "+v"(gy), "+v"(boffs));
+                    {
+                        const F* Bg = Bs + boffs + 3 * NBP + bo;
+#pragma unroll
+                        for (int q = 0; q < nb; ++q) gz += uu[q] * Bg[q];
+                    }
+                    asm volatile("" : "+v"(gz), "+v"(roff), "+v"(boffs));
+                });
+                if (a.msg) {
+                    F* mrow = a.msg + (size_t)(eb + le) * NLM * K + k0;
+#pragma unroll
+                    for (int q = 0; q < NLM; ++q) *reinterpret_cast<Vec<F, CPL>*>(mrow + q * K) = mg[q];
                 }
             }
-            double fx = -(us[le * 3] * srad + gx);
-            double fy = -(us[le * 3 + 1] * srad + gy);
-            double fz = -(us[le * 3 + 2] * srad + gz);
-            fx = team_sum<LPR>(fx); fy = team_sum<LPR>(fy); fz = team_sum<LPR>(fz);
-            if (lane == 0 && gridDim.y == 1) {
-                double* f = a.forces + 3 * (size_t)(eb + le);
-                if (a.accumulate_forces) { f[0] += fx; f[1] += fy; f[2] += fz; }
+            const double sr = (double)srad;
+            const double fx = wave_sum(-(us[le * 4] * sr + (double)gx));
+            const double fy = wave_sum(-(us[le * 4 + 1] * sr + (double)gy));
+            const double fz = wave_sum(-(us[le * 4 + 2] * sr + (double)gz));
+            if (lane == 0) {
+                double* f = fout + 3 * (size_t)(eb + le);
+                if (add_forces) { f[0] += fx; f[1] += fy; f[2] += fz; }
                 else { f[0] = fx; f[1] = fy; f[2] = fz; }
             }
         }
     }
 }
 
-template <typename F, int LMAXH, int LPR, int CPL, int EC, bool BWD>
+template <typename F, int LMAXH, int CPL, int EC, bool BWD>
 hipError_t launch_agg_t(const AggParams<F>& p, hipStream_t s)
 {
-    using PT = Paths<LMAXH>;
-    constexpr int RPB = 256 / LPR;
-    const size_t per_team = (TeamLds<F, PT::NB, BWD>::bytes(EC) + 15) / 16 * 16;
-    const size_t lds = per_team * RPB;
-    dim3 grid((p.num_nodes + RPB - 1) / RPB, (p.K + LPR * CPL - 1) / (LPR * CPL));
+    using WL = WaveLds<F, LMAXH, BWD>;
+    const int groups = (p.K + 64 * CPL - 1) / (64 * CPL);
+    if (p.K % CPL != 0) return hipErrorInvalidValue;
+    if (BWD && groups > 1 && !p.fpart) return hipErrorInvalidValue;
+    const size_t lds = WL::lists(p.num_terms) + 4 * WL::per_wave(EC);
+    dim3 grid((p.num_nodes + 3) / 4, groups);
     if (grid.x == 0) return hipSuccess;
-    if (BWD && grid.y != 1) return hipErrorInvalidValue;
-    void (*kern)(const AggParams<F>);
-    if constexpr (BWD) kern = k_agg_bwd<F, LMAXH, LPR, CPL, EC>;
-    else kern = k_agg_fwd<F, LMAXH, LPR, CPL, EC>;
+    void (*kern)(const AggParams<F>, const int);
+    if constexpr (BWD) kern = k_agg_bwd<F, LMAXH, CPL, EC>;
+    else kern = k_agg_fwd<F, LMAXH, CPL, EC>;
     if (lds > 64 * 1024) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, p);
+    hipLaunchKernelGGL(kern, grid, dim3(256), lds, s, p, p.num_terms);
     return hipGetLastError();
+}
+
+// channels per lane: two where the channel count allows paired loads and the registers hold the accumulators
+template <typename F, int LMAXH, bool BWD>
+constexpr int agg_cpl_wide()
+{
+    if (LMAXH == 0) return 2;
+    return BWD ? 1 : 2;   // the adjoint of the l <= 1 paths holds 40 adjoint values per channel
 }
 
 template <typename F, int LMAXH, bool BWD>
 hipError_t launch_agg_sel(const AggParams<F>& p, hipStream_t s)
 {
-    const int K = p.K;
-    if (LMAXH == 0) {
-        constexpr int EC = BWD ? 8 : 16;
-        if (K <= 32) return launch_agg_t<F, LMAXH, 32, 1, EC, BWD>(p, s);
-        if (K <= 64) return launch_agg_t<F, LMAXH, 32, 2, EC, BWD>(p, s);
-        if (K <= 96) return launch_agg_t<F, LMAXH, 32, 3, EC, BWD>(p, s);
-        if (K <= 128) return launch_agg_t<F, LMAXH, 32, 4, EC, BWD>(p, s);
-        if (K <= 256) return launch_agg_t<F, LMAXH, 64, 4, EC, BWD>(p, s);
-        return hipErrorInvalidValue;
-    } else {
-        constexpr int EC = BWD ? 4 : 8;
-        if (K <= 32) return launch_agg_t<F, LMAXH, 32, 1, EC, BWD>(p, s);
-        if (K <= 64) return launch_agg_t<F, LMAXH, 32, 2, EC, BWD>(p, s);
-        if (K <= 128) return launch_agg_t<F, LMAXH, 64, 2, EC, BWD>(p, s);
-        return hipErrorInvalidValue;
-    }
+    constexpr int EC = LMAXH == 0 ? 16 : (BWD ? (sizeof(F) == 4 ? 8 : 4) : 16);
+    constexpr int CW = agg_cpl_wide<F, LMAXH, BWD>();
+    if (CW == 2 && p.K > 64 && p.K % 2 == 0) return launch_agg_t<F, LMAXH, CW, EC, BWD>(p, s);
+    return launch_agg_t<F, LMAXH, 1, EC, BWD>(p, s);
 }
 
 }  // namespace
@@ -420,6 +383,14 @@ hipError_t launch_agg_bwd(int L_max_H, const AggParams<F>& p, hipStream_t s)
     if (L_max_H == 1) return launch_agg_sel<F, 1, true>(p, s);
     return hipErrorInvalidValue;
 }
+template <typename F>
+int agg_bwd_groups(int L_max_H, int K)
+{
+    int cpl = 1;
+    if (K > 64 && K % 2 == 0)
+        cpl = L_max_H == 0 ? agg_cpl_wide<F, 0, true>() : agg_cpl_wide<F, 1, true>();
+    return (K + 64 * cpl - 1) / (64 * cpl);
+}
 // This file is compiled four times (SMX_EDGE_PART = 0..3), one object per
 // precision and direction, so that the instantiations build in parallel.
 #ifndef SMX_EDGE_PART
@@ -431,8 +402,10 @@ template hipError_t launch_agg_fwd<double>(int, const AggParams<double>&, hipStr
 template hipError_t launch_agg_fwd<float>(int, const AggParams<float>&, hipStream_t);
 #elif SMX_EDGE_PART == 2
 template hipError_t launch_agg_bwd<double>(int, const AggParams<double>&, hipStream_t);
+template int agg_bwd_groups<double>(int, int);
 #else
 template hipError_t launch_agg_bwd<float>(int, const AggParams<float>&, hipStream_t);
+template int agg_bwd_groups<float>(int, int);
 #endif
 
 #if SMX_EDGE_PART == 0

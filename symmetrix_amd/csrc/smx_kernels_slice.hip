@@ -14,56 +14,12 @@
 //     order, no atomics: results are bit-reproducible.
 // The adjoint kernel writes, per slice, a partial force per edge; a last kernel
 // adds the partials over slices in a fixed order.
+#include "smx_device.hpp"
 #include "smx_kernels.hpp"
 
 namespace smx {
 
 namespace {
-
-__device__ __forceinline__ void sph_l3_s(double x, double y, double z, double* Y)
-{
-    const double s3 = 1.7320508075688772, s15 = 3.872983346207417, s5h = 1.118033988749895;
-    const double s15h = 1.9364916731037085, c3a = 2.091650066335189, s105 = 10.246950765959598;
-    const double c3c = 1.620185174601965, c3d = 1.3228756555322954, c3e = 5.123475382979799;
-    const double xx = x * x, yy = y * y, zz = z * z;
-    Y[0] = 1.0;
-    Y[1] = s3 * y; Y[2] = s3 * z; Y[3] = s3 * x;
-    Y[4] = s15 * x * y; Y[5] = s15 * y * z; Y[6] = s5h * (2 * zz - xx - yy);
-    Y[7] = s15 * x * z; Y[8] = s15h * (xx - yy);
-    Y[9] = c3a * y * (3 * xx - yy); Y[10] = s105 * x * y * z;
-    Y[11] = c3c * y * (4 * zz - xx - yy); Y[12] = c3d * z * (2 * zz - 3 * xx - 3 * yy);
-    Y[13] = c3c * x * (4 * zz - xx - yy); Y[14] = c3e * (xx - yy) * z; Y[15] = c3a * x * (xx - 3 * yy);
-}
-
-// harmonics Y[16] and the derivative of their homogeneous forms along the permuted axes, g[3][16]
-__device__ __forceinline__ void sph_l3_g(double x, double y, double z, double* Y, double (*g)[16])
-{
-    const double s3 = 1.7320508075688772, s15 = 3.872983346207417, s5h = 1.118033988749895;
-    const double s15h = 1.9364916731037085, c3a = 2.091650066335189, s105 = 10.246950765959598;
-    const double c3c = 1.620185174601965, c3d = 1.3228756555322954, c3e = 5.123475382979799;
-    const double xx = x * x, yy = y * y, zz = z * z;
-    Y[0] = 1.0;                              g[0][0] = 0;               g[1][0] = 0;                g[2][0] = 0;
-    Y[1] = s3 * y;                           g[0][1] = 0;               g[1][1] = s3;               g[2][1] = 0;
-    Y[2] = s3 * z;                           g[0][2] = 0;               g[1][2] = 0;                g[2][2] = s3;
-    Y[3] = s3 * x;                           g[0][3] = s3;              g[1][3] = 0;                g[2][3] = 0;
-    Y[4] = s15 * x * y;                      g[0][4] = s15 * y;         g[1][4] = s15 * x;          g[2][4] = 0;
-    Y[5] = s15 * y * z;                      g[0][5] = 0;               g[1][5] = s15 * z;          g[2][5] = s15 * y;
-    Y[6] = s5h * (2 * zz - xx - yy);         g[0][6] = -2 * s5h * x;    g[1][6] = -2 * s5h * y;     g[2][6] = 4 * s5h * z;
-    Y[7] = s15 * x * z;                      g[0][7] = s15 * z;         g[1][7] = 0;                g[2][7] = s15 * x;
-    Y[8] = s15h * (xx - yy);                 g[0][8] = 2 * s15h * x;    g[1][8] = -2 * s15h * y;    g[2][8] = 0;
-    Y[9] = c3a * y * (3 * xx - yy);          g[0][9] = 6 * c3a * x * y; g[1][9] = 3 * c3a * (xx - yy); g[2][9] = 0;
-    Y[10] = s105 * x * y * z;                g[0][10] = s105 * y * z;   g[1][10] = s105 * x * z;    g[2][10] = s105 * x * y;
-    Y[11] = c3c * y * (4 * zz - xx - yy);    g[0][11] = -2 * c3c * x * y; g[1][11] = c3c * (4 * zz - xx - 3 * yy); g[2][11] = 8 * c3c * y * z;
-    Y[12] = c3d * z * (2 * zz - 3 * xx - 3 * yy); g[0][12] = -6 * c3d * x * z; g[1][12] = -6 * c3d * y * z; g[2][12] = 3 * c3d * (2 * zz - xx - yy);
-    Y[13] = c3c * x * (4 * zz - xx - yy);    g[0][13] = c3c * (4 * zz - 3 * xx - yy); g[1][13] = -2 * c3c * x * y; g[2][13] = 8 * c3c * x * z;
-    Y[14] = c3e * (xx - yy) * z;             g[0][14] = 2 * c3e * x * z; g[1][14] = -2 * c3e * y * z; g[2][14] = c3e * (xx - yy);
-    Y[15] = c3a * x * (xx - 3 * yy);         g[0][15] = 3 * c3a * (xx - yy); g[1][15] = -6 * c3a * x * y; g[2][15] = 0;
-}
-
-__device__ __forceinline__ int pair_index_s(int T, int a, int b)
-{
-    return (a <= b) ? a * (2 * T - a - 1) / 2 + b : b * (2 * T - b - 1) / 2 + a;
-}
 
 __device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, size_t bytes)
 {
@@ -73,8 +29,6 @@ __device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, si
     const size_t n = bytes / 16;
     for (size_t q = threadIdx.x; q < n; q += blockDim.x) d[q] = s[q];
 }
-
-constexpr int lm_l(int lm) { return lm < 1 ? 0 : (lm < 4 ? 1 : (lm < 9 ? 2 : 3)); }
 
 struct EdgeGeo {
     double dx, dy, dz, r;
@@ -89,31 +43,6 @@ __device__ __forceinline__ EdgeGeo load_edge(const AggParams<F>& a, int e)
     q.g = a.gather[e];
     q.tj = a.neigh_types[e];
     return q;
-}
-
-// value of the lane ROT places further round its 16-lane row (DPP row_ror: a VALU move, no LDS traffic)
-template <int ROT>
-__device__ __forceinline__ float row_rotate(float v)
-{
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + ROT, 0xf, 0xf, false));
-}
-template <int ROT>
-__device__ __forceinline__ double row_rotate(double v)
-{
-    const long long b = __double_as_longlong(v);
-    const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), 0x120 + ROT, 0xf, 0xf, false);
-    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), 0x120 + ROT, 0xf, 0xf, false);
-    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
-}
-// sum over the lanes of a 16-lane row whose index agrees modulo CL (CL = 1, 2, 4 or 8)
-template <int CL, typename T>
-__device__ __forceinline__ T row_sum_strided(T v)
-{
-    if constexpr (CL <= 8) v += row_rotate<8>(v);
-    if constexpr (CL <= 4) v += row_rotate<4>(v);
-    if constexpr (CL <= 2) v += row_rotate<2>(v);
-    if constexpr (CL <= 1) v += row_rotate<1>(v);
-    return v;
 }
 
 // ---------------------------------------------------------------------------
@@ -163,13 +92,13 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
                 const EdgeGeo cu = nx;
                 if (e + EPR < e1) nx = load_edge(a, e + EPR);
                 const int tj = cu.tj;
-                if (p.U > 1 && a.pair_table[pair_index_s(a.T, ti, tj)] != u) continue;
+                if (p.U > 1 && a.pair_table[pair_index(a.T, ti, tj)] != u) continue;
                 const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
                 const double r = cu.r;
                 const int g = cu.g;
                 const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
                 double Yd[16];
-                sph_l3_s(dz * inv, dx * inv, dy * inv, Yd);
+                sph_l3(dz * inv, dx * inv, dy * inv, Yd);
                 int n = (int)(r / a.spl_h);
                 n = min(max(n, 0), R - 1);
                 const F x = (F)(r - a.spl_h * n);
@@ -259,7 +188,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                 bool on = e < e1;
                 const EdgeGeo cu = nx;
                 if (e + EPR < e1) nx = load_edge(a, e + EPR);
-                if (on && p.U > 1 && a.pair_table[pair_index_s(a.T, ti, cu.tj)] != u) on = false;
+                if (on && p.U > 1 && a.pair_table[pair_index(a.T, ti, cu.tj)] != u) on = false;
                 double fx = 0.0, fy = 0.0, fz = 0.0;
                 if (on) {
                     const double dx = cu.dx, dy = cu.dy, dz = cu.dz;

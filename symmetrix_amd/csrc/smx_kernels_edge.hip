@@ -39,6 +39,20 @@ struct WaveLds {
     }
 };
 
+// Everything computed from roff or boffs after this point is scheduled after the four sums are final.
+template <typename F>
+__device__ __forceinline__ void order_after(F& gx, F& gy, F& gz, F& srad, size_t& roff, int& boffs)
+{
+    asm volatile("" : "+v"(gx), "+v"(gy), "+v"(gz), "+v"(srad), "+v"(roff), "+v"(boffs));
+}
+
+// The value is final here: keeps an accumulation from drifting past the fences (its operands would stay live).
+template <typename F>
+__device__ __forceinline__ void pin(F& v)
+{
+    asm volatile("" : "+v"(v));
+}
+
 template <typename F, int CPL>
 __device__ __forceinline__ Vec<F, CPL> ldv(const F* p)
 {
@@ -163,11 +177,8 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
 // row (mace.cpp:579-604), staged per edge for the deterministic sender-side sum.
 // With more than one channel group (gridDim.y > 1) each group writes its share
 // of the force to fpart[group][edge][3]; the caller adds the groups up.
-#ifndef EXP_WPE
-#define EXP_WPE 2
-#endif
 template <typename F, int LMAXH, int CPL, int EC>
-__global__ __launch_bounds__(256, EXP_WPE) void k_agg_bwd(const AggParams<F> a, const int num_terms)
+__global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const int num_terms)
 {
     using PT = Paths<LMAXH>;
     using WL = WaveLds<F, LMAXH, true>;
@@ -181,7 +192,7 @@ __global__ __launch_bounds__(256, EXP_WPE) void k_agg_bwd(const AggParams<F> a, 
     double* Yt = reinterpret_cast<double*>(base);                                 // [EC][4][16]: Y, dY/dx, dY/dy, dY/dz
     double* us = Yt + EC * 64;                                                    // [EC][4] unit vector xyz/r
     double* xs = us + EC * 4;                                                     // [EC]
-    F* Bs = reinterpret_cast<F*>(xs + EC);                                        // [EC][4][NBP]
+    F* Bs = reinterpret_cast<F*>(xs + EC);                                        // [EC][NBP][4]: B, dB/dx, dB/dy, dB/dz
     int* rows = reinterpret_cast<int*>(Bs + EC * 4 * NBP);
     int* grows = rows + EC;
 
@@ -234,8 +245,9 @@ __global__ __launch_bounds__(256, EXP_WPE) void k_agg_bwd(const AggParams<F> a, 
                 const double* y = Yt + le * 64 + cg_lm1[t];
                 s += cc * y[0]; sx += cc * y[16]; sy += cc * y[32]; sz += cc * y[48];
             }
-            F* o = Bs + (size_t)le * 4 * NBP + b;
-            o[0] = (F)s; o[NBP] = (F)sx; o[2 * NBP] = (F)sy; o[3 * NBP] = (F)sz;
+            Vec<F, 4> o;
+            o.v[0] = (F)s; o.v[1] = (F)sx; o.v[2] = (F)sy; o.v[3] = (F)sz;
+            *reinterpret_cast<Vec<F, 4>*>(Bs + ((size_t)le * NBP + b) * 4) = o;
         }
         wave_lds_sync();
         for (int le = 0; le < nE; ++le) {
@@ -262,52 +274,46 @@ __global__ __launch_bounds__(256, EXP_WPE) void k_agg_bwd(const AggParams<F> a, 
                     constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
                     constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1, nb = (2 * l + 1) * n2;
                     const F* rowp = a.tabK + roff;
-                    const F* B = Bs + boffs;
-                    Vec<F, 4> cf[CPL];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) cf[c] = ldv<F, 4>(rowp + (c * P + p) * 4);
-                    F Bv[nb], uu[nb];
-#pragma unroll
-                    for (int q = 0; q < nb; ++q) { Bv[q] = B[bo + q]; uu[q] = F(0); }
+                    F R[CPL], Rd[CPL];
 #pragma unroll
                     for (int c = 0; c < CPL; ++c) {
-                        const F R = cf[c].v[0] + x * (cf[c].v[1] + x * (cf[c].v[2] + x * cf[c].v[3]));
-                        const F Rd = cf[c].v[1] + x * (F(2) * cf[c].v[2] + F(3) * x * cf[c].v[3]);
+                        const Vec<F, 4> cf = ldv<F, 4>(rowp + (c * P + p) * 4);
+                        R[c] = cf.v[0] + x * (cf.v[1] + x * (cf.v[2] + x * cf.v[3]));
+                        Rd[c] = cf.v[1] + x * (F(2) * cf.v[2] + F(3) * x * cf.v[3]);
+                    }
+                    // rows m of B in groups of MG; a fence after each group bounds the LDS values in flight
+                    constexpr int MG = n2 == 1 ? 2 * l + 1 : 3;
+                    static_for<0, (2 * l + 1 + MG - 1) / MG>([&](auto gc) {
+                        constexpr int m0 = decltype(gc)::value * MG;
+                        constexpr int m1 = m0 + MG < 2 * l + 1 ? m0 + MG : 2 * l + 1;
+                        const F* B4 = Bs + boffs + (bo + m0 * n2) * 4;
+                        Vec<F, 4> b4[(m1 - m0) * n2];
 #pragma unroll
-                        for (int m = 0; m < 2 * l + 1; ++m) {
-                            const F dd = d[c][lme0 + m * es];
-                            const F t = dd * R, td = dd * Rd;
-                            F z = F(0);
+                        for (int q = 0; q < (m1 - m0) * n2; ++q) b4[q] = ldv<F, 4>(B4 + 4 * q);
 #pragma unroll
-                            for (int m2 = 0; m2 < n2; ++m2) {
-                                const F h = H[l2 * l2 + m2].v[c];
-                                z += Bv[m * n2 + m2] * h;
-                                mg[l2 * l2 + m2].v[c] += t * Bv[m * n2 + m2];
-                                uu[m * n2 + m2] += t * h;
+                        for (int c = 0; c < CPL; ++c) {
+#pragma unroll
+                            for (int m = m0; m < m1; ++m) {
+                                const F dd = d[c][lme0 + m * es];
+                                const F t = dd * R[c];
+                                F z = F(0), zx = F(0), zy = F(0), zz = F(0);
+#pragma unroll
+                                for (int m2 = 0; m2 < n2; ++m2) {
+                                    const F h = H[l2 * l2 + m2].v[c];
+                                    const Vec<F, 4>& bb = b4[(m - m0) * n2 + m2];
+                                    z += bb.v[0] * h; zx += bb.v[1] * h; zy += bb.v[2] * h; zz += bb.v[3] * h;
+                                    mg[l2 * l2 + m2].v[c] += t * bb.v[0];
+                                }
+                                srad += dd * Rd[c] * z;
+                                gx += t * zx; gy += t * zy; gz += t * zz;
                             }
-                            srad += td * z;
                         }
-                    }
-                    // the channels of this lane share the gradient of B; one component at a time (fenced like the paths)
-                    asm volatile("" : "+v"(uu[0]), "+v"(srad), "+v"(boffs));
-                    {
-                        const F* Bg = Bs + boffs + NBP + bo;
+                        order_after(gx, gy, gz, srad, roff, boffs);
 #pragma unroll
-                        for (int q = 0; q < nb; ++q) gx += uu[q] * Bg[q];
-                    }
-                    asm volatile("" : "+v"(gx), "+v"(boffs));
-                    {
-                        const F* Bg = Bs + boffs + 2 * NBP + bo;
+                        for (int m2 = 0; m2 < n2; ++m2)
 #pragma unroll
-                        for (int q = 0; q < nb; ++q) gy += uu[q] * Bg[q];
-                    }
-                    asm volatile("" : "+v"(gy), "+v"(boffs));
-                    {
-                        const F* Bg = Bs + boffs + 3 * NBP + bo;
-#pragma unroll
-                        for (int q = 0; q < nb; ++q) gz += uu[q] * Bg[q];
-                    }
-                    asm volatile("" : "+v"(gz), "+v"(roff), "+v"(boffs));
+                            for (int c = 0; c < CPL; ++c) pin(mg[l2 * l2 + m2].v[c]);
+                    });
                 });
                 if (a.msg) {
                     F* mrow = a.msg + (size_t)(eb + le) * NLM * K + k0;
@@ -350,20 +356,20 @@ hipError_t launch_agg_t(const AggParams<F>& p, hipStream_t s)
     return hipGetLastError();
 }
 
-// channels per lane: two where the channel count allows paired loads and the registers hold the accumulators
+// Channels per lane.  Two give paired loads and fewer broadcast reads per channel; the l <= 1 path list holds
+// 40 accumulators per channel, which leaves room for two channels only in the single-precision forward kernel.
 template <typename F, int LMAXH, bool BWD>
-constexpr int agg_cpl_wide()
+int agg_cpl(int K)
 {
-    if (LMAXH == 0) return 2;
-    return BWD ? 1 : 2;   // the adjoint of the l <= 1 paths holds 40 adjoint values per channel
+    const bool wide = LMAXH == 0 || (!BWD && sizeof(F) == 4);
+    return (wide && K > 64 && K % 2 == 0) ? 2 : 1;
 }
 
 template <typename F, int LMAXH, bool BWD>
 hipError_t launch_agg_sel(const AggParams<F>& p, hipStream_t s)
 {
     constexpr int EC = LMAXH == 0 ? 16 : (BWD ? (sizeof(F) == 4 ? 8 : 4) : 16);
-    constexpr int CW = agg_cpl_wide<F, LMAXH, BWD>();
-    if (CW == 2 && p.K > 64 && p.K % 2 == 0) return launch_agg_t<F, LMAXH, CW, EC, BWD>(p, s);
+    if (agg_cpl<F, LMAXH, BWD>(p.K) == 2) return launch_agg_t<F, LMAXH, 2, EC, BWD>(p, s);
     return launch_agg_t<F, LMAXH, 1, EC, BWD>(p, s);
 }
 
@@ -386,9 +392,7 @@ hipError_t launch_agg_bwd(int L_max_H, const AggParams<F>& p, hipStream_t s)
 template <typename F>
 int agg_bwd_groups(int L_max_H, int K)
 {
-    int cpl = 1;
-    if (K > 64 && K % 2 == 0)
-        cpl = L_max_H == 0 ? agg_cpl_wide<F, 0, true>() : agg_cpl_wide<F, 1, true>();
+    const int cpl = L_max_H == 0 ? agg_cpl<F, 0, true>(K) : agg_cpl<F, 1, true>(K);
     return (K + 64 * cpl - 1) / (64 * cpl);
 }
 // This file is compiled four times (SMX_EDGE_PART = 0..3), one object per

@@ -59,6 +59,8 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-atoms", type=int, default=0, help="atoms in the CPU sample (0 = whole workload)")
     ap.add_argument("--model-dir", default=tempfile.gettempdir())
+    ap.add_argument("--calibrate-copy", action="store_true",
+                    help="also launch one device-to-device copy of 1 GiB (a kernel of known traffic for counter runs)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives exist in it); use --gpus 1", file=sys.stderr)
@@ -133,6 +135,13 @@ def main():
         del eng
         return dict(ms_sync=1e3 * dt / steps, ms=1e3 * dt_async / steps, stages=stages, energy=energy, fmax=fmax,
                     forces=out_F.cpu().numpy().copy())
+
+    if args.calibrate_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB read + 1 GiB written
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
 
     res = run_mode(args.dtype, args.steps, args.warmup)
     other = "float32" if args.dtype == "float64" else "float64"

@@ -99,9 +99,9 @@ static void upload_as(DVec<T>& d, const std::vector<S>& h, hipStream_t s)
 
 static const char* kStageNames =
     "prep;agg0_fwd;A0_lin;M0;H1;agg1_fwd;A1;M1;H2;readout;rev_H2;rev_M1;rev_A1;agg1_bwd;sender_reduce;"
-    "rev_H1;rev_M0;rev_A0_lin;agg0_bwd";
+    "rev_H1;rev_M0;rev_A0_lin;agg0_bwd;force_sum1;force_sum0";
 enum Stage { ST_PREP, ST_AGG0F, ST_A0LIN, ST_M0, ST_H1, ST_AGG1F, ST_A1, ST_M1, ST_H2, ST_READOUT, ST_REVH2,
-             ST_REVM1, ST_REVA1, ST_AGG1B, ST_SRED, ST_REVH1, ST_REVM0, ST_REVA0LIN, ST_AGG0B, ST_COUNT };
+             ST_REVM1, ST_REVA1, ST_AGG1B, ST_SRED, ST_REVH1, ST_REVM0, ST_REVA0LIN, ST_AGG0B, ST_FSUM1, ST_FSUM0, ST_COUNT };
 
 struct EngineBase {
     virtual ~EngineBase() = default;
@@ -472,14 +472,25 @@ struct Engine : EngineBase {
         HIPCHK(launch_agg_fwd<F>(0, p, stream));
     }
     template <typename TA, typename TC, typename CT>
-    GemmParams<TA, TC, CT> gemm_base(const TA* A, long a_stride, TC* C, long c_stride, const CT* W, long w_type_stride,
-                                     bool typed, int N, int transW, int accumulate)
+    GemmParams<TA, TC, CT> gemm_base(int N, bool typed)
     {
         GemmParams<TA, TC, CT> g{};
-        g.A = A; g.a_node_stride = a_stride; g.C = C; g.c_node_stride = c_stride; g.W = W;
-        g.w_type_stride = w_type_stride; g.transW = transW; g.accumulate = accumulate; g.num_nodes = N;
-        if (typed) { g.node_types = node_types; g.perm = t_perm.p; g.tstart = t_start.p; g.T = hm.T; }
+        g.num_nodes = N;
+        if (typed) { need(t_perm.p, "species groups"); g.perm = t_perm.p; g.tstart = t_start.p; g.T = hm.T; }
         return g;
+    }
+    template <typename TA, typename TC, typename CT>
+    static GemmProb<TA, TC, CT> gemm_prob(const TA* A, long a_node_stride, long a_off, long a_sub_stride, TC* C,
+                                          long c_node_stride, long c_off, long c_sub_stride, const CT* W,
+                                          long w_type_stride, long w_off, int transW, int accumulate, int Kd, int Nn,
+                                          int sub)
+    {
+        GemmProb<TA, TC, CT> q{};
+        q.A = A; q.a_node_stride = a_node_stride; q.a_off = a_off; q.a_sub_stride = a_sub_stride;
+        q.C = C; q.c_node_stride = c_node_stride; q.c_off = c_off; q.c_sub_stride = c_sub_stride;
+        q.W = W; q.w_type_stride = w_type_stride; q.w_off = w_off; q.transW = transW; q.accumulate = accumulate;
+        q.Kd = Kd; q.Nn = Nn; q.sub = sub;
+        return q;
     }
     // A0[i, l-block] = Phi0[i, l-block] . A0_weights[type_i][l]  (reverse: transposed weights)
     void st_A0_lin(int N, bool reverse)
@@ -488,10 +499,11 @@ struct Engine : EngineBase {
         const F* src = reverse ? A0_adj.p : Phi0.p;
         if (reverse) Phi0.size_to((size_t)N * 16 * k, stream); else A0.size_to((size_t)N * 16 * k, stream);
         F* dst = reverse ? Phi0.p : A0.p;
-        auto g = gemm_base<F, F, F>(src, 16L * k, dst, 16L * k, A0w.p, 4L * k * k, true, N, reverse ? 1 : 0, 0);
+        auto g = gemm_base<F, F, F>(N, true);
         g.nprob = 4;
         for (int l = 0; l < 4; ++l)
-            g.prob[l] = GemmProb{(long)l * l * k, k, (long)l * l * k, k, (long)l * k * k, k, k, 2 * l + 1};
+            g.prob[l] = gemm_prob<F, F, F>(src, 16L * k, (long)l * l * k, k, dst, 16L * k, (long)l * l * k, k, A0w.p,
+                                           4L * k * k, (long)l * k * k, reverse ? 1 : 0, 0, k, k, 2 * l + 1);
         HIPCHK((launch_gemm<F, F, F>(g, stream)));
     }
     void st_poly(int N, bool layer1)
@@ -517,11 +529,13 @@ struct Engine : EngineBase {
         const int k = K(), nlm = NLM();
         if (reverse) M0_adj.size_to(M0.n, stream);
         else if (H1.n != M0.n) H1.resize(M0.n, stream);   // mace.cpp:400
-        auto g = gemm_base<F, F, F>(reverse ? H1_adj.p : M0.p, (long)nlm * k, reverse ? M0_adj.p : H1.p, (long)nlm * k,
-                                    H1w.p, 0, false, N, reverse ? 1 : 0, 0);
+        const F* src = reverse ? H1_adj.p : M0.p;
+        F* dst = reverse ? M0_adj.p : H1.p;
+        auto g = gemm_base<F, F, F>(N, false);
         g.nprob = hm.L_max + 1;
         for (int l = 0; l <= hm.L_max; ++l)
-            g.prob[l] = GemmProb{(long)l * l * k, k, (long)l * l * k, k, (long)l * k * k, k, k, 2 * l + 1};
+            g.prob[l] = gemm_prob<F, F, F>(src, (long)nlm * k, (long)l * l * k, k, dst, (long)nlm * k, (long)l * l * k, k,
+                                           H1w.p, 0, (long)l * k * k, reverse ? 1 : 0, 0, k, k, 2 * l + 1);
         HIPCHK((launch_gemm<F, F, F>(g, stream)));
     }
     void st_agg1_fwd(int N)
@@ -543,48 +557,45 @@ struct Engine : EngineBase {
         const int k = K(), ne = NE();
         if (reverse) dPhi1.size_to(Phi1.n, stream); else A1.size_to((size_t)N * 16 * k, stream);
         long lme_off = 0;
-        if (!reverse) {
-            auto g = gemm_base<F, F, F>(Phi1.p, (long)ne * k, A1.p, 16L * k, A1w.p, 0, false, N, 0, 0);
-            g.nprob = 4;
-            for (int l = 0; l < 4; ++l) {
-                const int nel = hm.num_e[l];
-                g.prob[l] = GemmProb{lme_off * k, (long)nel * k, (long)l * l * k, k, A1w_off[l], nel * k, k, 2 * l + 1};
-                lme_off += (2 * l + 1) * nel;
-            }
-            HIPCHK((launch_gemm<F, F, F>(g, stream)));
-        } else {
-            auto g = gemm_base<F, F, F>(A1_adj.p, 16L * k, dPhi1.p, (long)ne * k, A1w.p, 0, false, N, 1, 0);
-            g.nprob = 4;
-            for (int l = 0; l < 4; ++l) {
-                const int nel = hm.num_e[l];
-                g.prob[l] = GemmProb{(long)l * l * k, k, lme_off * k, (long)nel * k, A1w_off[l], k, nel * k, 2 * l + 1};
-                lme_off += (2 * l + 1) * nel;
-            }
-            HIPCHK((launch_gemm<F, F, F>(g, stream)));
+        auto g = gemm_base<F, F, F>(N, false);
+        g.nprob = 4;
+        for (int l = 0; l < 4; ++l) {
+            const int nel = hm.num_e[l];
+            if (!reverse)
+                g.prob[l] = gemm_prob<F, F, F>(Phi1.p, (long)ne * k, lme_off * k, (long)nel * k, A1.p, 16L * k,
+                                               (long)l * l * k, k, A1w.p, 0, A1w_off[l], 0, 0, nel * k, k, 2 * l + 1);
+            else
+                g.prob[l] = gemm_prob<F, F, F>(A1_adj.p, 16L * k, (long)l * l * k, k, dPhi1.p, (long)ne * k, lme_off * k,
+                                               (long)nel * k, A1w.p, 0, A1w_off[l], 1, 0, k, nel * k, 2 * l + 1);
+            lme_off += (2 * l + 1) * nel;
         }
+        HIPCHK((launch_gemm<F, F, F>(g, stream)));
     }
+    // H2 = H1[l=0] . W_H1[type] + M1 . W_M1 in one launch (mace.cpp:820-845)
     void st_H2(int N)
     {
         const int k = K(), nlm = NLM();
         H2.size_to((size_t)N * k, stream);
-        auto g1 = gemm_base<F, double, double>(H1.p, (long)nlm * k, H2.p, k, H2w_H1.p, (long)k * k, true, N, 0, 0);
-        g1.nprob = 1; g1.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
-        HIPCHK((launch_gemm<F, double, double>(g1, stream)));
-        auto g2 = gemm_base<F, double, double>(M1.p, k, H2.p, k, H2w_M1.p, 0, false, N, 0, 1);
-        g2.nprob = 1; g2.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
-        HIPCHK((launch_gemm<F, double, double>(g2, stream)));
+        auto g = gemm_base<F, double, double>(N, true);
+        g.nprob = 1;
+        g.prob[0] = gemm_prob<F, double, double>(H1.p, (long)nlm * k, 0, 0, H2.p, k, 0, 0, H2w_H1.p, (long)k * k, 0, 0, 0,
+                                                 k, k, 1);
+        g.prob[0].A2 = M1.p; g.prob[0].a2_node_stride = k; g.prob[0].W2 = H2w_M1.p; g.prob[0].w2_type_stride = 0;
+        g.prob[0].transW2 = 0; g.prob[0].Kd2 = k;
+        HIPCHK((launch_gemm<F, double, double>(g, stream)));
     }
+    // H1_adj[l=0] += H2_adj . W_H1[type]^T and M1_adj = H2_adj . W_M1^T in one launch
     void st_reverse_H2(int N, bool zero_H1_adj)
     {
         const int k = K(), nlm = NLM();
         H1_adj.resize(H1.n, stream); M1_adj.size_to(M1.n, stream);
         if (zero_H1_adj) HIPCHK(hipMemsetAsync(H1_adj.p, 0, H1_adj.n * sizeof(F), stream));
-        auto g1 = gemm_base<double, F, double>(H2_adj.p, k, H1_adj.p, (long)nlm * k, H2w_H1.p, (long)k * k, true, N, 1, 1);
-        g1.nprob = 1; g1.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
-        HIPCHK((launch_gemm<double, F, double>(g1, stream)));
-        auto g2 = gemm_base<double, F, double>(H2_adj.p, k, M1_adj.p, k, H2w_M1.p, 0, false, N, 1, 0);
-        g2.nprob = 1; g2.prob[0] = GemmProb{0, 0, 0, 0, 0, k, k, 1};
-        HIPCHK((launch_gemm<double, F, double>(g2, stream)));
+        auto g = gemm_base<double, F, double>(N, true);
+        g.nprob = 2;
+        g.prob[0] = gemm_prob<double, F, double>(H2_adj.p, k, 0, 0, H1_adj.p, (long)nlm * k, 0, 0, H2w_H1.p, (long)k * k,
+                                                 0, 1, 1, k, k, 1);
+        g.prob[1] = gemm_prob<double, F, double>(H2_adj.p, k, 0, 0, M1_adj.p, k, 0, 0, H2w_M1.p, 0, 0, 1, 0, k, k, 1);
+        HIPCHK((launch_gemm<double, F, double>(g, stream)));
     }
     void st_readouts(int N, bool zero_energies)
     {
@@ -595,13 +606,15 @@ struct Engine : EngineBase {
         hidden.size_to((size_t)N * 16, stream);
         const int rows = (int)(H1.n / ((size_t)nlm * k));
         HIPCHK(launch_seed_H1_adj<F>(rows, N, nlm, k, ro1.p, H1_adj.p, stream));
-        auto g1 = gemm_base<double, double, double>(H2.p, k, hidden.p, 16, ro2_w1.p, 0, false, N, 1, 0);
-        g1.nprob = 1; g1.prob[0] = GemmProb{0, 0, 0, 0, 0, k, 16, 1};
+        auto g1 = gemm_base<double, double, double>(N, false);
+        g1.nprob = 1;
+        g1.prob[0] = gemm_prob<double, double, double>(H2.p, k, 0, 0, hidden.p, 16, 0, 0, ro2_w1.p, 0, 0, 1, 0, k, 16, 1);
         HIPCHK((launch_gemm<double, double, double>(g1, stream)));
         HIPCHK(launch_readout<F>(N, k, nlm, node_types, E0.p, ro1.p, H1.p, hidden.p, ro2_w2.p, hm.readout_2_scale,
                                  node_energies.p, zero_energies ? 1 : 0, stream));
-        auto g2 = gemm_base<double, double, double>(hidden.p, 16, H2_adj.p, k, ro2_w1.p, 0, false, N, 0, 0);
-        g2.nprob = 1; g2.prob[0] = GemmProb{0, 0, 0, 0, 0, 16, k, 1};
+        auto g2 = gemm_base<double, double, double>(N, false);
+        g2.nprob = 1;
+        g2.prob[0] = gemm_prob<double, double, double>(hidden.p, 16, 0, 0, H2_adj.p, k, 0, 0, ro2_w1.p, 0, 0, 0, 0, 16, k, 1);
         HIPCHK((launch_gemm<double, double, double>(g2, stream)));
     }
     void st_reverse_M1(int N)
@@ -629,13 +642,15 @@ struct Engine : EngineBase {
             fpart.size_to((size_t)S * 3 * E, stream);
             sp.a.d_out = dPhi1.p; sp.a.msg = msg.p; sp.fpart = fpart.p;
             HIPCHK(launch_slice_bwd<F>(sp, stream));
+            stage_end(ST_AGG1B);
+            stage_begin(ST_FSUM1);
             HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, stream));
+            stage_end(ST_FSUM1);
         } else {
             auto p = agg_params(1, N);
             p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
-            agg_bwd_general(hm.L_max, p);
+            agg_bwd_general(hm.L_max, p, ST_AGG1B, ST_FSUM1);
         }
-        stage_end(ST_AGG1B);
         // edges beyond the first N receivers carry no layer-1 adjoint
         const long EN = E;  // first_neigh[N] == E whenever the list covers exactly N receivers
         (void)EN;
@@ -655,24 +670,34 @@ struct Engine : EngineBase {
             const int S = (K() + sp.CH - 1) / sp.CH;
             fpart.size_to((size_t)S * 3 * E, stream);
             sp.a.d_out = Phi0.p; sp.a.msg = nullptr; sp.fpart = fpart.p;
+            stage_begin(ST_AGG0B);
             HIPCHK(launch_slice_bwd<F>(sp, stream));
+            stage_end(ST_AGG0B);
+            stage_begin(ST_FSUM0);
             HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, 1, stream));
+            stage_end(ST_FSUM0);
             return;
         }
         auto p = agg_params(0, N);
         p.d_out = Phi0.p; p.forces = node_forces.p; p.accumulate_forces = 1; p.msg = nullptr;
-        agg_bwd_general(0, p);
+        agg_bwd_general(0, p, ST_AGG0B, ST_FSUM0);
     }
     // general adjoint kernel; wide models are cut into channel groups whose partial forces are added in order
-    void agg_bwd_general(int L_max_H, AggParams<F>& p)
+    void agg_bwd_general(int L_max_H, AggParams<F>& p, int st_kernel, int st_sum)
     {
         const int groups = agg_bwd_groups<F>(L_max_H, K());
         if (groups > 1) {
             fpart.size_to((size_t)groups * 3 * E, stream);
             p.fpart = fpart.p;
         }
+        stage_begin(st_kernel);
         HIPCHK(launch_agg_bwd<F>(L_max_H, p, stream));
-        if (groups > 1) HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, p.accumulate_forces, stream));
+        stage_end(st_kernel);
+        if (groups > 1) {
+            stage_begin(st_sum);
+            HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, p.accumulate_forces, stream));
+            stage_end(st_sum);
+        }
     }
 
     // ------------------------------------------------------------------
@@ -719,7 +744,7 @@ struct Engine : EngineBase {
         stage_begin(ST_REVH1); st_H1(N, true); stage_end(ST_REVH1);
         stage_begin(ST_REVM0); st_reverse_M0(N); stage_end(ST_REVM0);
         stage_begin(ST_REVA0LIN); st_A0_lin(N, true); stage_end(ST_REVA0LIN);
-        stage_begin(ST_AGG0B); st_agg0_bwd(N); stage_end(ST_AGG0B);
+        st_agg0_bwd(N);
 
         if (d_energies) HIPCHK(hipMemcpyAsync(d_energies, node_energies.p, (size_t)N * sizeof(double), hipMemcpyDeviceToDevice, stream));
         if (d_forces && E) HIPCHK(hipMemcpyAsync(d_forces, node_forces.p, (size_t)3 * E * sizeof(double), hipMemcpyDeviceToDevice, stream));

@@ -116,30 +116,34 @@ template <typename F>
 hipError_t launch_poly_reverse(int N, int NP, int K, const F* M_grad, const F* M_adj, F* A_adj, hipStream_t s);
 
 // ---------------------------------------------------------------------------
-// Dense channel mixing on the matrix cores.
+// Dense channel mixing on the matrix cores.  A launch holds up to four
+// independent products (blockIdx.z), each
 //   C[row(node,s)][n] (+)= sum_k A[row(node,s)][k] * W[type(node)][k][n]   (or W^T)
+//                          (+ sum_k A2[node][k] * W2[type(node)][k][n] when A2 is set)
 // rows are (node, s) with s < sub; row (node,s) of A starts at
 // A + node*a_node_stride + a_off + s*a_sub_stride and is Kd long.
+template <typename TA, typename TC, typename CT>
 struct GemmProb {
-    long a_off, a_sub_stride;   // row (node,s) of A starts at A + node*a_node_stride + a_off + s*a_sub_stride
-    long c_off, c_sub_stride;
-    long w_off;                 // offset of this problem's weight block inside W[type]
-    int Kd, Nn, sub;            // inner size, output columns, rows per node
+    const TA* A; long a_node_stride, a_off, a_sub_stride;
+    TC* C; long c_node_stride, c_off, c_sub_stride;
+    const CT* W; long w_type_stride, w_off;   // w_type_stride 0: one matrix for all species
+    int transW;              // 0: W block is [Kd][Nn]; 1: W block is [Nn][Kd]
+    int accumulate;          // 1: C += ...
+    int Kd, Nn, sub;         // inner size, output columns, rows per node
+    // optional second product into the same rows (sub must be 1): row of A2 starts at A2 + node*a2_node_stride
+    const TA* A2; long a2_node_stride;
+    const CT* W2; long w2_type_stride;
+    int transW2, Kd2;
 };
 template <typename TA, typename TC, typename CT>
 struct GemmParams {
-    const TA* A; long a_node_stride;
-    TC* C; long c_node_stride;
-    const CT* W; long w_type_stride;
-    int transW;              // 0: W block is [Kd][Nn]; 1: W block is [Nn][Kd]
-    int accumulate;          // 1: C += ...
     int num_nodes;
-    const int* node_types;   // null -> single weight matrix
-    const int* perm;         // [num_nodes] nodes grouped by type (with node_types)
+    const int* perm;         // [num_nodes] nodes grouped by species, or null when no weight depends on the species
     const int* tstart;       // [T+1]
     int T;
-    int nprob;               // sub-problems selected by blockIdx.z (one per l)
-    GemmProb prob[4];
+    int nprob;
+    int vec_ok;              // set by launch_gemm: every offset and size is a multiple of four elements
+    GemmProb<TA, TC, CT> prob[4];
 };
 template <typename TA, typename TC, typename CT>
 hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p, hipStream_t s);

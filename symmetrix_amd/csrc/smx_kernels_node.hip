@@ -381,153 +381,6 @@ template hipError_t launch_poly_reverse<double>(int, int, int, const double*, co
 template hipError_t launch_poly_reverse<float>(int, int, int, const float*, const float*, float*, hipStream_t);
 
 // ===========================================================================
-// Channel-mixing linears on the matrix cores.
-//
-// Block tile: 64 rows x 64 columns, four wavefronts, wavefront w owns rows
-// 16w..16w+15 and all four 16-column tiles; K is consumed in slabs of 16 staged
-// through LDS.  v_mfma_f64_16x16x4_f64 / v_mfma_f32_16x16x4_f32 operand layout:
-// lane L supplies A[L%16][L/16] and B[L/16][L%16] of a 16x4 by 4x16 product;
-// accumulator register r holds column L%16 of row 4*(L/16)+r (f32) or of row
-// 4*r+L/16 (f64).
-namespace {
-constexpr int GM = 64, GN = 64, GK = 16;
-
-template <typename CT> struct Mfma;
-template <> struct Mfma<double> {
-    typedef double acc_t __attribute__((ext_vector_type(4)));
-    // accumulator register r of lane L holds output row 4*r + L/16
-    __device__ static int out_row(int lane, int r) { return 4 * r + (lane >> 4); }
-    __device__ static acc_t run(double a, double b, acc_t c) { return __builtin_amdgcn_mfma_f64_16x16x4f64(a, b, c, 0, 0, 0); }
-};
-template <> struct Mfma<float> {
-    typedef float acc_t __attribute__((ext_vector_type(4)));
-    // accumulator register r of lane L holds output row 4*(L/16) + r
-    __device__ static int out_row(int lane, int r) { return 4 * (lane >> 4) + r; }
-    __device__ static acc_t run(float a, float b, acc_t c) { return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0); }
-};
-
-template <typename TA, typename TC, typename CT>
-__global__ __launch_bounds__(256) void k_gemm(const GemmParams<TA, TC, CT> g)
-{
-    __shared__ CT As[GM][GK + 1];
-    __shared__ CT Ws[GK][GN + 1];
-    __shared__ long a_row_off[GM];
-    __shared__ long c_row_off[GM];
-    const GemmProb pr = g.prob[blockIdx.z];
-    const int Kd = pr.Kd, Nn = pr.Nn, sub = pr.sub;
-    if ((int)blockIdx.y * GN >= Nn) return;
-    // locate this block's type segment and row tile
-    int type = 0, tile = blockIdx.x, nrows_seg = g.num_nodes * sub, seg_node0 = 0;
-    if (g.node_types) {
-        bool found = false;
-        for (int t = 0; t < g.T; ++t) {
-            const int n_t = g.tstart[t + 1] - g.tstart[t];
-            const int tiles = (n_t * sub + GM - 1) / GM;
-            if (tile < tiles) { type = t; nrows_seg = n_t * sub; seg_node0 = g.tstart[t]; found = true; break; }
-            tile -= tiles;
-        }
-        if (!found) return;
-    } else if (tile * GM >= nrows_seg) {
-        return;
-    }
-    const int row0 = tile * GM;
-    const int col0 = blockIdx.y * GN;
-    const int tid = threadIdx.x;
-    if (tid < GM) {
-        const int rr = row0 + tid;
-        long ao = -1, co = -1;
-        if (rr < nrows_seg) {
-            const int ns = rr / sub, sb = rr % sub;
-            const int node = g.node_types ? g.perm[seg_node0 + ns] : ns;
-            ao = (long)node * g.a_node_stride + pr.a_off + (long)sb * pr.a_sub_stride;
-            co = (long)node * g.c_node_stride + pr.c_off + (long)sb * pr.c_sub_stride;
-        }
-        a_row_off[tid] = ao;
-        c_row_off[tid] = co;
-    }
-    __syncthreads();
-    const CT* W = g.W + (size_t)type * g.w_type_stride + pr.w_off;
-    const int wave = tid >> 6, lane = tid & 63;
-    typename Mfma<CT>::acc_t acc[GN / 16];
-#pragma unroll
-    for (int t = 0; t < GN / 16; ++t) acc[t] = {0, 0, 0, 0};
-
-    for (int k0 = 0; k0 < Kd; k0 += GK) {
-        // stage A: 64 x 16, thread t loads row t/4, columns 4*(t%4)..+3
-        {
-            const int r = tid >> 2, c4 = (tid & 3) * 4;
-            const long ao = a_row_off[r];
-#pragma unroll
-            for (int c = 0; c < 4; ++c) {
-                const int kk = k0 + c4 + c;
-                As[r][c4 + c] = (ao >= 0 && kk < Kd) ? (CT)g.A[ao + kk] : CT(0);
-            }
-        }
-        // stage W: 16 x 64
-        {
-            if (!g.transW) {
-                const int r = tid >> 4, c4 = (tid & 15) * 4;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int kk = k0 + r, nn = col0 + c4 + c;
-                    Ws[r][c4 + c] = (kk < Kd && nn < Nn) ? W[(size_t)kk * Nn + nn] : CT(0);
-                }
-            } else {
-                // W is [Nn][Kd]: thread t loads column n = t/4, k = 4*(t%4)..+3 (contiguous in memory)
-                const int n = tid >> 2, r4 = (tid & 3) * 4;
-#pragma unroll
-                for (int c = 0; c < 4; ++c) {
-                    const int kk = k0 + r4 + c, nn = col0 + n;
-                    Ws[r4 + c][n] = (kk < Kd && nn < Nn) ? W[(size_t)nn * Kd + kk] : CT(0);
-                }
-            }
-        }
-        __syncthreads();
-#pragma unroll
-        for (int kk = 0; kk < GK; kk += 4) {
-            const CT av = As[wave * 16 + (lane & 15)][kk + (lane >> 4)];
-#pragma unroll
-            for (int t = 0; t < GN / 16; ++t) {
-                const CT bv = Ws[kk + (lane >> 4)][t * 16 + (lane & 15)];
-                acc[t] = Mfma<CT>::run(av, bv, acc[t]);
-            }
-        }
-        __syncthreads();
-    }
-#pragma unroll
-    for (int t = 0; t < GN / 16; ++t) {
-        const int nn = col0 + t * 16 + (lane & 15);
-        if (nn >= Nn) continue;
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-            const long co = c_row_off[wave * 16 + Mfma<CT>::out_row(lane, r)];
-            if (co < 0) continue;
-            const CT v = acc[t][r];
-            if (g.accumulate) g.C[co + nn] = (TC)((CT)g.C[co + nn] + v);
-            else g.C[co + nn] = (TC)v;
-        }
-    }
-}
-}  // namespace
-
-template <typename TA, typename TC, typename CT>
-hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p, hipStream_t s)
-{
-    if (p.num_nodes <= 0 || p.nprob <= 0) return hipSuccess;
-    int max_sub = 0, max_n = 0;
-    for (int z = 0; z < p.nprob; ++z) { max_sub = max_sub > p.prob[z].sub ? max_sub : p.prob[z].sub; max_n = max_n > p.prob[z].Nn ? max_n : p.prob[z].Nn; }
-    const long rows = (long)p.num_nodes * max_sub;
-    const unsigned gx = (unsigned)((rows + GM - 1) / GM + (p.node_types ? p.T : 0));
-    const unsigned gy = (unsigned)((max_n + GN - 1) / GN);
-    hipLaunchKernelGGL((k_gemm<TA, TC, CT>), dim3(gx, gy, p.nprob), dim3(256), 0, s, p);
-    return hipGetLastError();
-}
-template hipError_t launch_gemm<double, double, double>(const GemmParams<double, double, double>&, hipStream_t);
-template hipError_t launch_gemm<float, float, float>(const GemmParams<float, float, float>&, hipStream_t);
-template hipError_t launch_gemm<float, double, double>(const GemmParams<float, double, double>&, hipStream_t);
-template hipError_t launch_gemm<double, float, double>(const GemmParams<double, float, double>&, hipStream_t);
-
-// ===========================================================================
 // Readout tail
 namespace {
 template <typename F>

@@ -104,6 +104,30 @@ __device__ __forceinline__ void sph_l3_grad(double x, double y, double z, double
     }
 }
 
+// 1/sqrt(a) and 1/a for positive normal a: hardware estimate (about 23 bits) and two Newton steps, good to
+// the last bit or two.  The library forms (sqrt then divide, IEEE divide) cost four to five times as many
+// instructions, and the edge kernels evaluate them per (edge, channel slice).
+__device__ __forceinline__ double rsqrt_pos(double a)
+{
+    double y = __builtin_amdgcn_rsq(a);
+    const double h = 0.5 * a;
+    y = fma(y, fma(-h * y, y, 0.5), y);
+    y = fma(y, fma(-h * y, y, 0.5), y);
+    return y;
+}
+__device__ __forceinline__ double rcp_pos(double a)
+{
+    double y = __builtin_amdgcn_rcp(a);
+    y = fma(y, fma(-a, y, 1.0), y);
+    y = fma(y, fma(-a, y, 1.0), y);
+    return y;
+}
+// spline interval of r: floor(r / h) computed with the reciprocal spacing, clamped to the table
+__device__ __forceinline__ int spline_interval(double r, double inv_h, int last)
+{
+    return min(max((int)(r * inv_h), 0), last);
+}
+
 __device__ __forceinline__ int pair_index(int T, int a, int b)
 {
     return (a <= b) ? a * (2 * T - a - 1) / 2 + b : b * (2 * T - b - 1) / 2 + a;

@@ -172,7 +172,7 @@ struct Engine : EngineBase {
     const double *xyz = nullptr, *r = nullptr;
     long E = 0;
     int N_geo = 0;
-    DVec<int> first_neigh, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
+    DVec<int> first_neigh, recv_order, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
     int sender_rows = 0;
 
     // ---- state (mace.hpp members)
@@ -334,10 +334,7 @@ struct Engine : EngineBase {
         for (int q = 0; q < 16; ++q) p.cdiag[q] = layer == 0 ? 1.0 : cdiag1[q];
         p.E = E;
         p.num_cus = num_cus;
-        {
-            const char* ov = getenv(layer == 0 ? "SMX_SPLIT0" : "SMX_SPLIT1");
-            p.split_override = ov ? atoi(ov) : 0;
-        }
+        p.order = recv_order.p;
         return p;
     }
 
@@ -370,6 +367,8 @@ struct Engine : EngineBase {
         first_neigh.size_to((size_t)N + 1, s);
         scan_tmp.size_to((size_t)N / 1024 + 2, s);
         HIPCHK(launch_scan_exclusive(num_neigh, first_neigh.p, N, scan_tmp.p, s));
+        recv_order.size_to((size_t)N, s);
+        HIPCHK(launch_degree_order(N, first_neigh.p, recv_order.p, s));
         N_geo = N;
     }
     void build_type_groups(int N)
@@ -440,7 +439,7 @@ struct Engine : EngineBase {
         AggParams<F> p{};
         p.num_nodes = N; p.K = hm.K;
         p.first_neigh = first_neigh.p; p.node_types = node_types; p.neigh_types = neigh_types;
-        p.xyz = xyz; p.r = r; p.T = hm.T; p.spl_nodes = hm.spl_nodes; p.spl_h = hm.spl_h;
+        p.xyz = xyz; p.r = r; p.T = hm.T; p.spl_nodes = hm.spl_nodes; p.spl_h = hm.spl_h; p.spl_inv_h = 1.0 / hm.spl_h;
         p.num_edges = E;
         if (layer == 0) {
             p.gather = neigh_types; p.Hsrc = H0.p; p.tab = tab0.p; p.tabK = tabK0.p; p.pair_table = pair_table0.p;

@@ -33,6 +33,7 @@ struct AggParams {
     int T;
     int spl_nodes;
     double spl_h;
+    double spl_inv_h;         // 1 / spl_h
     const int* B_start;       // [NB+1] rows of the coupling list
     const int* B_lm1;
     const double* B_c;
@@ -68,7 +69,7 @@ struct SliceParams {
     double* fpart;     // bwd: [slices][E][3] partial forces
     long E;
     int num_cus;
-    int split_override;   // lanes per receiver, 0 = choose from the average degree
+    const int* order;     // [num_nodes] receivers by decreasing degree: entry 4t+q is row q of task t
 };
 template <typename F> hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s);
 template <typename F> hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s);
@@ -83,6 +84,8 @@ hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const in
 // ---------------------------------------------------------------------------
 // Integer list preparation
 hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums, hipStream_t s);  // out[n] = total
+// order[N]: receivers by decreasing degree
+hipError_t launch_degree_order(int N, const int* first_neigh, int* order, hipStream_t s);
 hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
                                int* slist, int* block_sums, hipStream_t s);
 hipError_t launch_type_groups(const int* node_types, int N, int T, int* tcount, int* tstart, int* cursor,

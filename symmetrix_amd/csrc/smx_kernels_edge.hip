@@ -101,14 +101,13 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
         if (lane < nE) {
             const int e = eb + lane;
             const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
-            const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
+            const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
             double Y[16];
             sph_l3(dz * inv, dx * inv, dy * inv, Y);
 #pragma unroll
             for (int q = 0; q < 16; ++q) Yt[lane * 16 + q] = Y[q];
             const double r = a.r[e];
-            int n = (int)(r / a.spl_h);
-            n = min(max(n, 0), a.spl_nodes - 2);
+            const int n = spline_interval(r, a.spl_inv_h, a.spl_nodes - 2);
             xs[lane] = r - a.spl_h * n;
             const int tbl = a.pair_table[pair_index(a.T, ti, a.neigh_types[e])];
             rows[lane] = tbl * (a.spl_nodes - 1) + n;
@@ -224,13 +223,13 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
         if (lane < nE) {
             const int e = eb + lane;
             const double dx = a.xyz[3 * (size_t)e], dy = a.xyz[3 * (size_t)e + 1], dz = a.xyz[3 * (size_t)e + 2];
-            const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
+            const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
             sph_l3_grad_store<16>(dz * inv, dx * inv, dy * inv, inv, Yt + lane * 64);
             const double r = a.r[e];
             // radial direction as the reference forms it: xyz / r with the caller's r
-            us[lane * 4] = dx / r; us[lane * 4 + 1] = dy / r; us[lane * 4 + 2] = dz / r;
-            int n = (int)(r / a.spl_h);
-            n = min(max(n, 0), a.spl_nodes - 2);
+            const double ir = rcp_pos(r);
+            us[lane * 4] = dx * ir; us[lane * 4 + 1] = dy * ir; us[lane * 4 + 2] = dz * ir;
+            const int n = spline_interval(r, a.spl_inv_h, a.spl_nodes - 2);
             xs[lane] = r - a.spl_h * n;
             const int tbl = a.pair_table[pair_index(a.T, ti, a.neigh_types[e])];
             rows[lane] = tbl * (a.spl_nodes - 1) + n;
@@ -449,7 +448,7 @@ __global__ void k_sph_harm(const double* xyz, long E, double* Y, double* Yg)
     const long e = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (e >= E) return;
     const double dx = xyz[3 * e], dy = xyz[3 * e + 1], dz = xyz[3 * e + 2];
-    const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
+    const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
     double y[16], G[3][16];
     sph_l3_grad(dz * inv, dx * inv, dy * inv, inv, y, G);
     for (int q = 0; q < 16; ++q) {

@@ -138,6 +138,42 @@ __global__ __launch_bounds__(1024) void k_type_groups(const int* node_types, int
         if (t >= 0 && t < T) perm[cnt[t] + atomicAdd(&cur[t], 1)] = i;
     }
 }
+// Receivers in order of decreasing degree (counting sort on min(degree, 1023), one block).  The edge
+// kernels hand consecutive entries to the rows of a wavefront, which then finish together; the order
+// inside a degree class is whatever the LDS atomics leave and has no influence on any result.
+__global__ __launch_bounds__(1024) void k_degree_order(int N, const int* first_neigh, int* order)
+{
+    __shared__ int start[1024];
+    __shared__ int cur[1024];
+    __shared__ int wsum[16];
+    const int tid = threadIdx.x;
+    start[tid] = 0; cur[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < N; i += 1024) {
+        const int d = min(first_neigh[i + 1] - first_neigh[i], 1023);
+        atomicAdd(&start[1023 - d], 1);
+    }
+    __syncthreads();
+    // exclusive scan of the 1024 counts: wavefront scans, then the 16 wavefront totals
+    const int c = start[tid];
+    int incl = c;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+        const int o = __shfl_up(incl, off, 64);
+        if ((tid & 63) >= off) incl += o;
+    }
+    if ((tid & 63) == 63) wsum[tid >> 6] = incl;
+    __syncthreads();
+    int base = 0;
+    for (int w = 0; w < (tid >> 6); ++w) base += wsum[w];
+    __syncthreads();
+    start[tid] = base + incl - c;
+    __syncthreads();
+    for (int i = tid; i < N; i += 1024) {
+        const int b = 1023 - min(first_neigh[i + 1] - first_neigh[i], 1023);
+        order[start[b] + atomicAdd(&cur[b], 1)] = i;
+    }
+}
 __global__ void k_check_range(const int* v, long n, int limit, int* flags)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -220,6 +256,12 @@ hipError_t launch_type_groups(const int* node_types, int N, int T, int* tcount, 
     // order inside a species group is left as placed: every output row of the products
     // that use this grouping is computed independently of its tile mates
     hipLaunchKernelGGL(k_type_groups, dim3(1), dim3(1024), 2 * T * sizeof(int), s, node_types, N, T, tstart, perm);
+    return hipGetLastError();
+}
+
+hipError_t launch_degree_order(int N, const int* first_neigh, int* order, hipStream_t s)
+{
+    if (N > 0) hipLaunchKernelGGL(k_degree_order, dim3(1), dim3(1024), 0, s, N, first_neigh, order);
     return hipGetLastError();
 }
 

@@ -73,8 +73,9 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
         copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
         __syncthreads();
         for (int task = wave_id; task < wave_tasks; task += wave_stride) {
-            const int i = task * 4 + (lane >> 4);
-            const bool live = i < a.num_nodes;
+            const int slot = task * 4 + (lane >> 4);
+            const bool live = slot < a.num_nodes;
+            const int i = live ? p.order[slot] : 0;
             int e0 = 0, e1 = 0, ti = 0;
             if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
             F acc[16][CPLN];
@@ -96,11 +97,10 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
                 const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
                 const double r = cu.r;
                 const int g = cu.g;
-                const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
+                const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
                 double Yd[16];
                 sph_l3(dz * inv, dx * inv, dy * inv, Yd);
-                int n = (int)(r / a.spl_h);
-                n = min(max(n, 0), R - 1);
+                const int n = spline_interval(r, a.spl_inv_h, R - 1);
                 const F x = (F)(r - a.spl_h * n);
                 const F* row = lds + (size_t)n * W + cs * CPLN;
                 F t[4][CPLN];
@@ -164,8 +164,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
         copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
         __syncthreads();
         for (int task = wave_id; task < wave_tasks; task += wave_stride) {
-            const int i = task * 4 + (lane >> 4);
-            const bool live = i < a.num_nodes;
+            const int slot = task * 4 + (lane >> 4);
+            const bool live = slot < a.num_nodes;
+            const int i = live ? p.order[slot] : 0;
             int e0 = 0, e1 = 0, ti = 0;
             if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
             F d[16][CPLN];
@@ -194,12 +195,11 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                     const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
                     const double r = cu.r;
                     const int g = cu.g;
-                    const double inv = 1.0 / sqrt(dx * dx + dy * dy + dz * dz);
+                    const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
                     const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
                     double Yd[16], gd[3][16];
                     sph_l3_g(ux, uy, uz, Yd, gd);
-                    int n = (int)(r / a.spl_h);
-                    n = min(max(n, 0), R - 1);
+                    const int n = spline_interval(r, a.spl_inv_h, R - 1);
                     const F x = (F)(r - a.spl_h * n);
                     const F* row = lds + (size_t)n * W + cs * CPLN;
                     F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
@@ -232,7 +232,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                     // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
                     // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
                     const double sr = (double)srad, lt = (double)lterm;
-                    const double ir = 1.0 / r;
+                    const double ir = rcp_pos(r);
                     fx = -(dx * ir * sr + ((double)wy - uy * lt) * inv);   // original x is permuted axis 1
                     fy = -(dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
                     fz = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0

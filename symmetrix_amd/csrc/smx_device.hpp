@@ -133,20 +133,33 @@ __device__ __forceinline__ int pair_index(int T, int a, int b)
     return (a <= b) ? a * (2 * T - a - 1) / 2 + b : b * (2 * T - b - 1) / 2 + a;
 }
 
-// value of the lane ROT places further round its 16-lane row (DPP row_ror: a VALU move, no LDS traffic)
-template <int ROT>
-__device__ __forceinline__ float row_rotate(float v)
+// DPP lane moves inside a 16-lane row (VALU moves, no LDS traffic).  Every lane of a row has a
+// source lane, so no previous value of the destination is needed (mov_dpp leaves it undefined, which
+// spares the register copy that update_dpp would make).
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v)
 {
-    return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), 0x120 + ROT, 0xf, 0xf, false));
+    const int b = __float_as_int(v);
+    return __int_as_float(__builtin_amdgcn_mov_dpp(b, CTRL, 0xf, 0xf, false));
 }
-template <int ROT>
-__device__ __forceinline__ double row_rotate(double v)
+template <int CTRL>
+__device__ __forceinline__ double dpp_move(double v)
 {
     const long long b = __double_as_longlong(v);
-    const int lo = __builtin_amdgcn_update_dpp(0, (int)(b & 0xffffffffll), 0x120 + ROT, 0xf, 0xf, false);
-    const int hi = __builtin_amdgcn_update_dpp(0, (int)(b >> 32), 0x120 + ROT, 0xf, 0xf, false);
+    const int l = (int)(b & 0xffffffffll), h = (int)(b >> 32);
+    const int lo = __builtin_amdgcn_mov_dpp(l, CTRL, 0xf, 0xf, false);
+    const int hi = __builtin_amdgcn_mov_dpp(h, CTRL, 0xf, 0xf, false);
     return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
+// value of the lane ROT places further round its 16-lane row (row_ror)
+template <int ROT, typename T>
+__device__ __forceinline__ T row_rotate(T v) { return dpp_move<0x120 + ROT>(v); }
+// value of the neighbouring lane (lane ^ 1): quad_perm [1,0,3,2]
+template <typename T>
+__device__ __forceinline__ T lane_xor1(T v) { return dpp_move<0xB1>(v); }
+// value of lane ^ 2: quad_perm [2,3,0,1]
+template <typename T>
+__device__ __forceinline__ T lane_xor2(T v) { return dpp_move<0x4E>(v); }
 // sum over the lanes of a 16-lane row whose index agrees modulo CL (CL = 1, 2, 4 or 8)
 template <int CL, typename T>
 __device__ __forceinline__ T row_sum_strided(T v)

@@ -238,10 +238,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                     fz = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
                 }
                 // channels of the slice are spread over CL adjacent lanes: add their partial forces
-#pragma unroll
-                for (int off = 1; off < CL; off <<= 1) {
-                    fx += __shfl_xor(fx, off, 64); fy += __shfl_xor(fy, off, 64); fz += __shfl_xor(fz, off, 64);
-                }
+                static_assert(CL <= 4, "the partner lanes of an edge are reached with quad permutes");
+                if constexpr (CL >= 2) { fx += lane_xor1(fx); fy += lane_xor1(fy); fz += lane_xor1(fz); }
+                if constexpr (CL >= 4) { fx += lane_xor2(fx); fy += lane_xor2(fy); fz += lane_xor2(fz); }
                 if (on && cs == 0) {
                     fpart[3 * (size_t)e] = fx; fpart[3 * (size_t)e + 1] = fy; fpart[3 * (size_t)e + 2] = fz;
                 }

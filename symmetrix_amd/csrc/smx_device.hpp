@@ -160,6 +160,9 @@ __device__ __forceinline__ T lane_xor1(T v) { return dpp_move<0xB1>(v); }
 // value of lane ^ 2: quad_perm [2,3,0,1]
 template <typename T>
 __device__ __forceinline__ T lane_xor2(T v) { return dpp_move<0x4E>(v); }
+// value of the lane mirrored inside its group of eight (lane i <-> 7 - i): row_half_mirror
+template <typename T>
+__device__ __forceinline__ T half_mirror(T v) { return dpp_move<0x141>(v); }
 // sum over the lanes of a 16-lane row whose index agrees modulo CL (CL = 1, 2, 4 or 8)
 template <int CL, typename T>
 __device__ __forceinline__ T row_sum_strided(T v)

@@ -45,6 +45,19 @@ __device__ __forceinline__ EdgeGeo load_edge(const AggParams<F>& a, int e)
     return q;
 }
 
+// Scheduling fences without instructions: what is computed from vx, vy, vz after order_l cannot start
+// before the five sums are final; pin_value ends the live range of an accumulation's operands here.
+template <typename F>
+__device__ __forceinline__ void order_l(F& s0, F& s1, F& s2, F& s3, F& s4, double& vx, double& vy, double& vz)
+{
+    asm volatile("" : "+v"(s0), "+v"(s1), "+v"(s2), "+v"(s3), "+v"(s4), "+v"(vx), "+v"(vy), "+v"(vz));
+}
+template <typename F>
+__device__ __forceinline__ void pin_value(F& v)
+{
+    asm volatile("" : "+v"(v));
+}
+
 // ---------------------------------------------------------------------------
 // Lane mapping of both kernels.  A wavefront works on four receivers at a time,
 // one per 16-lane row.  Inside a row, CL lanes share an edge and split the CH
@@ -197,18 +210,28 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                     const int g = cu.g;
                     const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
                     const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
-                    double Yd[16], gd[3][16];
-                    sph_l3_g(ux, uy, uz, Yd, gd);
                     const int n = spline_interval(r, a.spl_inv_h, R - 1);
                     const F x = (F)(r - a.spl_h * n);
                     const F* row = lds + (size_t)n * W + cs * CPLN;
                     F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
+                    F h[CPLN], mg[CPLN];
 #pragma unroll
-                    for (int c = 0; c < CPLN; ++c) {
-                        const F h = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)];
-                        F mg = F(0);
+                    for (int c = 0; c < CPLN; ++c) { h[c] = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)]; mg[c] = F(0); }
+                    // One order l at a time: its harmonics are formed, used for all channels of the lane and
+                    // dropped; the fence keeps the next order's harmonics from being formed early (all 16
+                    // with their derivatives would hold 128 registers).
+                    double vx = ux, vy = uy, vz = uz;
+                    static_for<0, 4>([&](auto lc) {
+                        constexpr int l = decltype(lc)::value;
+                        F Yl[2 * l + 1], g0[2 * l + 1], g1[2 * l + 1], g2[2 * l + 1];
+                        static_for<0, 2 * l + 1>([&](auto mc) {
+                            constexpr int m = decltype(mc)::value;
+                            double y, a0, a1, a2;
+                            ylm_g<l * l + m>(vx, vy, vz, y, a0, a1, a2);
+                            Yl[m] = (F)y; g0[m] = (F)a0; g1[m] = (F)a1; g2[m] = (F)a2;
+                        });
 #pragma unroll
-                        for (int l = 0; l < 4; ++l) {
+                        for (int c = 0; c < CPLN; ++c) {
                             const F c0 = row[(0 * 4 + l) * CH + c], c1 = row[(1 * 4 + l) * CH + c];
                             const F c2 = row[(2 * 4 + l) * CH + c], c3 = row[(3 * 4 + l) * CH + c];
                             const F Rv = c0 + x * (c1 + x * (c2 + x * c3));
@@ -216,18 +239,24 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                             F ul = F(0), v0 = F(0), v1 = F(0), v2 = F(0);
 #pragma unroll
                             for (int m = 0; m < 2 * l + 1; ++m) {
-                                const int q = l * l + m;
-                                const F dd = d[q][c];
-                                ul += dd * (F)Yd[q];
-                                v0 += dd * (F)gd[0][q]; v1 += dd * (F)gd[1][q]; v2 += dd * (F)gd[2][q];
+                                const F dd = d[l * l + m][c];
+                                ul += dd * Yl[m];
+                                v0 += dd * g0[m]; v1 += dd * g1[m]; v2 += dd * g2[m];
                             }
-                            const F Rh = Rv * h;
-                            srad += Rd * h * ul;
+                            const F Rh = Rv * h[c];
+                            srad += Rd * h[c] * ul;
                             wx += Rh * v0; wy += Rh * v1; wz += Rh * v2;
                             lterm += Rh * ul * F(l);
-                            mg += Rv * ul;
+                            mg[c] += Rv * ul;
                         }
-                        if (a.msg && kc + c < K) a.msg[(size_t)e * K + kc + c] = mg;
+                        order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
+#pragma unroll
+                        for (int c = 0; c < CPLN; ++c) pin_value(mg[c]);
+                    });
+                    if (a.msg) {
+#pragma unroll
+                        for (int c = 0; c < CPLN; ++c)
+                            if (kc + c < K) a.msg[(size_t)e * K + kc + c] = mg[c];
                     }
                     // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
                     // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
@@ -238,9 +267,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                     fz = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
                 }
                 // channels of the slice are spread over CL adjacent lanes: add their partial forces
-                static_assert(CL <= 4, "the partner lanes of an edge are reached with quad permutes");
                 if constexpr (CL >= 2) { fx += lane_xor1(fx); fy += lane_xor1(fy); fz += lane_xor1(fz); }
                 if constexpr (CL >= 4) { fx += lane_xor2(fx); fy += lane_xor2(fy); fz += lane_xor2(fz); }
+                if constexpr (CL >= 8) { fx += half_mirror(fx); fy += half_mirror(fy); fz += half_mirror(fz); }
                 if (on && cs == 0) {
                     fpart[3 * (size_t)e] = fx; fpart[3 * (size_t)e + 1] = fy; fpart[3 * (size_t)e + 2] = fz;
                 }
@@ -258,11 +287,9 @@ __global__ void k_fpart_reduce(long n3, int nslices, const double* fpart, double
     forces[t] = s;
 }
 
-template <typename F, int CH, bool BWD>
-hipError_t launch_slice_t(const SliceParams<F>& p, hipStream_t s)
+template <typename F, int CH, int CL, int BT, bool BWD>
+hipError_t launch_slice_cfg(const SliceParams<F>& p, hipStream_t s)
 {
-    constexpr int BT = 512;
-    constexpr int CL = 2;
     const int S = (p.a.K + CH - 1) / CH;
     const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F);
     const int waves_per_block = BT / 64;
@@ -281,6 +308,16 @@ hipError_t launch_slice_t(const SliceParams<F>& p, hipStream_t s)
     }
     hipLaunchKernelGGL(kern, grid, dim3(BT), lds, s, p);
     return hipGetLastError();
+}
+
+// Four lanes per edge and twelve wavefronts per block measured best for both directions and both
+// precisions: the kernels wait on dependent LDS reads and arithmetic chains, and a third wavefront
+// per SIMD (168 registers each) hides more of that than wider per-lane work does.
+template <typename F, int CH, bool BWD>
+hipError_t launch_slice_t(const SliceParams<F>& p, hipStream_t s)
+{
+    if constexpr (CH % 4 == 0) return launch_slice_cfg<F, CH, 4, 768, BWD>(p, s);
+    else return launch_slice_cfg<F, CH, 2, 512, BWD>(p, s);
 }
 
 }  // namespace

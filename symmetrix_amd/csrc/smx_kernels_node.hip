@@ -308,19 +308,34 @@ template hipError_t launch_convert<float, float>(const float*, float*, long, hip
 // P = sum_v x_v * (their partial sum).
 namespace {
 constexpr int POLY_BLOCK = 128;
-constexpr int POLY_NB = 2;       // atoms per thread
+// Atoms per thread: as many as fill one 16-byte LDS word, so that one ds_read_b128 brings a variable of
+// all of them and every loaded coefficient serves them all.  (Twice as many was measured slower: fewer
+// blocks than the chip holds at once.)
+template <typename F> constexpr int poly_nb() { return 16 / (int)sizeof(F); }
+template <typename F, int N>
+struct alignas(16) PolyVec {
+    F v[N];
+};
+
+// POLY_VG groups of POLY_BLOCK threads share the variables of a block in LDS; group g walks the lists of
+// the variables v = g, g + POLY_VG, ...  A block is latency bound (every list entry needs a coefficient
+// from L2), so spreading the 16 lists of an atom group over four times as many wavefronts shortens the
+// kernel by nearly that factor.
+constexpr int POLY_VG = 4;
 
 template <typename F>
-__global__ __launch_bounds__(POLY_BLOCK) void k_poly(const PolyParams<F> a)
+__global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<F> a)
 {
-    __shared__ F X[POLY_NB][17][POLY_BLOCK];
-    const int tid = threadIdx.x;
-    // species segment and pair of atoms of this block row
+    constexpr int NB = poly_nb<F>();
+    __shared__ PolyVec<F, NB> X[17][POLY_BLOCK];
+    __shared__ PolyVec<F, NB> fsum[POLY_VG][POLY_BLOCK];
+    const int tid = threadIdx.x % POLY_BLOCK, vg = threadIdx.x / POLY_BLOCK;
+    // species segment and group of atoms of this block row
     const int kblocks = (a.K + POLY_BLOCK - 1) / POLY_BLOCK;
     int type = -1, grp = blockIdx.x / kblocks, seg0 = 0, seg_n = 0;
     for (int t = 0; t < a.T; ++t) {
         const int n_t = a.tstart[t + 1] - a.tstart[t];
-        const int groups = (n_t + POLY_NB - 1) / POLY_NB;
+        const int groups = (n_t + NB - 1) / NB;
         if (grp < groups) { type = t; seg0 = a.tstart[t]; seg_n = n_t; break; }
         grp -= groups;
     }
@@ -328,59 +343,79 @@ __global__ __launch_bounds__(POLY_BLOCK) void k_poly(const PolyParams<F> a)
     const int k = (blockIdx.x % kblocks) * POLY_BLOCK + tid;
     const bool klive = k < a.K;
     const int kk = klive ? k : a.K - 1;
-    int node[POLY_NB];
-    bool nlive[POLY_NB];
+    int node[NB];
+    bool nlive[NB];
 #pragma unroll
-    for (int b = 0; b < POLY_NB; ++b) {
-        const int j = grp * POLY_NB + b;
+    for (int b = 0; b < NB; ++b) {
+        const int j = grp * NB + b;
         nlive[b] = j < seg_n;
         node[b] = a.perm[seg0 + (nlive[b] ? j : seg_n - 1)];
-#pragma unroll
-        for (int q = 0; q < 16; ++q) X[b][q][tid] = a.A[((size_t)node[b] * 16 + q) * a.K + kk];
-        X[b][16][tid] = F(1);
     }
-    // a thread reads back only its own columns: no barrier needed
+    for (int q = vg; q < 17; q += POLY_VG) {
+        PolyVec<F, NB> x;
+#pragma unroll
+        for (int b = 0; b < NB; ++b) x.v[b] = q < 16 ? a.A[((size_t)node[b] * 16 + q) * a.K + kk] : F(1);
+        X[q][tid] = x;
+    }
+    __syncthreads();
     for (int pl = 0; pl < a.NP; ++pl) {
         const int4* pk = a.packed[pl];
         const int* nch = a.chunks[pl];
         const F* coef = a.coef[pl] + (size_t)type * (a.num_entries[pl] + 1) * a.K + kk;
-        F f[POLY_NB];
+        F f[NB];
 #pragma unroll
-        for (int b = 0; b < POLY_NB; ++b) f[b] = F(0);
-        int4 cur = pk[0];
-        int c = 0;
+        for (int b = 0; b < NB; ++b) f[b] = F(0);
+        int c = 0;   // first chunk of variable v
         for (int v = 0; v < 16; ++v) {
-            F g[POLY_NB];
+            const int n0 = nch[2 * v], n1 = nch[2 * v + 1];
+            if (v % POLY_VG == vg) {
+                F g[NB];
 #pragma unroll
-            for (int b = 0; b < POLY_NB; ++b) g[b] = F(0);
-#pragma unroll
-            for (int part = 0; part < 2; ++part) {
-                const int n = nch[2 * v + part];
-                for (int j = 0; j < n; ++j) {
-                    const int4 nxt = pk[c + 1];   // next chunk's indices are in flight while this one is used
+                for (int b = 0; b < NB; ++b) g[b] = F(0);
+                int4 cur = pk[c];
+                for (int j = 0; j < n0 + n1; ++j) {
+                    const int4 nxt = pk[c + j + 1];   // next chunk's indices are in flight while this one is used
                     const int e4[4] = {cur.x, cur.y, cur.z, cur.w};
 #pragma unroll
                     for (int q = 0; q < 4; ++q) {
                         const int mono = e4[q] & 0xffff, ia = (e4[q] >> 16) & 0xff, ib = (e4[q] >> 24) & 0xff;
                         const F w = coef[(size_t)mono * a.K];
+                        const PolyVec<F, NB> xa = X[ia][tid], xb = X[ib][tid];
 #pragma unroll
-                        for (int b = 0; b < POLY_NB; ++b) g[b] += w * (X[b][ia][tid] * X[b][ib][tid]);
+                        for (int b = 0; b < NB; ++b) g[b] += w * (xa.v[b] * xb.v[b]);
                     }
                     cur = nxt;
-                    ++c;
-                }
-                if (part == 0) {
+                    if (j == n0 - 1) {
+                        // the monomials that start with v are done: their sum times x_v is v's share of P
+                        const PolyVec<F, NB> xv = X[v][tid];
 #pragma unroll
-                    for (int b = 0; b < POLY_NB; ++b) f[b] += X[b][v][tid] * g[b];
+                        for (int b = 0; b < NB; ++b) f[b] += xv.v[b] * g[b];
+                    }
                 }
+#pragma unroll
+                for (int b = 0; b < NB; ++b)
+                    if (klive && nlive[b]) a.M_grad[(((size_t)node[b] * a.NP + pl) * 16 + v) * a.K + k] = g[b];
             }
-#pragma unroll
-            for (int b = 0; b < POLY_NB; ++b)
-                if (klive && nlive[b]) a.M_grad[(((size_t)node[b] * a.NP + pl) * 16 + v) * a.K + k] = g[b];
+            c += n0 + n1;
         }
+        // P = sum of the groups' shares, added in group order
+        {
+            PolyVec<F, NB> fv;
 #pragma unroll
-        for (int b = 0; b < POLY_NB; ++b)
-            if (klive && nlive[b]) a.M[((size_t)node[b] * a.NP + pl) * a.K + k] = f[b];
+            for (int b = 0; b < NB; ++b) fv.v[b] = f[b];
+            fsum[vg][tid] = fv;
+        }
+        __syncthreads();
+        if (vg == 0) {
+#pragma unroll
+            for (int b = 0; b < NB; ++b) {
+                F t = F(0);
+#pragma unroll
+                for (int g2 = 0; g2 < POLY_VG; ++g2) t += fsum[g2][tid].v[b];
+                if (klive && nlive[b]) a.M[((size_t)node[b] * a.NP + pl) * a.K + k] = t;
+            }
+        }
+        __syncthreads();
     }
 }
 
@@ -405,8 +440,8 @@ hipError_t launch_poly(const PolyParams<F>& p, hipStream_t s)
 {
     if (p.num_nodes <= 0) return hipSuccess;
     const int kblocks = (p.K + POLY_BLOCK - 1) / POLY_BLOCK;
-    const unsigned groups = (unsigned)((p.num_nodes + POLY_NB - 1) / POLY_NB + p.T);
-    hipLaunchKernelGGL(k_poly<F>, dim3(groups * kblocks), dim3(POLY_BLOCK), 0, s, p);
+    const unsigned groups = (unsigned)((p.num_nodes + poly_nb<F>() - 1) / poly_nb<F>() + p.T);
+    hipLaunchKernelGGL(k_poly<F>, dim3(groups * kblocks), dim3(POLY_BLOCK * POLY_VG), 0, s, p);
     return hipGetLastError();
 }
 template hipError_t launch_poly<double>(const PolyParams<double>&, hipStream_t);

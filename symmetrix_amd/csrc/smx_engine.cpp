@@ -279,9 +279,9 @@ struct Engine : EngineBase {
         if ((size_t)prop.sharedMemPerBlockOptin > lds_cap) lds_cap = prop.sharedMemPerBlockOptin;
         if (lds_cap > 160 * 1024) lds_cap = 160 * 1024;
         for (int CH = sizeof(F) == 8 ? 4 : 8; CH >= 2; CH /= 2) {
-            int W = 16 * CH;
-            const int step = 16 / (int)sizeof(F);
-            while (((W * (int)sizeof(F) / 4) / 4) % 2 == 0) W += step;   // rows land on different LDS bank groups
+            // row = [4 coefficients][4 paths][CH channels], padded as the kernels of this precision want it
+            const int W = slice_row_elements<F>(CH);
+            if (W == 0) continue;
             if ((size_t)R * W * sizeof(F) > lds_cap) continue;
             const int S = (Kc + CH - 1) / CH;
             std::vector<F> buf((size_t)S * U * R * W, F(0));

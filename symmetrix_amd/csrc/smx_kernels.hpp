@@ -71,6 +71,8 @@ struct SliceParams {
     int num_cus;
     const int* order;     // [num_nodes] receivers by decreasing degree: entry 4t+q is row q of task t
 };
+// padded row length W (elements) of the per-slice table for CH channels, 0 if the kernels cannot take that CH
+template <typename F> int slice_row_elements(int CH);
 template <typename F> hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s);
 template <typename F> hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s);
 // forces (+)= sum over slices of fpart, slices added in ascending order

@@ -58,6 +58,22 @@ __device__ __forceinline__ void pin_value(F& v)
     asm volatile("" : "+v"(v));
 }
 
+// Single precision: the kernels wait on the LDS, and reading the paths in an order rotated by the lane's edge
+// slot removes the bank conflicts between the edges served in one LDS cycle (rows are multiples of 128 bytes
+// there, the four paths of a coefficient lie 32 bytes apart).  Double precision: the kernels wait on vector
+// issue, the selects that undo the rotation cost more than the conflicts; rows are padded to an odd number of
+// 16-byte words instead.  The host lays the table out accordingly (slice_row_elements).
+template <typename F> __host__ __device__ constexpr bool slice_rotates() { return sizeof(F) == 4; }
+
+// v[l] <- v[(l - rot) & 3] for rot = 0..3, as two conditional rotations by one and by two
+template <typename F>
+__device__ __forceinline__ void unrotate4(F* v, int rot)
+{
+    const bool r1 = rot & 1, r2 = rot & 2;
+    const F a0 = r1 ? v[3] : v[0], a1 = r1 ? v[0] : v[1], a2 = r1 ? v[1] : v[2], a3 = r1 ? v[2] : v[3];
+    v[0] = r2 ? a2 : a0; v[1] = r2 ? a3 : a1; v[2] = r2 ? a0 : a2; v[3] = r2 ? a1 : a3;
+}
+
 // ---------------------------------------------------------------------------
 // Lane mapping of both kernels.  A wavefront works on four receivers at a time,
 // one per 16-lane row.  Inside a row, CL lanes share an edge and split the CH
@@ -78,6 +94,10 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int sub = lane & 15, e_sub = sub / CL, cs = sub % CL;
     const int kc = slice * CH + cs * CPLN;                 // first channel of this lane
+    const int rot = slice_rotates<F>() ? (e_sub & 3) : 0;
+    int poff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) poff[i] = ((i + rot) & 3) * CH;
     const int wave_tasks = (a.num_nodes + 3) / 4;
     const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
 
@@ -116,22 +136,24 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
                 const int n = spline_interval(r, a.spl_inv_h, R - 1);
                 const F x = (F)(r - a.spl_h * n);
                 const F* row = lds + (size_t)n * W + cs * CPLN;
-                F t[4][CPLN];
+                // step i reads path (i + rot) & 3, rot = this lane's edge slot in single precision, else 0
+                F t[CPLN][4];
 #pragma unroll
                 for (int c = 0; c < CPLN; ++c) {
                     const F h = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)];
 #pragma unroll
-                    for (int l = 0; l < 4; ++l) {
-                        const F c0 = row[(0 * 4 + l) * CH + c], c1 = row[(1 * 4 + l) * CH + c];
-                        const F c2 = row[(2 * 4 + l) * CH + c], c3 = row[(3 * 4 + l) * CH + c];
-                        t[l][c] = (c0 + x * (c1 + x * (c2 + x * c3))) * h;
+                    for (int i = 0; i < 4; ++i) {
+                        const F* rp = row + poff[i] + c;
+                        const F c0 = rp[0], c1 = rp[4 * CH], c2 = rp[8 * CH], c3 = rp[12 * CH];
+                        t[c][i] = (c0 + x * (c1 + x * (c2 + x * c3))) * h;
                     }
+                    if constexpr (slice_rotates<F>()) unrotate4(t[c], rot);
                 }
 #pragma unroll
                 for (int q = 0; q < 16; ++q) {
                     const F y = (F)Yd[q];
 #pragma unroll
-                    for (int c = 0; c < CPLN; ++c) acc[q][c] += t[lm_l(q)][c] * y;
+                    for (int c = 0; c < CPLN; ++c) acc[q][c] += t[c][lm_l(q)] * y;
                 }
             }
             // add up the lanes of the row that hold the same channels (they took alternate edges)
@@ -168,6 +190,10 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int sub = lane & 15, e_sub = sub / CL, cs = sub % CL;
     const int kc = slice * CH + cs * CPLN;
+    const int rot = slice_rotates<F>() ? (e_sub & 3) : 0;
+    int poff[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) poff[i] = ((i + rot) & 3) * CH;
     const int wave_tasks = (a.num_nodes + 3) / 4;
     const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
     double* fpart = p.fpart + (size_t)slice * p.E * 3;
@@ -214,9 +240,20 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                     const F x = (F)(r - a.spl_h * n);
                     const F* row = lds + (size_t)n * W + cs * CPLN;
                     F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
-                    F h[CPLN], mg[CPLN];
+                    F h[CPLN], mg[CPLN], Rv[CPLN][4], Rd[CPLN][4];
 #pragma unroll
-                    for (int c = 0; c < CPLN; ++c) { h[c] = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)]; mg[c] = F(0); }
+                    for (int c = 0; c < CPLN; ++c) {
+                        h[c] = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)]; mg[c] = F(0);
+                        // paths read in the rotated order of this lane's edge slot (see the forward kernel)
+#pragma unroll
+                        for (int i = 0; i < 4; ++i) {
+                            const F* rp = row + poff[i] + c;
+                            const F c0 = rp[0], c1 = rp[4 * CH], c2 = rp[8 * CH], c3 = rp[12 * CH];
+                            Rv[c][i] = c0 + x * (c1 + x * (c2 + x * c3));
+                            Rd[c][i] = c1 + x * (F(2) * c2 + F(3) * x * c3);
+                        }
+                        if constexpr (slice_rotates<F>()) { unrotate4(Rv[c], rot); unrotate4(Rd[c], rot); }
+                    }
                     // One order l at a time: its harmonics are formed, used for all channels of the lane and
                     // dropped; the fence keeps the next order's harmonics from being formed early (all 16
                     // with their derivatives would hold 128 registers).
@@ -232,10 +269,6 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                         });
 #pragma unroll
                         for (int c = 0; c < CPLN; ++c) {
-                            const F c0 = row[(0 * 4 + l) * CH + c], c1 = row[(1 * 4 + l) * CH + c];
-                            const F c2 = row[(2 * 4 + l) * CH + c], c3 = row[(3 * 4 + l) * CH + c];
-                            const F Rv = c0 + x * (c1 + x * (c2 + x * c3));
-                            const F Rd = c1 + x * (F(2) * c2 + F(3) * x * c3);
                             F ul = F(0), v0 = F(0), v1 = F(0), v2 = F(0);
 #pragma unroll
                             for (int m = 0; m < 2 * l + 1; ++m) {
@@ -243,11 +276,11 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                                 ul += dd * Yl[m];
                                 v0 += dd * g0[m]; v1 += dd * g1[m]; v2 += dd * g2[m];
                             }
-                            const F Rh = Rv * h[c];
-                            srad += Rd * h[c] * ul;
+                            const F Rh = Rv[c][l] * h[c];
+                            srad += Rd[c][l] * h[c] * ul;
                             wx += Rh * v0; wy += Rh * v1; wz += Rh * v2;
                             lterm += Rh * ul * F(l);
-                            mg[c] += Rv * ul;
+                            mg[c] += Rv[c][l] * ul;
                         }
                         order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
 #pragma unroll
@@ -344,6 +377,17 @@ hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s)
     default: return hipErrorInvalidValue;
     }
 }
+template <typename F>
+int slice_row_elements(int CH)
+{
+    int W = 16 * CH;
+    if (slice_rotates<F>()) return (W * (int)sizeof(F)) % 128 == 0 ? W : 0;
+    const int step = 16 / (int)sizeof(F);
+    while (((W * (int)sizeof(F) / 4) / 4) % 2 == 0) W += step;   // rows start on different 16-byte bank groups
+    return W;
+}
+template int slice_row_elements<double>(int);
+template int slice_row_elements<float>(int);
 template hipError_t launch_slice_fwd<double>(const SliceParams<double>&, hipStream_t);
 template hipError_t launch_slice_fwd<float>(const SliceParams<float>&, hipStream_t);
 template hipError_t launch_slice_bwd<double>(const SliceParams<double>&, hipStream_t);

@@ -419,19 +419,31 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
     }
 }
 
-template <typename F>
-__global__ void k_poly_reverse(long total, int NP, int K, const F* M_grad, const F* M_adj, F* A_adj)
+template <typename F, int V>
+struct alignas(sizeof(F) * V > 16 ? 16 : sizeof(F) * V) RevVec {
+    F v[V];
+};
+// four consecutive channels per thread when K allows 16/32-byte accesses (V = 4), else one
+template <typename F, int V>
+__global__ void k_poly_reverse(long total_v, int NP, int K, const F* M_grad, const F* M_adj, F* A_adj)
 {
-    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;  // over [N][16][K]
-    if (idx >= total) return;
-    const int k = (int)(idx % K);
-    const long t = idx / K;
+    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;  // over [N][16][K / V]
+    if (idx >= total_v) return;
+    const int KV = K / V;
+    const int kq = (int)(idx % KV) * V;
+    const long t = idx / KV;
     const int lm = (int)(t % 16);
     const long i = t / 16;
-    F s = F(0);
-    for (int p = 0; p < NP; ++p)
-        s += M_grad[((i * NP + p) * 16 + lm) * K + k] * M_adj[(i * NP + p) * K + k];
-    A_adj[idx] = s;
+    RevVec<F, V> s;
+#pragma unroll
+    for (int j = 0; j < V; ++j) s.v[j] = F(0);
+    for (int p = 0; p < NP; ++p) {
+        const RevVec<F, V> g = *reinterpret_cast<const RevVec<F, V>*>(M_grad + ((i * NP + p) * 16 + lm) * K + kq);
+        const RevVec<F, V> m = *reinterpret_cast<const RevVec<F, V>*>(M_adj + (i * NP + p) * K + kq);
+#pragma unroll
+        for (int j = 0; j < V; ++j) s.v[j] += g.v[j] * m.v[j];
+    }
+    *reinterpret_cast<RevVec<F, V>*>(A_adj + (i * 16 + lm) * K + kq) = s;
 }
 }  // namespace
 
@@ -450,8 +462,14 @@ template hipError_t launch_poly<float>(const PolyParams<float>&, hipStream_t);
 template <typename F>
 hipError_t launch_poly_reverse(int N, int NP, int K, const F* M_grad, const F* M_adj, F* A_adj, hipStream_t s)
 {
-    const long total = (long)N * 16 * K;
-    if (total > 0) hipLaunchKernelGGL(k_poly_reverse<F>, dim3(nblk(total, 256)), dim3(256), 0, s, total, NP, K, M_grad, M_adj, A_adj);
+    if (N <= 0) return hipSuccess;
+    if (K % 4 == 0) {
+        const long total = (long)N * 16 * (K / 4);
+        hipLaunchKernelGGL((k_poly_reverse<F, 4>), dim3(nblk(total, 256)), dim3(256), 0, s, total, NP, K, M_grad, M_adj, A_adj);
+    } else {
+        const long total = (long)N * 16 * K;
+        hipLaunchKernelGGL((k_poly_reverse<F, 1>), dim3(nblk(total, 256)), dim3(256), 0, s, total, NP, K, M_grad, M_adj, A_adj);
+    }
     return hipGetLastError();
 }
 template hipError_t launch_poly_reverse<double>(int, int, int, const double*, const double*, double*, hipStream_t);

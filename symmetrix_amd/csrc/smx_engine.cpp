@@ -174,6 +174,7 @@ struct Engine : EngineBase {
     int N_geo = 0;
     DVec<int> first_neigh, recv_order, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
     int sender_rows = 0;
+    bool counters_zeroed = false;   // the sender counters were cleared by the fused node-list launch
 
     // ---- state (mace.hpp members)
     DVec<F> Phi0, A0, A0_adj, M0, M0_grad, M0_adj, H1, H1_adj, Phi1, dPhi1, A1, A1_adj, M1, M1_grad, M1_adj, msg;
@@ -385,7 +386,9 @@ struct Engine : EngineBase {
         s_count.size_to((size_t)2 * rows, s); s_start.size_to((size_t)rows + 1, s);
         s_list.size_to((size_t)E, s);
         scan_tmp.size_to((size_t)rows / 1024 + 2, s);
-        HIPCHK(launch_sender_lists(neigh_indices, (int)E, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p, s));
+        HIPCHK(launch_sender_lists(neigh_indices, (int)E, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p,
+                                   counters_zeroed ? 1 : 0, s));
+        counters_zeroed = false;
         sender_rows = rows;
     }
     // Host-path validation of what the reference leaves unchecked (mace.cpp:17-64 trusts
@@ -715,10 +718,23 @@ struct Engine : EngineBase {
         }
         stage_begin(ST_PREP);
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, on_device);
-        build_first_neigh(N);
         // range checks come before any kernel that uses these integers as indices
-        if (!on_device) validate(N, N);
-        build_type_groups(N);
+        if (on_device && N <= 65536) {
+            // one launch for first_neigh, degree order, species groups and the cleared sender counters
+            hipStream_t s = stream;
+            first_neigh.size_to((size_t)N + 1, s); recv_order.size_to((size_t)N, s);
+            t_start.size_to((size_t)hm.T + 1, s); t_perm.size_to((size_t)N, s);
+            s_count.size_to((size_t)2 * N, s); s_start.size_to((size_t)N + 1, s);
+            scan_tmp.size_to((size_t)N / 1024 + 2, s);
+            HIPCHK(launch_node_lists(num_neigh, N, first_neigh.p, recv_order.p, node_types, hm.T, t_start.p, t_perm.p,
+                                     s_count.p, 2L * N, s));
+            N_geo = N;
+            counters_zeroed = true;
+        } else {
+            build_first_neigh(N);
+            if (!on_device) validate(N, N);
+            build_type_groups(N);
+        }
         sender_rows = -1;
         build_sender_lists(N);
         stage_end(ST_PREP);
@@ -904,7 +920,7 @@ struct Engine : EngineBase {
                 rf_recv.upload(hr.data(), hr.size(), s);
                 HIPCHK(hipStreamSynchronize(s));
                 rf_rstart.size_to((size_t)num_atoms + 1, s); rf_rlist.size_to((size_t)E, s);
-                HIPCHK(launch_sender_lists(rf_recv.p, (int)E, num_atoms, rf_count.p, rf_rstart.p, rf_cursor.p, rf_rlist.p, scan_tmp.p, s));
+                HIPCHK(launch_sender_lists(rf_recv.p, (int)E, num_atoms, rf_count.p, rf_rstart.p, rf_cursor.p, rf_rlist.p, scan_tmp.p, 0, s));
                 rstart = rf_rstart.p; rlist = rf_rlist.p;
             } else {
                 if (num_atoms < N_geo) throw Error(SMX_EINVAL, "num_atoms is smaller than the number of receivers");
@@ -917,7 +933,7 @@ struct Engine : EngineBase {
                 HIPCHK(hipStreamSynchronize(s));
                 rstart = rf_rstart.p;
             }
-            HIPCHK(launch_sender_lists(rf_send.p, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, s));
+            HIPCHK(launch_sender_lists(rf_send.p, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, 0, s));
             rf_out.size_to((size_t)3 * num_atoms, s);
             HIPCHK(launch_force_scatter(num_atoms, rstart, rlist, rf_sstart.p, rf_slist.p, node_forces.p, rf_out.p, s));
             HIPCHK(hipMemcpyAsync(atom_forces, rf_out.p, (size_t)3 * num_atoms * sizeof(double), hipMemcpyDeviceToHost, s));

@@ -115,9 +115,9 @@ __global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows,
     }
 }
 // species groups in one block: LDS histogram, scan over the (few) species, placement
-__global__ __launch_bounds__(1024) void k_type_groups(const int* node_types, int N, int T, int* tstart, int* perm)
+__device__ void type_groups_body(const int* node_types, int N, int T, int* tstart, int* perm, int* sh)
 {
-    extern __shared__ int sh[];   // [T] counts, [T] cursors
+    // sh: [T] counts, [T] cursors
     int* cnt = sh;
     int* cur = sh + T;
     for (int t = threadIdx.x; t < T; t += blockDim.x) { cnt[t] = 0; cur[t] = 0; }
@@ -138,10 +138,15 @@ __global__ __launch_bounds__(1024) void k_type_groups(const int* node_types, int
         if (t >= 0 && t < T) perm[cnt[t] + atomicAdd(&cur[t], 1)] = i;
     }
 }
+__global__ __launch_bounds__(1024) void k_type_groups(const int* node_types, int N, int T, int* tstart, int* perm)
+{
+    extern __shared__ int sh[];
+    type_groups_body(node_types, N, T, tstart, perm, sh);
+}
 // Receivers in order of decreasing degree (counting sort on min(degree, 1023), one block).  The edge
 // kernels hand consecutive entries to the rows of a wavefront, which then finish together; the order
 // inside a degree class is whatever the LDS atomics leave and has no influence on any result.
-__global__ __launch_bounds__(1024) void k_degree_order(int N, const int* first_neigh, int* order)
+__device__ void degree_order_body(int N, const int* first_neigh, int* order)
 {
     __shared__ int start[1024];
     __shared__ int cur[1024];
@@ -174,6 +179,10 @@ __global__ __launch_bounds__(1024) void k_degree_order(int N, const int* first_n
         order[start[b] + atomicAdd(&cur[b], 1)] = i;
     }
 }
+__global__ __launch_bounds__(1024) void k_degree_order(int N, const int* first_neigh, int* order)
+{
+    degree_order_body(N, first_neigh, order);
+}
 __global__ void k_check_range(const int* v, long n, int limit, int* flags)
 {
     const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
@@ -200,7 +209,7 @@ inline unsigned nblk(long n, int bs) { return (unsigned)((n + bs - 1) / bs); }
 
 // whole scan in one block (tiles visited in order with a running carry): one launch
 // instead of three while the array is short
-__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_single(const int* in, int* out, int n)
+__device__ void scan_single_body(const int* in, int* out, int n)
 {
     int carry = 0;
     for (int b0 = 0; b0 < n; b0 += SCAN_BLOCK) {
@@ -213,7 +222,35 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_scan_single(const int* in, int* 
     }
     if (threadIdx.x == 0) out[n] = carry;
 }
+__global__ __launch_bounds__(SCAN_BLOCK) void k_scan_single(const int* in, int* out, int n)
+{
+    scan_single_body(in, out, n);
+}
+// The node-level lists of one evaluation in one launch (one block): first_neigh = exclusive scan of
+// num_neigh, receivers by decreasing degree, species groups, and the zeroing of `zero_n` counters that the
+// sender-list kernels count into.  Each part is the body of the stand-alone kernel of the same name.
+__global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists(const int* num_neigh, int N, int* first_neigh, int* order,
+                                                          const int* node_types, int T, int* tstart, int* perm,
+                                                          int* zero_p, long zero_n)
+{
+    extern __shared__ int sh[];
+    for (long i = threadIdx.x; i < zero_n; i += SCAN_BLOCK) zero_p[i] = 0;
+    scan_single_body(num_neigh, first_neigh, N);
+    __syncthreads();   // first_neigh, written by this block, is read back below
+    degree_order_body(N, first_neigh, order);
+    __syncthreads();
+    type_groups_body(node_types, N, T, tstart, perm, sh);
+}
 }  // namespace
+
+hipError_t launch_node_lists(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
+                             int* tstart, int* perm, int* zero_p, long zero_n, hipStream_t s)
+{
+    if (N <= 0 || N > 64 * SCAN_BLOCK || T <= 0) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_node_lists, dim3(1), dim3(SCAN_BLOCK), 2 * T * sizeof(int), s, num_neigh, N, first_neigh, order,
+                       node_types, T, tstart, perm, zero_p, zero_n);
+    return hipGetLastError();
+}
 
 hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums, hipStream_t s)
 {
@@ -229,10 +266,12 @@ hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums
 }
 
 hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
-                               int* slist, int* block_sums, hipStream_t s)
+                               int* slist, int* block_sums, int counters_are_zero, hipStream_t s)
 {
     if (rows <= 0) return hipSuccess;
-    if (cursor == count + rows) {
+    if (counters_are_zero) {
+        // k_node_lists has cleared them
+    } else if (cursor == count + rows) {
         hipLaunchKernelGGL(k_fill<int>, dim3(nblk(2L * rows, 256)), dim3(256), 0, s, count, 2L * rows, 0);
     } else {
         hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, count, (long)rows, 0);

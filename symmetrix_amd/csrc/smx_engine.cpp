@@ -174,6 +174,10 @@ struct Engine : EngineBase {
     int N_geo = 0;
     DVec<int> first_neigh, recv_order, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
     int sender_rows = 0;
+    // caller's output arrays of the running whole-pipeline call; the kernel that forms the final values writes
+    // them too and clears the pointer, otherwise a copy is enqueued at the end
+    double* energies_copy = nullptr;
+    double* forces_copy = nullptr;
     bool counters_zeroed = false;   // the sender counters were cleared by the fused node-list launch
 
     // ---- state (mace.hpp members)
@@ -613,7 +617,8 @@ struct Engine : EngineBase {
         g1.prob[0] = gemm_prob<double, double, double>(H2.p, k, 0, 0, hidden.p, 16, 0, 0, ro2_w1.p, 0, 0, 1, 0, k, 16, 1);
         HIPCHK((launch_gemm<double, double, double>(g1, stream)));
         HIPCHK(launch_readout<F>(N, k, nlm, node_types, E0.p, ro1.p, H1.p, hidden.p, ro2_w2.p, hm.readout_2_scale,
-                                 node_energies.p, zero_energies ? 1 : 0, stream));
+                                 node_energies.p, zero_energies ? 1 : 0, energies_copy, stream));
+        energies_copy = nullptr;
         auto g2 = gemm_base<double, double, double>(N, false);
         g2.nprob = 1;
         g2.prob[0] = gemm_prob<double, double, double>(hidden.p, 16, 0, 0, H2_adj.p, k, 0, 0, ro2_w1.p, 0, 0, 0, 0, 16, k, 1);
@@ -646,7 +651,7 @@ struct Engine : EngineBase {
             HIPCHK(launch_slice_bwd<F>(sp, stream));
             stage_end(ST_AGG1B);
             stage_begin(ST_FSUM1);
-            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, stream));
+            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
             stage_end(ST_FSUM1);
         } else {
             auto p = agg_params(1, N);
@@ -676,7 +681,8 @@ struct Engine : EngineBase {
             HIPCHK(launch_slice_bwd<F>(sp, stream));
             stage_end(ST_AGG0B);
             stage_begin(ST_FSUM0);
-            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, 1, stream));
+            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, 1, forces_copy, stream));
+            forces_copy = nullptr;
             stage_end(ST_FSUM0);
             return;
         }
@@ -697,7 +703,7 @@ struct Engine : EngineBase {
         stage_end(st_kernel);
         if (groups > 1) {
             stage_begin(st_sum);
-            HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, p.accumulate_forces, stream));
+            HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, p.accumulate_forces, nullptr, stream));
             stage_end(st_sum);
         }
     }
@@ -743,6 +749,7 @@ struct Engine : EngineBase {
         node_forces.size_to((size_t)3 * E, stream);
         if (N == 0) return;
 
+        energies_copy = d_energies; forces_copy = d_forces;
         stage_begin(ST_AGG0F); st_agg0_fwd(N); stage_end(ST_AGG0F);
         stage_begin(ST_A0LIN); st_A0_lin(N, false); stage_end(ST_A0LIN);
         stage_begin(ST_M0); st_poly(N, false); stage_end(ST_M0);
@@ -761,8 +768,9 @@ struct Engine : EngineBase {
         stage_begin(ST_REVA0LIN); st_A0_lin(N, true); stage_end(ST_REVA0LIN);
         st_agg0_bwd(N);
 
-        if (d_energies) HIPCHK(hipMemcpyAsync(d_energies, node_energies.p, (size_t)N * sizeof(double), hipMemcpyDeviceToDevice, stream));
-        if (d_forces && E) HIPCHK(hipMemcpyAsync(d_forces, node_forces.p, (size_t)3 * E * sizeof(double), hipMemcpyDeviceToDevice, stream));
+        if (energies_copy) HIPCHK(hipMemcpyAsync(energies_copy, node_energies.p, (size_t)N * sizeof(double), hipMemcpyDeviceToDevice, stream));
+        if (forces_copy && E) HIPCHK(hipMemcpyAsync(forces_copy, node_forces.p, (size_t)3 * E * sizeof(double), hipMemcpyDeviceToDevice, stream));
+        energies_copy = nullptr; forces_copy = nullptr;
     }
 
     // stage-level entry points (host arrays)
@@ -770,6 +778,7 @@ struct Engine : EngineBase {
                const double* x, const double* rr, long E_, int fa, int fb) override
     {
         const std::string s(name);
+        energies_copy = nullptr; forces_copy = nullptr;
         if (N < 0) throw Error(SMX_EINVAL, "negative num_nodes");
         if (hm.has_zbl || hm.A0_scaled || hm.A1_scaled)
             throw Error(SMX_EUNSUPPORTED, "models with ZBL or density normalisation are not implemented on the device yet");

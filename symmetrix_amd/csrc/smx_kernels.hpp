@@ -76,7 +76,9 @@ template <typename F> int slice_row_elements(int CH);
 template <typename F> hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s);
 template <typename F> hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s);
 // forces (+)= sum over slices of fpart, slices added in ascending order
-hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, hipStream_t s);
+// (`copy`, if not null, receives the same sums: the caller's output array of the whole-pipeline call)
+hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, double* copy,
+                               hipStream_t s);
 
 // H1_adj[j] (+)= sum over edges with sender j of msg[e], in ascending edge order.
 template <typename F>
@@ -165,7 +167,7 @@ hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p, hipStream_t s);
 template <typename F>
 hipError_t launch_readout(int N, int K, int num_LM, const int* node_types, const double* atomic_energies,
                           const double* w1, const F* H1, double* hidden_g, const double* w2, double scale,
-                          double* node_energies, int zero_energies, hipStream_t s);
+                          double* node_energies, int zero_energies, double* energies_copy, hipStream_t s);
 // H1_adj: zero everywhere (rows x num_LM x K), l=0 block of the first N rows = readout_1 weights
 template <typename F>
 hipError_t launch_seed_H1_adj(int rows, int N, int num_LM, int K, const double* w1, F* H1_adj, hipStream_t s);

@@ -520,7 +520,7 @@ namespace {
 template <typename F>
 __global__ void k_readout(int N, int K, int num_LM, const int* node_types, const double* E0, const double* w1,
                           const F* H1, double* hidden_g, const double* w2, double scale, double* node_energies,
-                          int zero_energies)
+                          int zero_energies, double* energies_copy)
 {
     // 16 threads per node: thread h owns hidden unit h
     const int i = blockIdx.x * (blockDim.x / 16) + threadIdx.x / 16;
@@ -540,7 +540,9 @@ __global__ void k_readout(int N, int K, int num_LM, const int* node_types, const
     for (int off = 8; off >= 1; off >>= 1) e += __shfl_xor(e, off, 64);
     if (h == 0) {
         const double base = zero_energies ? 0.0 : node_energies[i];
-        node_energies[i] = base + E0[node_types[i]] + e;
+        const double en = base + E0[node_types[i]] + e;
+        node_energies[i] = en;
+        if (energies_copy) energies_copy[i] = en;
     }
 }
 template <typename F>
@@ -559,15 +561,15 @@ __global__ void k_seed_H1_adj(long total, int N, int num_LM, int K, const double
 template <typename F>
 hipError_t launch_readout(int N, int K, int num_LM, const int* node_types, const double* atomic_energies,
                           const double* w1, const F* H1, double* hidden_g, const double* w2, double scale,
-                          double* node_energies, int zero_energies, hipStream_t s)
+                          double* node_energies, int zero_energies, double* energies_copy, hipStream_t s)
 {
     if (N > 0)
         hipLaunchKernelGGL(k_readout<F>, dim3(nblk((long)N * 16, 256)), dim3(256), 0, s, N, K, num_LM, node_types,
-                           atomic_energies, w1, H1, hidden_g, w2, scale, node_energies, zero_energies);
+                           atomic_energies, w1, H1, hidden_g, w2, scale, node_energies, zero_energies, energies_copy);
     return hipGetLastError();
 }
-template hipError_t launch_readout<double>(int, int, int, const int*, const double*, const double*, const double*, double*, const double*, double, double*, int, hipStream_t);
-template hipError_t launch_readout<float>(int, int, int, const int*, const double*, const double*, const float*, double*, const double*, double, double*, int, hipStream_t);
+template hipError_t launch_readout<double>(int, int, int, const int*, const double*, const double*, const double*, double*, const double*, double, double*, int, double*, hipStream_t);
+template hipError_t launch_readout<float>(int, int, int, const int*, const double*, const double*, const float*, double*, const double*, double, double*, int, double*, hipStream_t);
 
 template <typename F>
 hipError_t launch_seed_H1_adj(int rows, int N, int num_LM, int K, const double* w1, F* H1_adj, hipStream_t s)

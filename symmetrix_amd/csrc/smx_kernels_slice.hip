@@ -311,13 +311,14 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     }
 }
 
-__global__ void k_fpart_reduce(long n3, int nslices, const double* fpart, double* forces, int accumulate)
+__global__ void k_fpart_reduce(long n3, int nslices, const double* fpart, double* forces, int accumulate, double* copy)
 {
     const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n3) return;
     double s = accumulate ? forces[t] : 0.0;
     for (int q = 0; q < nslices; ++q) s += fpart[(size_t)q * n3 + t];
     forces[t] = s;
+    if (copy) copy[t] = s;
 }
 
 template <typename F, int CH, int CL, int BT, bool BWD>
@@ -393,11 +394,13 @@ template hipError_t launch_slice_fwd<float>(const SliceParams<float>&, hipStream
 template hipError_t launch_slice_bwd<double>(const SliceParams<double>&, hipStream_t);
 template hipError_t launch_slice_bwd<float>(const SliceParams<float>&, hipStream_t);
 
-hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, hipStream_t s)
+hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, double* copy,
+                               hipStream_t s)
 {
     const long n3 = 3 * E;
     if (n3 <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_fpart_reduce, dim3((unsigned)((n3 + 255) / 256)), dim3(256), 0, s, n3, nslices, fpart, forces, accumulate);
+    hipLaunchKernelGGL(k_fpart_reduce, dim3((unsigned)((n3 + 255) / 256)), dim3(256), 0, s, n3, nslices, fpart, forces,
+                       accumulate, copy);
     return hipGetLastError();
 }
 

@@ -106,6 +106,17 @@ int smx_compute_A0(smx_model* m, int num_nodes, const int* node_types, const int
                    const int* neigh_types, long num_edges);                             /* mace.cpp:150-201 */
 int smx_reverse_A0(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
                    const int* neigh_types, const double* xyz, const double* r, long num_edges); /* mace.cpp:203-271 */
+/* Density normalisation of the A-basis and its adjoint; no-ops for models with A0_scaled / A1_scaled false.
+ * SMX_ERANGE ("Out of bounds in CubicSpline::evaluate.") where the reference throws std::invalid_argument. */
+int smx_compute_A0_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* r, long num_edges);     /* mace.cpp:273-297 */
+int smx_reverse_A0_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* xyz, const double* r, long num_edges); /* mace.cpp:299-346 */
+int smx_compute_A1_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* r, long num_edges);     /* mace.cpp:681-705 */
+int smx_reverse_A1_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* xyz, const double* r, long num_edges,
+                          int zero_dxyz);                                               /* mace.cpp:707-757 */
 int smx_compute_M0(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:348-370 */
 int smx_reverse_M0(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:372-395 */
 int smx_compute_H1(smx_model* m, int num_nodes);                                        /* mace.cpp:397-423 */

@@ -86,11 +86,30 @@ public:
         check(smx_reverse_A0(m_, num_nodes, node_types.data(), num_neigh.data(), neigh_types.data(), xyz.data(), r.data(), (long)r.size()));
         pull("node_forces", node_forces);
     }
-    // density normalisation: no-ops for models without it (mace.cpp:280, 307, 688, 716); models with it do not load
-    void compute_A0_scaled(const int, std::span<const int>, std::span<const int>, std::span<const int>, std::span<const double>) {}
-    void reverse_A0_scaled(const int, std::span<const int>, std::span<const int>, std::span<const int>, std::span<const double>, std::span<const double>) {}
-    void compute_A1_scaled(const int, std::span<const int>, std::span<const int>, std::span<const int>, std::span<const double>) {}
-    void reverse_A1_scaled(const int, std::span<const int>, std::span<const int>, std::span<const int>, std::span<const double>, std::span<const double>, bool = true) {}
+    // density normalisation: no-ops for models without it (mace.cpp:280, 307, 688, 716)
+    void compute_A0_scaled(const int num_nodes, std::span<const int> node_types, std::span<const int> num_neigh,
+                           std::span<const int> neigh_types, std::span<const double> r)
+    {
+        check(smx_compute_A0_scaled(m_, num_nodes, node_types.data(), num_neigh.data(), neigh_types.data(), r.data(), (long)r.size()));
+    }
+    void reverse_A0_scaled(const int num_nodes, std::span<const int> node_types, std::span<const int> num_neigh,
+                           std::span<const int> neigh_types, std::span<const double> xyz, std::span<const double> r)
+    {
+        check(smx_reverse_A0_scaled(m_, num_nodes, node_types.data(), num_neigh.data(), neigh_types.data(), xyz.data(), r.data(), (long)r.size()));
+        pull("node_forces", node_forces);
+    }
+    void compute_A1_scaled(const int num_nodes, std::span<const int> node_types, std::span<const int> num_neigh,
+                           std::span<const int> neigh_types, std::span<const double> r)
+    {
+        check(smx_compute_A1_scaled(m_, num_nodes, node_types.data(), num_neigh.data(), neigh_types.data(), r.data(), (long)r.size()));
+    }
+    void reverse_A1_scaled(const int num_nodes, std::span<const int> node_types, std::span<const int> num_neigh,
+                           std::span<const int> neigh_types, std::span<const double> xyz, std::span<const double> r,
+                           bool zero_dxyz = true)
+    {
+        check(smx_reverse_A1_scaled(m_, num_nodes, node_types.data(), num_neigh.data(), neigh_types.data(), xyz.data(), r.data(), (long)r.size(), zero_dxyz ? 1 : 0));
+        pull("node_forces", node_forces);
+    }
     void compute_M0(const int num_nodes, std::span<const int> node_types) { check(smx_compute_M0(m_, num_nodes, node_types.data())); }
     void reverse_M0(const int num_nodes, std::span<const int> node_types) { check(smx_reverse_M0(m_, num_nodes, node_types.data())); }
     void compute_H1(const int num_nodes) { check(smx_compute_H1(m_, num_nodes)); pull("H1", H1); }

@@ -174,6 +174,24 @@ struct Engine : EngineBase {
     int N_geo = 0;
     DVec<int> first_neigh, recv_order, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
     int sender_rows = 0;
+    // pair terms: ZBL constants per species pair, density-normalisation splines, divisors of the last forward pass
+    DVec<double> zbl_a, zbl_rmax, zbl_zz, A0spl, A1spl, div0, div1;
+    ZblParams zbl_params() const
+    {
+        ZblParams z{};
+        z.T = hm.T; z.a_pair = zbl_a.p; z.rmax_pair = zbl_rmax.p; z.zz_pair = zbl_zz.p;
+        for (int q = 0; q < 4; ++q) z.c[q] = hm.zbl_c[q];
+        z.p = hm.zbl_p;
+        return z;
+    }
+    PairSpline scale_spline(int layer) const
+    {
+        PairSpline sp{};
+        sp.c = layer == 0 ? A0spl.p : A1spl.p;
+        sp.h = layer == 0 ? hm.A0_spline_h : hm.A1_spline_h;
+        sp.nodes = layer == 0 ? hm.A0_spline_nodes : hm.A1_spline_nodes;
+        return sp;
+    }
     // caller's output arrays of the running whole-pipeline call; the kernel that forms the final values writes
     // them too and clears the pointer, otherwise a copy is enqueued at the end
     double* energies_copy = nullptr;
@@ -242,6 +260,23 @@ struct Engine : EngineBase {
         upload_as(ro2_w1, hm.readout_2_w1, s);
         upload_as(ro2_w2, hm.readout_2_w2, s);
         upload_as(E0, hm.atomic_energies, s);
+        if (hm.has_zbl) {
+            // zbl.cpp:22-35: screening length and envelope radius of every ordered species pair
+            const int T = hm.T;
+            std::vector<double> a((size_t)T * T), rm((size_t)T * T), zz((size_t)T * T);
+            for (int i = 0; i < T; ++i)
+                for (int j = 0; j < T; ++j) {
+                    const int Zi = hm.atomic_numbers[i], Zj = hm.atomic_numbers[j];
+                    if (Zi < 0 || Zj < 0 || Zi >= (int)hm.zbl_covalent_radii.size() || Zj >= (int)hm.zbl_covalent_radii.size())
+                        throw Error(SMX_EFILE, "model file: zbl_covalent_radii does not cover the atomic numbers of the model");
+                    a[(size_t)i * T + j] = hm.zbl_a_prefactor * 0.529 / (std::pow((double)Zi, hm.zbl_a_exp) + std::pow((double)Zj, hm.zbl_a_exp));
+                    rm[(size_t)i * T + j] = hm.zbl_covalent_radii[Zi] + hm.zbl_covalent_radii[Zj];
+                    zz[(size_t)i * T + j] = (double)Zi * (double)Zj;
+                }
+            upload_as(zbl_a, a, s); upload_as(zbl_rmax, rm, s); upload_as(zbl_zz, zz, s);
+        }
+        if (hm.A0_scaled) upload_as(A0spl, hm.A0_spline_c, s);
+        if (hm.A1_scaled) upload_as(A1spl, hm.A1_spline_c, s);
         auto up_poly = [&](DevPoly& d, const PolySpec& p) {
             upload_as(d.packed, p.packed, s); upload_as(d.chunks, p.chunks, s);
             upload_as(d.coef, p.coef, s);
@@ -512,6 +547,45 @@ struct Engine : EngineBase {
                                            4L * k * k, (long)l * k * k, reverse ? 1 : 0, 0, k, k, 2 * l + 1);
         HIPCHK((launch_gemm<F, F, F>(g, stream)));
     }
+    // density normalisation of A0 / A1 and its adjoint; no-ops for models without it (mace.cpp:280, 688)
+    void st_scale(int layer, int N, bool reverse)
+    {
+        if (!(layer == 0 ? hm.A0_scaled : hm.A1_scaled)) return;
+        need(r, "r"); need(first_neigh.p, "num_neigh"); need(node_types, "node_types"); need(neigh_types, "neigh_types");
+        DVec<double>& dv = layer == 0 ? div0 : div1;
+        DVec<F>& A = layer == 0 ? A0 : A1;
+        DVec<F>& Aa = layer == 0 ? A0_adj : A1_adj;
+        const int width = 16 * K();
+        if (A.n < (size_t)N * width) throw Error(SMX_EINVAL, "density normalisation called before its A-basis exists");
+        if (!reverse) {
+            dv.size_to((size_t)N, stream);
+            HIPCHK(launch_scale_fwd<F>(N, first_neigh.p, node_types, neigh_types, r, scale_spline(layer), hm.T, A.p, width,
+                                       dv.p, flags.p, stream));
+        } else {
+            need(xyz, "xyz");
+            if (dv.n < (size_t)N || Aa.n < (size_t)N * width)
+                throw Error(SMX_EINVAL, "adjoint of the density normalisation called before its forward pass");
+            node_forces.resize((size_t)3 * E, stream);
+            HIPCHK(launch_scale_bwd<F>(N, first_neigh.p, node_types, neigh_types, xyz, r, scale_spline(layer), hm.T, A.p,
+                                       Aa.p, width, dv.p, node_forces.p, flags.p, stream));
+        }
+    }
+    void check_spline_flag()
+    {
+        int f = 0;
+        HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, stream));
+        HIPCHK(hipStreamSynchronize(stream));
+        if (f & 4) {
+            HIPCHK(hipMemsetAsync(flags.p, 0, sizeof(int), stream));
+            throw Error(SMX_ERANGE, "Out of bounds in CubicSpline::evaluate.");
+        }
+    }
+    void st_zbl(int N)
+    {
+        if (!hm.has_zbl) return;
+        HIPCHK(launch_zbl(N, first_neigh.p, node_types, neigh_types, xyz, r, zbl_params(), node_energies.p,
+                          node_forces.p, stream));
+    }
     void st_poly(int N, bool layer1)
     {
         PolyParams<F> p{};
@@ -713,8 +787,6 @@ struct Engine : EngineBase {
                  const double* rr, long E_, bool on_device, double* d_energies, double* d_forces) override
     {
         if (N < 0 || E_ < 0) throw Error(SMX_EINVAL, "negative num_nodes or num_edges");
-        if (hm.has_zbl || hm.A0_scaled || hm.A1_scaled)
-            throw Error(SMX_EUNSUPPORTED, "models with ZBL or density normalisation are not implemented on the device yet");
         if (!on_device) edges_from_counts_check(N, nn, E_);
         if (N == 0) {
             if (E_ != 0) throw Error(SMX_EINVAL, "edges without nodes");
@@ -750,27 +822,42 @@ struct Engine : EngineBase {
         if (N == 0) return;
 
         energies_copy = d_energies; forces_copy = d_forces;
+        // Terms that add to the forces before the layer-1 adjoint writes them (mace.cpp:27-35, 56): with any of
+        // them the force array starts at zero and every later stage accumulates.
+        const bool early_forces = hm.has_zbl || hm.A1_scaled;
+        if (early_forces) HIPCHK(launch_fill<double>(node_forces.p, 3 * E, 0.0, stream));
+        if (hm.has_zbl) {
+            HIPCHK(launch_fill<double>(node_energies.p, (long)N, 0.0, stream));
+            st_zbl(N);
+        }
         stage_begin(ST_AGG0F); st_agg0_fwd(N); stage_end(ST_AGG0F);
         stage_begin(ST_A0LIN); st_A0_lin(N, false); stage_end(ST_A0LIN);
+        st_scale(0, N, false);
         stage_begin(ST_M0); st_poly(N, false); stage_end(ST_M0);
         stage_begin(ST_H1); st_H1(N, false); stage_end(ST_H1);
         stage_begin(ST_AGG1F); st_agg1_fwd(N); stage_end(ST_AGG1F);
         stage_begin(ST_A1); st_A1(N, false); stage_end(ST_A1);
+        st_scale(1, N, false);
         stage_begin(ST_M1); st_poly(N, true); stage_end(ST_M1);
         stage_begin(ST_H2); st_H2(N); stage_end(ST_H2);
-        stage_begin(ST_READOUT); st_readouts(N, true); stage_end(ST_READOUT);
+        stage_begin(ST_READOUT); st_readouts(N, !hm.has_zbl); stage_end(ST_READOUT);
         stage_begin(ST_REVH2); st_reverse_H2(N, false); stage_end(ST_REVH2);
         stage_begin(ST_REVM1); st_reverse_M1(N); stage_end(ST_REVM1);
+        st_scale(1, N, true);
         stage_begin(ST_REVA1); st_A1(N, true); stage_end(ST_REVA1);
-        st_agg1_bwd(N, true, false);
+        st_agg1_bwd(N, !early_forces, false);
         stage_begin(ST_REVH1); st_H1(N, true); stage_end(ST_REVH1);
         stage_begin(ST_REVM0); st_reverse_M0(N); stage_end(ST_REVM0);
+        st_scale(0, N, true);
         stage_begin(ST_REVA0LIN); st_A0_lin(N, true); stage_end(ST_REVA0LIN);
         st_agg0_bwd(N);
 
         if (energies_copy) HIPCHK(hipMemcpyAsync(energies_copy, node_energies.p, (size_t)N * sizeof(double), hipMemcpyDeviceToDevice, stream));
         if (forces_copy && E) HIPCHK(hipMemcpyAsync(forces_copy, node_forces.p, (size_t)3 * E * sizeof(double), hipMemcpyDeviceToDevice, stream));
         energies_copy = nullptr; forces_copy = nullptr;
+        // the reference throws from CubicSpline::evaluate for an edge beyond the normalisation spline
+        // (cubic_spline.cpp:19-20); callers of the device-resident variant vouch for their edge lengths
+        if (!on_device && (hm.A0_scaled || hm.A1_scaled)) check_spline_flag();
     }
 
     // stage-level entry points (host arrays)
@@ -780,8 +867,6 @@ struct Engine : EngineBase {
         const std::string s(name);
         energies_copy = nullptr; forces_copy = nullptr;
         if (N < 0) throw Error(SMX_EINVAL, "negative num_nodes");
-        if (hm.has_zbl || hm.A0_scaled || hm.A1_scaled)
-            throw Error(SMX_EUNSUPPORTED, "models with ZBL or density normalisation are not implemented on the device yet");
         if (nn && E_ >= 0) edges_from_counts_check(N, nn, E_);
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, false);
         if (nn) build_first_neigh(N);
@@ -789,6 +874,17 @@ struct Engine : EngineBase {
         if (s == "Y" || s == "R0" || s == "R1") return;  // geometry remembered; evaluated inside the fused kernels
         if (s == "A0") { build_type_groups(N); st_agg0_fwd(N); st_A0_lin(N, false); }
         else if (s == "reverse_A0") { build_type_groups(N); st_A0_lin(N, true); st_agg0_bwd(N); }
+        else if (s == "A0_scaled") { st_scale(0, N, false); if (hm.A0_scaled) check_spline_flag(); }
+        else if (s == "reverse_A0_scaled") { st_scale(0, N, true); if (hm.A0_scaled) check_spline_flag(); }
+        else if (s == "A1_scaled") { st_scale(1, N, false); if (hm.A1_scaled) check_spline_flag(); }
+        else if (s == "reverse_A1_scaled") {
+            if (hm.A1_scaled) {
+                node_forces.resize((size_t)3 * E, stream);
+                if (fa) HIPCHK(launch_fill<double>(node_forces.p, 3 * E, 0.0, stream));
+            }
+            st_scale(1, N, true);
+            if (hm.A1_scaled) check_spline_flag();
+        }
         else if (s == "M0") { build_type_groups(N); st_poly(N, false); }
         else if (s == "reverse_M0") st_reverse_M0(N);
         else if (s == "H1") st_H1(N, false);
@@ -1155,6 +1251,27 @@ int smx_reverse_A0(smx_model* m, int num_nodes, const int* node_types, const int
                    const double* xyz, const double* r, long num_edges)
 {
     SMX_STAGE(smx_reverse_A0, "reverse_A0", node_types, num_neigh, nullptr, neigh_types, xyz, r, num_edges, 0, 0);
+}
+int smx_compute_A0_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* r, long num_edges)
+{
+    SMX_STAGE(smx_compute_A0_scaled, "A0_scaled", node_types, num_neigh, nullptr, neigh_types, nullptr, r, num_edges, 0, 0);
+}
+int smx_reverse_A0_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* xyz, const double* r, long num_edges)
+{
+    SMX_STAGE(smx_reverse_A0_scaled, "reverse_A0_scaled", node_types, num_neigh, nullptr, neigh_types, xyz, r, num_edges, 0, 0);
+}
+int smx_compute_A1_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* r, long num_edges)
+{
+    SMX_STAGE(smx_compute_A1_scaled, "A1_scaled", node_types, num_neigh, nullptr, neigh_types, nullptr, r, num_edges, 0, 0);
+}
+int smx_reverse_A1_scaled(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh,
+                          const int* neigh_types, const double* xyz, const double* r, long num_edges, int zero_dxyz)
+{
+    SMX_STAGE(smx_reverse_A1_scaled, "reverse_A1_scaled", node_types, num_neigh, nullptr, neigh_types, xyz, r, num_edges,
+              zero_dxyz, 0);
 }
 int smx_compute_M0(smx_model* m, int num_nodes, const int* node_types)
 {

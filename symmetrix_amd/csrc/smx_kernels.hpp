@@ -86,6 +86,34 @@ hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const in
                                 F* H_adj, int zero_first, hipStream_t s);
 
 // ---------------------------------------------------------------------------
+// Pair terms of the edge length alone (smx_kernels_pair.hip)
+struct ZblParams {
+    int T;
+    const double* a_pair;      // [T][T] screening length of the species pair
+    const double* rmax_pair;   // [T][T] envelope radius: sum of the covalent radii
+    const double* zz_pair;     // [T][T] Z_i * Z_j
+    double c[4];
+    int p;
+};
+struct PairSpline {
+    const double* c;           // [pairs][nodes-1][4], unordered pairs (a <= b) row-major upper triangle
+    double h;
+    int nodes;
+};
+// node_energies[i] += sum_j V(r_ij), node_forces[ij] -= V'(r_ij) xyz_ij / r_ij      (zbl.cpp:96-125)
+hipError_t launch_zbl(int N, const int* first_neigh, const int* node_types, const int* neigh_types, const double* xyz,
+                      const double* r, const ZblParams& z, double* energies, double* forces, hipStream_t s);
+// A[i] /= 1 + sum_j s(r_ij), divisor kept (mace.cpp:273-297, 681-705); bit 4 of *flags: r outside the spline
+template <typename F>
+hipError_t launch_scale_fwd(int N, const int* first_neigh, const int* node_types, const int* neigh_types, const double* r,
+                            const PairSpline& sp, int T, F* A, int width, double* divisor, int* flags, hipStream_t s);
+// adjoint of the above (mace.cpp:299-346, 707-757): forces += ..., A_adj /= divisor
+template <typename F>
+hipError_t launch_scale_bwd(int N, const int* first_neigh, const int* node_types, const int* neigh_types,
+                            const double* xyz, const double* r, const PairSpline& sp, int T, const F* A, F* A_adj,
+                            int width, const double* divisor, double* forces, int* flags, hipStream_t s);
+
+// ---------------------------------------------------------------------------
 // Integer list preparation
 hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums, hipStream_t s);  // out[n] = total
 // order[N]: receivers by decreasing degree

@@ -155,16 +155,24 @@ class MACE:
         _lib.check(self._L.smx_reverse_A0(self._h, int(num_nodes), _pi(nt), _pi(nn), _pi(nty), _pd(x), _pd(rr), C.c_long(len(rr))))
 
     def compute_A0_scaled(self, num_nodes, node_types, num_neigh, neigh_types, r):
-        pass  # no-op for models without density normalisation (mace.cpp:280)
+        nt, nn, nty, rr = _i(node_types), _i(num_neigh), _i(neigh_types), _d(r)
+        _lib.check(self._L.smx_compute_A0_scaled(self._h, int(num_nodes), _pi(nt), _pi(nn), _pi(nty), _pd(rr), C.c_long(len(rr))))
 
     def reverse_A0_scaled(self, num_nodes, node_types, num_neigh, neigh_types, xyz, r):
-        pass
+        nt, nn, nty = _i(node_types), _i(num_neigh), _i(neigh_types)
+        x, rr = _d(xyz).reshape(-1), _d(r)
+        _lib.check(self._L.smx_reverse_A0_scaled(self._h, int(num_nodes), _pi(nt), _pi(nn), _pi(nty), _pd(x), _pd(rr),
+                                                 C.c_long(len(rr))))
 
     def compute_A1_scaled(self, num_nodes, node_types, num_neigh, neigh_types, r):
-        pass
+        nt, nn, nty, rr = _i(node_types), _i(num_neigh), _i(neigh_types), _d(r)
+        _lib.check(self._L.smx_compute_A1_scaled(self._h, int(num_nodes), _pi(nt), _pi(nn), _pi(nty), _pd(rr), C.c_long(len(rr))))
 
-    def reverse_A1_scaled(self, num_nodes, node_types, num_neigh, neigh_types, xyz, r):
-        pass
+    def reverse_A1_scaled(self, num_nodes, node_types, num_neigh, neigh_types, xyz, r, zero_dxyz=True):
+        nt, nn, nty = _i(node_types), _i(num_neigh), _i(neigh_types)
+        x, rr = _d(xyz).reshape(-1), _d(r)
+        _lib.check(self._L.smx_reverse_A1_scaled(self._h, int(num_nodes), _pi(nt), _pi(nn), _pi(nty), _pd(x), _pd(rr),
+                                                 C.c_long(len(rr)), int(bool(zero_dxyz))))
 
     def compute_M0(self, num_nodes, node_types):
         nt = _i(node_types)

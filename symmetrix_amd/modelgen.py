@@ -61,6 +61,19 @@ def _radial_tables(rng, r, n_bessel, mlp, n_out, r_cut, p):
     return vals.T.copy(), ders.T.copy()  # [n_out][n_pts]
 
 
+def _density_splines(rng, r, h, T, n_bessel, r_cut, p, name):
+    """tanh(density_fn(bessels)^2) per unordered pair, splined like the radial tables (extract_mace_data.py:204-226)."""
+    feats = _bessel_cutoff(r, r_cut, n_bessel, p)
+    vals, ders = [], []
+    for a in range(T):
+        for b in range(a, T):
+            w = rng.normal(size=n_bessel) / sqrt(n_bessel)
+            spl = CubicSpline(r, np.tanh((feats @ w) ** 2), bc_type=("not-a-knot", "clamped"))
+            vals.append(spl(r).tolist())
+            ders.append(spl.derivative()(r).tolist())
+    return {f"{name}_spline_h": float(h), f"{name}_spline_values": vals, f"{name}_spline_derivs": ders}
+
+
 def generate_model(
     atomic_numbers,
     num_channels,
@@ -74,8 +87,15 @@ def generate_model(
     avg_num_neighbors=30.0,
     seed=0,
     pair_dependent_radial=True,
+    zbl=False,
+    density_normalisation=False,
 ):
-    """Return the model as a dict ready for json.dump."""
+    """Return the model as a dict ready for json.dump.
+
+    zbl adds the pair-repulsion keys (extract_mace_data.py:130-138); density_normalisation makes both
+    interaction layers "density" layers: one normalisation spline per unordered species pair
+    (extract_mace_data.py:201-226, 386-411).
+    """
     rng = np.random.default_rng(seed)
     Z = sorted(int(z) for z in atomic_numbers)
     T = len(Z)
@@ -92,8 +112,19 @@ def generate_model(
         "L_max": int(L_max),
         "atomic_numbers": Z,
         "atomic_energies": rng.normal(size=T).tolist(),
-        "has_zbl": False,
+        "has_zbl": bool(zbl),
     }
+    if zbl:
+        # constants of mace's ZBLBasis; covalent radii indexed by atomic number (synthetic beyond H, C, N, O)
+        radii = [0.2] + [0.5 + 0.004 * z for z in range(1, max(Z) + 1)]
+        for z, rad in ((1, 0.31), (6, 0.76), (7, 0.71), (8, 0.66)):
+            if z < len(radii):
+                radii[z] = rad
+        out["zbl_a_exp"] = 0.3
+        out["zbl_a_prefactor"] = 0.4543
+        out["zbl_c"] = [0.1818 * 0.8, 0.5099 * 0.8, 0.2802 * 0.8, 0.02817 * 0.8]
+        out["zbl_covalent_radii"] = radii
+        out["zbl_p"] = 6
 
     # ----- radial splines: one table per unordered pair (a<=b), row-major upper triangle
     r, h = np.linspace(1e-12, r_cut, num_spline_points, retstep=True)
@@ -118,9 +149,14 @@ def generate_model(
 
     # ----- layer 0
     out["H0_weights"] = rng.normal(size=T * K).tolist()
-    out["A0_scaled"] = False
+    out["A0_scaled"] = bool(density_normalisation)
+    if density_normalisation:
+        out.update(_density_splines(rng, r, h, T, n_bessel, r_cut, cutoff_p, "A0"))
+    # (the extractor drops the 1/avg_num_neighbors factor for density layers; a random model keeps a comparable
+    # magnitude by dividing by the typical divisor instead)
+    norm0 = avg_num_neighbors / 3.0 if density_normalisation else avg_num_neighbors
     out["A0_weights"] = [
-        [(rng.normal(size=(K, K)) / (sqrt(K) * avg_num_neighbors) * 4.0).ravel().tolist()
+        [(rng.normal(size=(K, K)) / (sqrt(K) * norm0) * 4.0).ravel().tolist()
          for _ in range(l_max + 1)]
         for _ in range(T)
     ]
@@ -191,9 +227,12 @@ def generate_model(
     out["Phi1_clebsch_gordan"] = cg_val
     out["Phi1_lelm1lm2"] = cg_q
 
-    out["A1_scaled"] = False
+    out["A1_scaled"] = bool(density_normalisation)
+    if density_normalisation:
+        out.update(_density_splines(rng, r, h, T, n_bessel, r_cut, cutoff_p, "A1"))
+    norm1 = avg_num_neighbors / 3.0 if density_normalisation else avg_num_neighbors
     out["A1_weights"] = [
-        (rng.normal(size=(num_e[l], K, K)) / (sqrt(num_e[l] * K) * avg_num_neighbors) * 4.0).ravel().tolist()
+        (rng.normal(size=(num_e[l], K, K)) / (sqrt(num_e[l] * K) * norm1) * 4.0).ravel().tolist()
         for l in range(l_max + 1)
     ]
 

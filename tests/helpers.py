@@ -7,9 +7,9 @@ import numpy as np
 from symmetrix_amd import modelgen, neighbors, systems
 
 
-def tiny_model(K=4, L_max=1, T=(1, 6, 8), r_cut=4.0, n_pts=48, seed=3, pair=True):
+def tiny_model(K=4, L_max=1, T=(1, 6, 8), r_cut=4.0, n_pts=48, seed=3, pair=True, zbl=False, density=False):
     return modelgen.generate_model(list(T), K, L_max, r_cut, num_spline_points=n_pts, seed=seed,
-                                   pair_dependent_radial=pair)
+                                   pair_dependent_radial=pair, zbl=zbl, density_normalisation=density)
 
 
 def write_model(model, path):

@@ -112,6 +112,57 @@ def test_golden_fixture(gpu, dtype):
         assert np.abs(getattr(eng, name) - z[name]).max() <= tol["inter"] * 10 * max(1.0, np.abs(z[name]).max()), name
 
 
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("K,L_max,natoms,zbl,density", [(32, 0, 40, True, False), (96, 0, 48, True, True),
+                                                        (48, 1, 30, True, True), (128, 1, 24, False, True)])
+def test_pair_terms_match_oracle(gpu, tmp_models, K, L_max, natoms, zbl, density, dtype):
+    """Models with ZBL repulsion and / or density-normalised layers (mace.cpp:27-35, 273-346, 681-757)."""
+    model = H.tiny_model(K=K, L_max=L_max, n_pts=64, seed=K + L_max, pair=(K != 96), zbl=zbl, density=density)
+    path = H.write_model(model, tmp_models / f"p_{K}_{L_max}_{int(zbl)}{int(density)}.json")
+    orc = _oracle()(model)
+    eng = gpu(path, dtype)
+    pos, cell, sp = H.small_system(natoms, seed=natoms + 1)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K={K} L_max={L_max} atoms={natoms} zbl={zbl} density={density} {dtype}", flush=True)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    _compare(orc, eng, dtype)
+    f1, e1 = eng.node_forces, eng.node_energies
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    assert np.array_equal(f1, eng.node_forces) and np.array_equal(e1, eng.node_energies)
+
+
+def test_density_normalisation_stage_calls(gpu, tmp_models):
+    """compute_A0_scaled / reverse_A0_scaled and their layer-1 twins called stage by stage, as test_mace.py does."""
+    model = H.tiny_model(K=8, L_max=1, n_pts=40, seed=9, density=True)
+    path = H.write_model(model, tmp_models / "stage_scaled.json")
+    orc = _oracle()(model)
+    eng = gpu(path)
+    pos, cell, sp = H.small_system(10, seed=3)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    N, nt, nn, ni, nty, xyz, r = H.call_args(ea)
+    rng = np.random.default_rng(1)
+    for m in (orc, eng):
+        m.compute_Y(xyz); m.compute_R0(N, nt, nn, nty, r); m.compute_A0(N, nt, nn, nty)
+        m.compute_A0_scaled(N, nt, nn, nty, r)
+    assert np.allclose(orc.A0, eng.A0, atol=1e-12)
+    adj = rng.normal(size=len(orc.A0))
+    for m in (orc, eng):
+        m.A0_adj = adj
+        m.node_forces = np.zeros(len(xyz))
+        m.reverse_A0_scaled(N, nt, nn, nty, xyz, r)
+    assert np.allclose(orc.A0_adj, eng.A0_adj, atol=1e-12)
+    assert np.allclose(orc.node_forces, eng.node_forces, atol=1e-11)
+    A1 = rng.normal(size=N * 16 * 8)
+    for m in (orc, eng):
+        m.A1 = A1
+        m.compute_A1_scaled(N, nt, nn, nty, r)
+        m.A1_adj = adj[:len(A1)]
+        m.reverse_A1_scaled(N, nt, nn, nty, xyz, r, True)
+    assert np.allclose(orc.A1, eng.A1, atol=1e-12) and np.allclose(orc.A1_adj, eng.A1_adj, atol=1e-12)
+    assert np.allclose(orc.node_forces, eng.node_forces, atol=1e-11)
+
+
 def test_stage_level_calls_follow_the_reference_test_method(gpu, tmp_models):
     """symmetrix/test/test_mace.py drives the evaluator stage by stage and overwrites
     intermediates between calls (e.g. :246-249).  Same here, against the oracle."""

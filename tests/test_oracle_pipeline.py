@@ -172,6 +172,87 @@ def test_total_energy_per_edge_forces(setup):
     assert np.allclose(-orc.node_forces, g, rtol=1e-4, atol=1e-6)
 
 
+# ---------------------------------------------------------------------------
+# ZBL and density normalisation (mace.cpp:27-35, 273-346, 681-757).  The reference holds no stored value for
+# these stages that can be used here; they are pinned by what the mathematics fixes.
+@pytest.mark.parametrize("L_max", [0, 1])
+def test_pair_terms_forces_are_the_energy_gradient(L_max):
+    """Whole pipeline with ZBL and both normalisations switched on: node_forces[ij] = -dE/dxyz_ij."""
+    model = H.tiny_model(K=3, L_max=L_max, n_pts=40, zbl=True, density=True)
+    orc = OracleMACE(model)
+    pos, cell, sp = H.small_system(7, seed=4)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    args = list(H.call_args(ea))
+
+    def f(xyz):
+        a = list(args); a[5] = xyz; a[6] = _r_of(xyz)
+        orc.compute_node_energies_forces(*a)
+        return orc.node_energies.sum()
+    xyz = ea["xyz"].copy()
+    g = numerical_gradient(f, xyz)
+    assert np.allclose(-orc.node_forces, g, rtol=1e-4, atol=1e-6)
+
+
+def test_density_normalisation_special_cases():
+    """s(r) = 0 leaves the model unchanged; s(r) = c divides A0 by 1 + c * degree (mace.cpp:285-296)."""
+    base = H.tiny_model(K=3, L_max=1, n_pts=40, density=True)
+    pos, cell, sp = H.small_system(8, seed=5)
+    nl, ea = H.edges_of(pos, cell, sp, base["r_cut"])
+    geo = (ea["num_nodes"], ea["node_types"], ea["num_neigh"], ea["neigh_types"])
+
+    def with_spline(value):
+        m = json.loads(json.dumps(base))
+        for name in ("A0", "A1"):
+            n_pairs, n_pts = len(m[f"{name}_spline_values"]), len(m[f"{name}_spline_values"][0])
+            m[f"{name}_spline_values"] = [[value] * n_pts for _ in range(n_pairs)]
+            m[f"{name}_spline_derivs"] = [[0.0] * n_pts for _ in range(n_pairs)]
+        return m
+    plain = json.loads(json.dumps(base)); plain["A0_scaled"] = False; plain["A1_scaled"] = False
+    o_plain, o_zero, o_const = OracleMACE(plain), OracleMACE(with_spline(0.0)), OracleMACE(with_spline(0.25))
+    for o in (o_plain, o_zero, o_const):
+        o.compute_node_energies_forces(*H.call_args(ea))
+    assert np.array_equal(o_zero.node_energies, o_plain.node_energies)
+    assert np.array_equal(o_zero.node_forces, o_plain.node_forces)
+    # A0 of the constant-spline model against the plain model's A0, atom by atom
+    for o in (o_plain, o_const):
+        o.compute_Y(ea["xyz"]); o.compute_R0(*geo, ea["r"]); o.compute_A0(*geo); o.compute_A0_scaled(*geo, ea["r"])
+    width = len(o_plain.A0) // ea["num_nodes"]
+    expect = o_plain.A0.reshape(-1, width) / (1.0 + 0.25 * ea["num_neigh"][:, None])
+    assert np.allclose(o_const.A0.reshape(-1, width), expect, rtol=1e-14, atol=0)
+
+
+def test_zbl_adds_the_pair_sum():
+    """has_zbl adds sum_j V(r_ij) to every node energy and -V'(r_ij) xyz/r to every edge force (zbl.cpp:96-125);
+    V itself is pinned against the reference's object code in test_oracle_leaves.py."""
+    m0 = H.tiny_model(K=3, L_max=0, n_pts=40)
+    m1 = json.loads(json.dumps(m0))
+    zb = H.tiny_model(K=3, L_max=0, n_pts=40, zbl=True)
+    for k in ("has_zbl", "zbl_a_exp", "zbl_a_prefactor", "zbl_c", "zbl_covalent_radii", "zbl_p"):
+        m1[k] = zb[k]
+    pos, cell, sp = H.small_system(9, seed=6)
+    nl, ea = H.edges_of(pos, cell, sp, m0["r_cut"])
+    o0, o1 = OracleMACE(m0), OracleMACE(m1)
+    o0.compute_node_energies_forces(*H.call_args(ea)); o1.compute_node_energies_forces(*H.call_args(ea))
+    dE = o1.node_energies - o0.node_energies
+    dF = (o1.node_forces - o0.node_forces).reshape(-1, 3)
+    # the added force is radial and its magnitude is the derivative of the added energy along r
+    xyz = ea["xyz"].reshape(-1, 3)
+    assert np.abs(np.cross(dF, xyz)).max() < 1e-12
+    first = np.concatenate([[0], np.cumsum(ea["num_neigh"])])
+
+    def pair_energy(r):
+        a = list(H.call_args(ea)); a[6] = r; a[5] = (xyz / ea["r"][:, None] * r[:, None]).ravel()
+        o1.compute_node_energies_forces(*a); e1 = o1.node_energies.copy()
+        o0.compute_node_energies_forces(*a); return e1 - o0.node_energies
+    h = 1e-5
+    rp, rm = ea["r"] + h, ea["r"] - h
+    dEdr_sum = (pair_energy(rp) - pair_energy(rm)) / (2 * h)       # all edges of an atom stretched together
+    radial = -(dF * xyz).sum(1) / ea["r"]                          # V'(r_ij) per edge
+    per_atom = np.array([radial[first[i]:first[i + 1]].sum() for i in range(ea["num_nodes"])])
+    assert np.allclose(per_atom, dEdr_sum, rtol=1e-5, atol=1e-8)
+    assert np.abs(dE).max() > 0
+
+
 def test_invariances():
     model = H.tiny_model(K=4, L_max=1, n_pts=40)
     orc = OracleMACE(model)

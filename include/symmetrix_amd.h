@@ -166,6 +166,26 @@ int smx_synchronize(smx_model* m);
 int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const int* receiver_atom,
                       double* atom_forces, double* virial);
 
+/* Full neighbour list built on the device, counterpart of the edge construction of
+ * pair_symmetrix_mace.cpp:246-315 (ghost images, r^2 < r_cut^2) and of the ASE caller's
+ * neighbor_list('ijdD') (symmetrix_calc.py:77-83), in the canonical order of this library: receivers
+ * ascending, senders ascending within a receiver, images of one sender in the order of the shift list.
+ * The caller lists the periodic images to consider: shift_int[num_shifts][3] (integer cell shifts, in
+ * lexicographic order; (0,0,0) marks the shift for which a pair i == j is no edge) and
+ * shift_vec[num_shifts][3] = shift . cell in Cartesian coordinates (host arrays).  d_positions[num_atoms][3]
+ * and d_types[num_atoms] (may be NULL) are device arrays.  Edge vectors are (x_j + shift) - x_i and
+ * r = sqrt((d0*d0 + d1*d1) + d2*d2), every operation rounded once.  The arrays stay on the device and belong to
+ * the list object until the next build; their addresses can be handed to smx_compute_device. */
+typedef struct smx_nlist smx_nlist;
+smx_nlist* smx_nlist_create(void);
+void smx_nlist_free(smx_nlist* nl);
+int smx_nlist_build(smx_nlist* nl, int num_atoms, const double* d_positions, const int* d_types, int num_shifts,
+                    const int* shift_int, const double* shift_vec, double r_cut, void* stream, long* num_edges);
+int smx_nlist_arrays(smx_nlist* nl, const int** num_neigh, const int** first_neigh, const int** neigh_indices,
+                     const int** neigh_types, const int** neigh_shift, const double** xyz, const double** r);
+int smx_nlist_copy_to_host(smx_nlist* nl, int* num_neigh, int* neigh_indices, int* neigh_types, int* neigh_shift,
+                           double* xyz, double* r);
+
 #ifdef __cplusplus
 }
 #endif

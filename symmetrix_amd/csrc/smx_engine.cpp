@@ -1113,6 +1113,80 @@ smx::EngineBase& E(smx_model* m)
 
 }  // namespace
 
+// ---------------------------------------------------------------------------
+// Device neighbour list (canonical order; see smx_kernels_nlist.hip)
+namespace smx {
+struct NeighborList {
+    DVec<double> part, shift_vec, xyz, r;
+    DVec<int> shift_int, atom_bin, bin_count, bin_start, bin_atoms, count, first, num_neigh, neigh_indices, neigh_types,
+        neigh_shift, scan_tmp;
+    DVec<long long> keys;
+    int N = 0;
+    long E = 0;
+
+    long build(int N_, const double* d_pos, const int* d_types, int num_shifts, const int* h_shift_int,
+               const double* h_shift_vec, double r_cut, hipStream_t s)
+    {
+        if (N_ < 0 || num_shifts <= 0 || !(r_cut > 0.0) || !h_shift_int || !h_shift_vec || (N_ > 0 && !d_pos))
+            throw Error(SMX_EINVAL, "neighbour list: bad arguments");
+        int zero_shift = -1;
+        for (int q = 0; q < num_shifts; ++q)
+            if (h_shift_int[3 * q] == 0 && h_shift_int[3 * q + 1] == 0 && h_shift_int[3 * q + 2] == 0) zero_shift = q;
+        N = N_; E = 0;
+        first.size_to((size_t)N + 1, s); num_neigh.size_to((size_t)N, s);
+        if (N == 0) {
+            HIPCHK(hipMemsetAsync(first.p, 0, sizeof(int), s));
+            return 0;
+        }
+        shift_int.upload(h_shift_int, (size_t)3 * num_shifts, s);
+        shift_vec.upload(h_shift_vec, (size_t)3 * num_shifts, s);
+        // bounding box (per-block partials, finished on the host)
+        const int nblk = std::min(256, (N + 255) / 256);
+        part.size_to((size_t)nblk * 6, s);
+        HIPCHK(launch_nl_bbox(d_pos, N, part.p, nblk, s));
+        std::vector<double> hp((size_t)nblk * 6);
+        HIPCHK(hipMemcpyAsync(hp.data(), part.p, hp.size() * sizeof(double), hipMemcpyDeviceToHost, s));
+        HIPCHK(hipStreamSynchronize(s));
+        NlGrid g{};
+        long nbins = 1;
+        for (int k = 0; k < 3; ++k) {
+            double lo = 1e300, hi = -1e300;
+            for (int b = 0; b < nblk; ++b) { lo = std::min(lo, hp[(size_t)b * 6 + k]); hi = std::max(hi, hp[(size_t)b * 6 + 3 + k]); }
+            if (!(lo <= hi)) throw Error(SMX_EINVAL, "neighbour list: positions are not finite");
+            g.lo[k] = lo; g.hi[k] = hi;
+            const double ext = hi - lo;
+            int nb = (int)std::floor(ext / r_cut);
+            nb = std::max(1, std::min(nb, 128));
+            g.nb[k] = nb;
+            g.inv_bs[k] = ext > 0.0 ? nb / ext : 0.0;
+            nbins *= nb;
+        }
+        atom_bin.size_to((size_t)N, s); bin_count.size_to((size_t)2 * nbins, s); bin_start.size_to((size_t)nbins + 1, s);
+        bin_atoms.size_to((size_t)N, s); scan_tmp.size_to((size_t)std::max<long>(nbins, N) / 1024 + 2, s);
+        HIPCHK(hipMemsetAsync(bin_count.p, 0, (size_t)2 * nbins * sizeof(int), s));
+        HIPCHK(launch_nl_bins(d_pos, N, g, atom_bin.p, bin_count.p, s));
+        HIPCHK(launch_scan_exclusive(bin_count.p, bin_start.p, (int)nbins, scan_tmp.p, s));
+        HIPCHK(launch_nl_bin_fill(N, atom_bin.p, bin_start.p, bin_count.p + nbins, bin_atoms.p, s));
+        count.size_to((size_t)N, s);
+        HIPCHK(launch_nl_search(false, d_pos, N, g, bin_start.p, bin_atoms.p, num_shifts, shift_vec.p, zero_shift, r_cut,
+                                count.p, nullptr, nullptr, s));
+        HIPCHK(launch_scan_exclusive(count.p, first.p, N, scan_tmp.p, s));
+        int total = 0;
+        HIPCHK(hipMemcpyAsync(&total, first.p + N, sizeof(int), hipMemcpyDeviceToHost, s));
+        HIPCHK(hipStreamSynchronize(s));
+        E = total;
+        keys.size_to((size_t)E, s);
+        neigh_indices.size_to((size_t)E, s); neigh_types.size_to((size_t)E, s); neigh_shift.size_to((size_t)3 * E, s);
+        xyz.size_to((size_t)3 * E, s); r.size_to((size_t)E, s);
+        HIPCHK(launch_nl_search(true, d_pos, N, g, bin_start.p, bin_atoms.p, num_shifts, shift_vec.p, zero_shift, r_cut,
+                                nullptr, first.p, keys.p, s));
+        HIPCHK(launch_nl_emit(d_pos, d_types, N, first.p, keys.p, num_shifts, shift_vec.p, shift_int.p, num_neigh.p,
+                              neigh_indices.p, neigh_types.p, neigh_shift.p, xyz.p, r.p, s));
+        return E;
+    }
+};
+}  // namespace smx
+
 extern "C" {
 
 const char* smx_last_error(void) { return smx::g_last_error.c_str(); }
@@ -1371,6 +1445,54 @@ int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const
                       double* atom_forces, double* virial)
 {
     return guarded([&] { E(m).reduce_forces(num_atoms, sender_atom, receiver_atom, atom_forces, virial); });
+}
+
+smx_nlist* smx_nlist_create(void)
+{
+    smx_nlist* out = nullptr;
+    guarded([&] { out = reinterpret_cast<smx_nlist*>(new smx::NeighborList()); });
+    return out;
+}
+void smx_nlist_free(smx_nlist* nl) { delete reinterpret_cast<smx::NeighborList*>(nl); }
+int smx_nlist_build(smx_nlist* nl, int num_atoms, const double* d_positions, const int* d_types, int num_shifts,
+                    const int* shift_int, const double* shift_vec, double r_cut, void* stream, long* num_edges)
+{
+    return guarded([&] {
+        if (!nl || !shift_int || !shift_vec || (num_atoms > 0 && !d_positions)) throw smx::Error(SMX_EINVAL, "null argument");
+        const long e = reinterpret_cast<smx::NeighborList*>(nl)->build(num_atoms, d_positions, d_types, num_shifts,
+                                                                      shift_int, shift_vec, r_cut, (hipStream_t)stream);
+        if (num_edges) *num_edges = e;
+    });
+}
+int smx_nlist_arrays(smx_nlist* nl, const int** num_neigh, const int** first_neigh, const int** neigh_indices,
+                     const int** neigh_types, const int** neigh_shift, const double** xyz, const double** r)
+{
+    return guarded([&] {
+        if (!nl) throw smx::Error(SMX_EINVAL, "null argument");
+        auto& n = *reinterpret_cast<smx::NeighborList*>(nl);
+        if (num_neigh) *num_neigh = n.num_neigh.p;
+        if (first_neigh) *first_neigh = n.first.p;
+        if (neigh_indices) *neigh_indices = n.neigh_indices.p;
+        if (neigh_types) *neigh_types = n.neigh_types.p;
+        if (neigh_shift) *neigh_shift = n.neigh_shift.p;
+        if (xyz) *xyz = n.xyz.p;
+        if (r) *r = n.r.p;
+    });
+}
+int smx_nlist_copy_to_host(smx_nlist* nl, int* num_neigh, int* neigh_indices, int* neigh_types, int* neigh_shift,
+                           double* xyz, double* r)
+{
+    return guarded([&] {
+        if (!nl) throw smx::Error(SMX_EINVAL, "null argument");
+        auto& n = *reinterpret_cast<smx::NeighborList*>(nl);
+        const size_t E = (size_t)n.E, N = (size_t)n.N;
+        if (num_neigh && N) HIPCHK(hipMemcpy(num_neigh, n.num_neigh.p, N * sizeof(int), hipMemcpyDeviceToHost));
+        if (neigh_indices && E) HIPCHK(hipMemcpy(neigh_indices, n.neigh_indices.p, E * sizeof(int), hipMemcpyDeviceToHost));
+        if (neigh_types && E) HIPCHK(hipMemcpy(neigh_types, n.neigh_types.p, E * sizeof(int), hipMemcpyDeviceToHost));
+        if (neigh_shift && E) HIPCHK(hipMemcpy(neigh_shift, n.neigh_shift.p, 3 * E * sizeof(int), hipMemcpyDeviceToHost));
+        if (xyz && E) HIPCHK(hipMemcpy(xyz, n.xyz.p, 3 * E * sizeof(double), hipMemcpyDeviceToHost));
+        if (r && E) HIPCHK(hipMemcpy(r, n.r.p, E * sizeof(double), hipMemcpyDeviceToHost));
+    });
 }
 
 }  // extern "C"

@@ -86,6 +86,25 @@ hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const in
                                 F* H_adj, int zero_first, hipStream_t s);
 
 // ---------------------------------------------------------------------------
+// Neighbour list on the device (smx_kernels_nlist.hip)
+struct NlGrid {
+    double lo[3], hi[3];     // bounding box of the positions
+    double inv_bs[3];        // 1 / bin size
+    int nb[3];               // bins per axis
+};
+hipError_t launch_nl_bbox(const double* pos, int N, double* part, int nblocks, hipStream_t s);
+hipError_t launch_nl_bins(const double* pos, int N, const NlGrid& g, int* atom_bin, int* bin_count, hipStream_t s);
+hipError_t launch_nl_bin_fill(int N, const int* atom_bin, const int* bin_start, int* bin_cursor, int* bin_atoms,
+                              hipStream_t s);
+hipError_t launch_nl_search(bool fill, const double* pos, int N, const NlGrid& g, const int* bin_start,
+                            const int* bin_atoms, int num_shifts, const double* shift_vec, int zero_shift,
+                            double r_cut, int* count, const int* first, long long* keys, hipStream_t s);
+hipError_t launch_nl_emit(const double* pos, const int* types, int N, const int* first, const long long* keys,
+                          int num_shifts, const double* shift_vec, const int* shift_int, int* num_neigh,
+                          int* neigh_indices, int* neigh_types, int* neigh_shift, double* xyz, double* r,
+                          hipStream_t s);
+
+// ---------------------------------------------------------------------------
 // Pair terms of the edge length alone (smx_kernels_pair.hip)
 struct ZblParams {
     int T;

@@ -31,6 +31,9 @@ def neighbor_list(positions, cell, r_cut, pbc=(True, True, True)):
     if cell.shape == (3,):
         cell = np.diag(cell)
     N = len(pos)
+    if N == 0:
+        return dict(i=np.zeros(0, np.int32), j=np.zeros(0, np.int32), S=np.zeros((0, 3), np.int32),
+                    xyz=np.zeros((0, 3)), r=np.zeros(0), first_neigh=np.zeros(1, np.int64))
     pbc = np.asarray(pbc, dtype=bool)
     # number of image shells needed along each lattice vector
     vol = abs(np.linalg.det(cell))
@@ -159,3 +162,77 @@ def edge_arrays(nl, species_index, num_nodes=None):
         xyz=np.ascontiguousarray(nl["xyz"], dtype=np.float64).reshape(-1),
         r=np.ascontiguousarray(nl["r"], dtype=np.float64),
     )
+
+
+def image_shifts(cell, r_cut, pbc=(True, True, True)):
+    """Integer cell shifts (lexicographic order) and their Cartesian vectors, as neighbor_list forms them."""
+    cell = np.asarray(cell, dtype=np.float64)
+    if cell.shape == (3,):
+        cell = np.diag(cell)
+    pbc = np.asarray(pbc, dtype=bool)
+    vol = abs(np.linalg.det(cell))
+    heights = np.array([vol / np.linalg.norm(np.cross(cell[(a + 1) % 3], cell[(a + 2) % 3])) for a in range(3)])
+    nshell = np.where(pbc, np.ceil(r_cut / heights).astype(int), 0)
+    ints, vecs = [], []
+    for sx in range(-nshell[0], nshell[0] + 1):
+        for sy in range(-nshell[1], nshell[1] + 1):
+            for sz in range(-nshell[2], nshell[2] + 1):
+                S = np.array([sx, sy, sz])
+                ints.append(S)
+                vecs.append(S.astype(np.float64) @ cell)
+    return np.ascontiguousarray(ints, dtype=np.int32), np.ascontiguousarray(vecs, dtype=np.float64)
+
+
+class DeviceNeighborList:
+    """The same list built on the GPU from device-resident positions (smx_nlist_* of the C ABI).
+
+    build() takes the address of a device array of positions ([N][3] float64) and, optionally, of species
+    indices ([N] int32); the edge arrays stay on the device (addresses in .ptr) for MACE.compute_device, and
+    to_host() returns them as the dict neighbor_list() / edge_arrays() would give.
+    """
+
+    def __init__(self):
+        import ctypes as C
+        from . import _lib
+        self._C, self._lib = C, _lib
+        self._L = _lib.lib()
+        self._h = self._L.smx_nlist_create()
+        if not self._h:
+            raise RuntimeError("smx_nlist_create failed: " + self._L.smx_last_error().decode())
+        self.num_atoms = 0
+        self.num_edges = 0
+        self.ptr = {}
+
+    def __del__(self):
+        try:
+            if self._h:
+                self._L.smx_nlist_free(self._h)
+        except Exception:
+            pass
+
+    def build(self, num_atoms, positions_ptr, types_ptr, cell, r_cut, pbc=(True, True, True), stream=0):
+        C = self._C
+        ints, vecs = image_shifts(cell, r_cut, pbc)
+        E = C.c_long(0)
+        self._lib.check(self._L.smx_nlist_build(
+            C.c_void_p(self._h), int(num_atoms), C.c_void_p(positions_ptr), C.c_void_p(types_ptr or 0), len(ints),
+            ints.ctypes.data_as(C.POINTER(C.c_int)), vecs.ctypes.data_as(C.POINTER(C.c_double)), C.c_double(r_cut),
+            C.c_void_p(stream), C.byref(E)))
+        self.num_atoms, self.num_edges = int(num_atoms), int(E.value)
+        names = ("num_neigh", "first_neigh", "neigh_indices", "neigh_types", "neigh_shift", "xyz", "r")
+        out = [C.c_void_p(0) for _ in names]
+        self._lib.check(self._L.smx_nlist_arrays(C.c_void_p(self._h), *[C.byref(o) for o in out]))
+        self.ptr = {n: (o.value or 0) for n, o in zip(names, out)}
+        return self.num_edges
+
+    def to_host(self):
+        C = self._C
+        N, E = self.num_atoms, self.num_edges
+        nn = np.zeros(N, dtype=np.int32); ni = np.zeros(E, dtype=np.int32); nty = np.zeros(E, dtype=np.int32)
+        S = np.zeros((E, 3), dtype=np.int32); xyz = np.zeros((E, 3)); r = np.zeros(E)
+        p = lambda a, t: a.ctypes.data_as(C.POINTER(t))
+        self._lib.check(self._L.smx_nlist_copy_to_host(C.c_void_p(self._h), p(nn, C.c_int), p(ni, C.c_int), p(nty, C.c_int),
+                                                       p(S, C.c_int), p(xyz, C.c_double), p(r, C.c_double)))
+        first = np.concatenate([[0], np.cumsum(nn)]).astype(np.int64)
+        return dict(i=np.repeat(np.arange(N, dtype=np.int32), nn), j=ni, S=S, xyz=xyz, r=r, first_neigh=first,
+                    num_neigh=nn, neigh_types=nty)

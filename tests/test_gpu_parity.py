@@ -336,3 +336,62 @@ def test_calculator_energy_forces_stress(gpu, tmp_models):
             return calc.compute(pos @ S.T, np.diag(cell) @ S.T, Z)["energy"]
         d = (strained(h) - strained(-h)) / (2 * h) / V
         assert d == pytest.approx(stress[q], abs=1e-6)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("case", ["ortho", "triclinic", "small_cell", "open", "empty"])
+def test_device_neighbor_list_is_bit_identical_to_the_host_builder(case):
+    """Edge order, integer arrays, xyz and r of the device builder against symmetrix_amd.neighbors.neighbor_list."""
+    import torch
+    from symmetrix_amd import neighbors
+    rng = np.random.default_rng(11)
+    pbc = (True, True, True)
+    if case == "ortho":
+        cell = np.array([13.0, 11.0, 12.5]); pos = rng.uniform(0, 1, size=(300, 3)) * cell; rc = 4.5
+    elif case == "triclinic":
+        cell = np.array([[9.0, 0.0, 0.0], [2.5, 8.0, 0.0], [-1.5, 2.0, 10.0]])
+        pos = rng.uniform(0, 1, size=(150, 3)) @ cell; rc = 5.0
+    elif case == "small_cell":
+        cell = np.array([3.1, 3.3, 2.9]); pos = rng.uniform(0, 1, size=(5, 3)) * cell; rc = 5.0   # several images per pair
+    elif case == "open":
+        cell = np.array([30.0, 30.0, 30.0]); pos = rng.uniform(5, 12, size=(60, 3)); rc = 4.0; pbc = (False, True, False)
+    else:
+        cell = np.array([10.0, 10.0, 10.0]); pos = np.zeros((0, 3)); rc = 4.0
+    types = rng.integers(0, 3, size=len(pos)).astype(np.int32)
+    ref = neighbors.neighbor_list(pos, cell, rc, pbc)
+    dpos = torch.from_numpy(np.ascontiguousarray(pos)).cuda()
+    dty = torch.from_numpy(types).cuda()
+    dnl = neighbors.DeviceNeighborList()
+    print(f"case {case} atoms={len(pos)} edges={len(ref['r'])}", flush=True)
+    E = dnl.build(len(pos), dpos.data_ptr(), dty.data_ptr(), cell, rc, pbc)
+    got = dnl.to_host()
+    assert E == len(ref["r"])
+    assert np.array_equal(got["i"], ref["i"]) and np.array_equal(got["j"], ref["j"])
+    assert np.array_equal(got["S"], ref["S"].reshape(-1, 3))
+    assert np.array_equal(got["xyz"], ref["xyz"].reshape(-1, 3)) and np.array_equal(got["r"], ref["r"])
+    assert np.array_equal(got["first_neigh"], ref["first_neigh"])
+    assert np.array_equal(got["neigh_types"], types[ref["j"]])
+
+
+@pytest.mark.gpu
+def test_device_resident_loop_positions_to_forces(gpu, tmp_models):
+    """positions on the device -> device neighbour list -> compute_device -> per-atom forces, against the host path."""
+    import torch
+    from symmetrix_amd import neighbors
+    model = H.tiny_model(K=16, L_max=1, n_pts=48, seed=5)
+    path = H.write_model(model, tmp_models / "loop.json")
+    eng = gpu(path)
+    pos, cell, sp = H.small_system(40, seed=8)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    e_ref, f_ref = eng.node_energies.copy(), eng.node_forces.copy()
+    dpos = torch.from_numpy(np.ascontiguousarray(pos)).cuda()
+    dty = torch.from_numpy(np.asarray(sp, dtype=np.int32)).cuda()
+    dnl = neighbors.DeviceNeighborList()
+    E = dnl.build(len(pos), dpos.data_ptr(), dty.data_ptr(), cell, model["r_cut"])
+    oE = torch.zeros(len(pos), dtype=torch.float64, device="cuda"); oF = torch.zeros(3 * E, dtype=torch.float64, device="cuda")
+    p = dnl.ptr
+    eng.compute_device(len(pos), dty.data_ptr(), p["num_neigh"], p["neigh_indices"], p["neigh_types"], p["xyz"], p["r"], E,
+                       oE.data_ptr(), oF.data_ptr(), torch.cuda.current_stream().cuda_stream)
+    torch.cuda.synchronize()
+    assert np.array_equal(oE.cpu().numpy(), e_ref) and np.array_equal(oF.cpu().numpy(), f_ref)

@@ -48,6 +48,21 @@ def test_empty_and_open_boundaries():
     assert len(nl["i"]) == 2                          # no image across the open direction
 
 
+def test_no_atoms_and_image_shift_table():
+    nl = neighbors.neighbor_list(np.zeros((0, 3)), [10.0, 10.0, 10.0], 4.0)
+    assert len(nl["r"]) == 0 and list(nl["first_neigh"]) == [0]
+    cell = np.array([[4.0, 0.0, 0.0], [1.0, 5.0, 0.0], [0.0, 0.0, 30.0]])
+    ints, vecs = neighbors.image_shifts(cell, 4.5, pbc=(True, True, False))
+    # two shells along a (height 4.0 below the cutoff), one along b, none along the open axis; lexicographic
+    assert ints.shape == (15, 3) and np.array_equal(ints[0], [-2, -1, 0]) and np.array_equal(ints[-1], [2, 1, 0])
+    assert [tuple(t) for t in ints] == sorted(tuple(t) for t in ints)
+    assert np.array_equal(vecs, ints.astype(float) @ cell)
+    # every shift the list uses is in the table
+    pos = np.random.default_rng(0).uniform(0, 1, size=(12, 3)) @ cell
+    used = {tuple(t) for t in neighbors.neighbor_list(pos, cell, 4.5, (True, True, False))["S"]}
+    assert used <= {tuple(t) for t in ints}
+
+
 def test_real_cg_couples_harmonics():
     rng = np.random.default_rng(0)
     u = rng.normal(size=(6, 3))

@@ -174,13 +174,22 @@ int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const
  * lexicographic order; (0,0,0) marks the shift for which a pair i == j is no edge) and
  * shift_vec[num_shifts][3] = shift . cell in Cartesian coordinates (host arrays).  d_positions[num_atoms][3]
  * and d_types[num_atoms] (may be NULL) are device arrays.  Edge vectors are (x_j + shift) - x_i and
- * r = sqrt((d0*d0 + d1*d1) + d2*d2), every operation rounded once.  The arrays stay on the device and belong to
- * the list object until the next build; their addresses can be handed to smx_compute_device. */
+ * r = sqrt((d0*d0 + d1*d1) + d2*d2), every operation rounded once.  Pairs closer than r_list >= r_cut are
+ * remembered (r_list - r_cut is the skin that smx_nlist_update relies on; the shift list must cover r_list); the
+ * edges are those closer than r_cut.  The arrays stay on the device and belong to the list object until the next
+ * build or update; their addresses can be handed to smx_compute_device. */
 typedef struct smx_nlist smx_nlist;
 smx_nlist* smx_nlist_create(void);
 void smx_nlist_free(smx_nlist* nl);
 int smx_nlist_build(smx_nlist* nl, int num_atoms, const double* d_positions, const int* d_types, int num_shifts,
-                    const int* shift_int, const double* shift_vec, double r_cut, void* stream, long* num_edges);
+                    const int* shift_int, const double* shift_vec, double r_list, double r_cut, void* stream,
+                    long* num_edges);
+/* Same list from new positions without a new search: the pairs found within r_list by the last build are
+ * re-measured and those inside r_cut kept, in the same canonical order (the cutoff filter that the LAMMPS caller
+ * applies to its skin list every step, pair_symmetrix_mace.cpp:287-315).  Equal to a fresh build at r_cut as long
+ * as no pair outside r_list at build time has come inside r_cut since. */
+int smx_nlist_update(smx_nlist* nl, const double* d_positions, const int* d_types, double r_cut, void* stream,
+                     long* num_edges);
 int smx_nlist_arrays(smx_nlist* nl, const int** num_neigh, const int** first_neigh, const int** neigh_indices,
                      const int** neigh_types, const int** neigh_shift, const double** xyz, const double** r);
 int smx_nlist_copy_to_host(smx_nlist* nl, int* num_neigh, int* neigh_indices, int* neigh_types, int* neigh_shift,

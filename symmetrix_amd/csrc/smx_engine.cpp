@@ -1118,26 +1118,25 @@ smx::EngineBase& E(smx_model* m)
 namespace smx {
 struct NeighborList {
     DVec<double> part, shift_vec, xyz, r;
-    DVec<int> shift_int, atom_bin, bin_count, bin_start, bin_atoms, count, first, num_neigh, neigh_indices, neigh_types,
-        neigh_shift, scan_tmp;
-    DVec<long long> keys;
-    int N = 0;
-    long E = 0;
+    DVec<int> shift_int, atom_bin, bin_count, bin_start, bin_atoms, count, cfirst, first, num_neigh, neigh_indices,
+        neigh_types, neigh_shift, scan_tmp;
+    DVec<long long> keys, sorted;
+    int N = 0, num_shifts = 0;
+    long E = 0, num_candidates = 0;
+    double r_list = 0.0;
 
-    long build(int N_, const double* d_pos, const int* d_types, int num_shifts, const int* h_shift_int,
-               const double* h_shift_vec, double r_cut, hipStream_t s)
+    // candidates: every (receiver, sender, image) closer than r_list, sorted per receiver
+    void build(int N_, const double* d_pos, int num_shifts_, const int* h_shift_int, const double* h_shift_vec,
+               double r_list_, hipStream_t s)
     {
-        if (N_ < 0 || num_shifts <= 0 || !(r_cut > 0.0) || !h_shift_int || !h_shift_vec || (N_ > 0 && !d_pos))
+        if (N_ < 0 || num_shifts_ <= 0 || !(r_list_ > 0.0) || !h_shift_int || !h_shift_vec || (N_ > 0 && !d_pos))
             throw Error(SMX_EINVAL, "neighbour list: bad arguments");
         int zero_shift = -1;
-        for (int q = 0; q < num_shifts; ++q)
+        for (int q = 0; q < num_shifts_; ++q)
             if (h_shift_int[3 * q] == 0 && h_shift_int[3 * q + 1] == 0 && h_shift_int[3 * q + 2] == 0) zero_shift = q;
-        N = N_; E = 0;
-        first.size_to((size_t)N + 1, s); num_neigh.size_to((size_t)N, s);
-        if (N == 0) {
-            HIPCHK(hipMemsetAsync(first.p, 0, sizeof(int), s));
-            return 0;
-        }
+        N = N_; num_shifts = num_shifts_; r_list = r_list_; E = 0; num_candidates = 0;
+        cfirst.size_to((size_t)N + 1, s);
+        if (N == 0) return;
         shift_int.upload(h_shift_int, (size_t)3 * num_shifts, s);
         shift_vec.upload(h_shift_vec, (size_t)3 * num_shifts, s);
         // bounding box (per-block partials, finished on the host)
@@ -1152,10 +1151,10 @@ struct NeighborList {
         for (int k = 0; k < 3; ++k) {
             double lo = 1e300, hi = -1e300;
             for (int b = 0; b < nblk; ++b) { lo = std::min(lo, hp[(size_t)b * 6 + k]); hi = std::max(hi, hp[(size_t)b * 6 + 3 + k]); }
-            if (!(lo <= hi)) throw Error(SMX_EINVAL, "neighbour list: positions are not finite");
+            if (!(lo <= hi) || !(hi - lo < 1e300)) throw Error(SMX_EINVAL, "neighbour list: positions are not finite");
             g.lo[k] = lo; g.hi[k] = hi;
             const double ext = hi - lo;
-            int nb = (int)std::floor(ext / r_cut);
+            int nb = (int)std::floor(std::min(ext / r_list, 1e6));
             nb = std::max(1, std::min(nb, 128));
             g.nb[k] = nb;
             g.inv_bs[k] = ext > 0.0 ? nb / ext : 0.0;
@@ -1168,20 +1167,42 @@ struct NeighborList {
         HIPCHK(launch_scan_exclusive(bin_count.p, bin_start.p, (int)nbins, scan_tmp.p, s));
         HIPCHK(launch_nl_bin_fill(N, atom_bin.p, bin_start.p, bin_count.p + nbins, bin_atoms.p, s));
         count.size_to((size_t)N, s);
-        HIPCHK(launch_nl_search(false, d_pos, N, g, bin_start.p, bin_atoms.p, num_shifts, shift_vec.p, zero_shift, r_cut,
+        HIPCHK(launch_nl_search(false, d_pos, N, g, bin_start.p, bin_atoms.p, num_shifts, shift_vec.p, zero_shift, r_list,
                                 count.p, nullptr, nullptr, s));
-        HIPCHK(launch_scan_exclusive(count.p, first.p, N, scan_tmp.p, s));
+        HIPCHK(launch_scan_exclusive(count.p, cfirst.p, N, scan_tmp.p, s));
+        int total = 0;
+        HIPCHK(hipMemcpyAsync(&total, cfirst.p + N, sizeof(int), hipMemcpyDeviceToHost, s));
+        HIPCHK(hipStreamSynchronize(s));
+        if (total < 0) throw Error(SMX_EINVAL, "neighbour list: more than 2^31 candidate pairs");
+        num_candidates = total;
+        keys.size_to((size_t)num_candidates, s); sorted.size_to((size_t)num_candidates, s);
+        HIPCHK(launch_nl_search(true, d_pos, N, g, bin_start.p, bin_atoms.p, num_shifts, shift_vec.p, zero_shift, r_list,
+                                nullptr, cfirst.p, keys.p, s));
+        HIPCHK(launch_nl_sort(N, cfirst.p, keys.p, sorted.p, s));
+    }
+
+    // edges: the candidates closer than r_cut at the given positions, in candidate order
+    long update(const double* d_pos, const int* d_types, double r_cut, hipStream_t s)
+    {
+        if (!(r_cut > 0.0) || r_cut > r_list || (N > 0 && !d_pos))
+            throw Error(SMX_EINVAL, "neighbour list: the cutoff must be positive and no larger than the radius of the last build");
+        E = 0;
+        first.size_to((size_t)N + 1, s); num_neigh.size_to((size_t)N, s);
+        if (N == 0) {
+            HIPCHK(hipMemsetAsync(first.p, 0, sizeof(int), s));
+            return 0;
+        }
+        HIPCHK(launch_nl_filter(false, d_pos, d_types, N, cfirst.p, sorted.p, num_shifts, shift_vec.p, shift_int.p, r_cut,
+                                num_neigh.p, nullptr, nullptr, nullptr, nullptr, nullptr, nullptr, s));
+        HIPCHK(launch_scan_exclusive(num_neigh.p, first.p, N, scan_tmp.p, s));
         int total = 0;
         HIPCHK(hipMemcpyAsync(&total, first.p + N, sizeof(int), hipMemcpyDeviceToHost, s));
         HIPCHK(hipStreamSynchronize(s));
         E = total;
-        keys.size_to((size_t)E, s);
         neigh_indices.size_to((size_t)E, s); neigh_types.size_to((size_t)E, s); neigh_shift.size_to((size_t)3 * E, s);
         xyz.size_to((size_t)3 * E, s); r.size_to((size_t)E, s);
-        HIPCHK(launch_nl_search(true, d_pos, N, g, bin_start.p, bin_atoms.p, num_shifts, shift_vec.p, zero_shift, r_cut,
-                                nullptr, first.p, keys.p, s));
-        HIPCHK(launch_nl_emit(d_pos, d_types, N, first.p, keys.p, num_shifts, shift_vec.p, shift_int.p, num_neigh.p,
-                              neigh_indices.p, neigh_types.p, neigh_shift.p, xyz.p, r.p, s));
+        HIPCHK(launch_nl_filter(true, d_pos, d_types, N, cfirst.p, sorted.p, num_shifts, shift_vec.p, shift_int.p, r_cut,
+                                nullptr, first.p, neigh_indices.p, neigh_types.p, neigh_shift.p, xyz.p, r.p, s));
         return E;
     }
 };
@@ -1455,12 +1476,24 @@ smx_nlist* smx_nlist_create(void)
 }
 void smx_nlist_free(smx_nlist* nl) { delete reinterpret_cast<smx::NeighborList*>(nl); }
 int smx_nlist_build(smx_nlist* nl, int num_atoms, const double* d_positions, const int* d_types, int num_shifts,
-                    const int* shift_int, const double* shift_vec, double r_cut, void* stream, long* num_edges)
+                    const int* shift_int, const double* shift_vec, double r_list, double r_cut, void* stream,
+                    long* num_edges)
 {
     return guarded([&] {
         if (!nl || !shift_int || !shift_vec || (num_atoms > 0 && !d_positions)) throw smx::Error(SMX_EINVAL, "null argument");
-        const long e = reinterpret_cast<smx::NeighborList*>(nl)->build(num_atoms, d_positions, d_types, num_shifts,
-                                                                      shift_int, shift_vec, r_cut, (hipStream_t)stream);
+        if (!(r_cut > 0.0) || r_cut > r_list) throw smx::Error(SMX_EINVAL, "neighbour list: need 0 < r_cut <= r_list");
+        auto& n = *reinterpret_cast<smx::NeighborList*>(nl);
+        n.build(num_atoms, d_positions, num_shifts, shift_int, shift_vec, r_list, (hipStream_t)stream);
+        const long e = n.update(d_positions, d_types, r_cut, (hipStream_t)stream);
+        if (num_edges) *num_edges = e;
+    });
+}
+int smx_nlist_update(smx_nlist* nl, const double* d_positions, const int* d_types, double r_cut, void* stream,
+                     long* num_edges)
+{
+    return guarded([&] {
+        if (!nl) throw smx::Error(SMX_EINVAL, "null argument");
+        const long e = reinterpret_cast<smx::NeighborList*>(nl)->update(d_positions, d_types, r_cut, (hipStream_t)stream);
         if (num_edges) *num_edges = e;
     });
 }

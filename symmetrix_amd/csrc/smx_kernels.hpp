@@ -99,10 +99,11 @@ hipError_t launch_nl_bin_fill(int N, const int* atom_bin, const int* bin_start, 
 hipError_t launch_nl_search(bool fill, const double* pos, int N, const NlGrid& g, const int* bin_start,
                             const int* bin_atoms, int num_shifts, const double* shift_vec, int zero_shift,
                             double r_cut, int* count, const int* first, long long* keys, hipStream_t s);
-hipError_t launch_nl_emit(const double* pos, const int* types, int N, const int* first, const long long* keys,
-                          int num_shifts, const double* shift_vec, const int* shift_int, int* num_neigh,
-                          int* neigh_indices, int* neigh_types, int* neigh_shift, double* xyz, double* r,
-                          hipStream_t s);
+hipError_t launch_nl_sort(int N, const int* cfirst, const long long* keys, long long* sorted, hipStream_t s);
+hipError_t launch_nl_filter(bool emit, const double* pos, const int* types, int N, const int* cfirst,
+                            const long long* sorted, int num_shifts, const double* shift_vec, const int* shift_int,
+                            double r_cut, int* count, const int* first, int* neigh_indices, int* neigh_types,
+                            int* neigh_shift, double* xyz, double* r, hipStream_t s);
 
 // ---------------------------------------------------------------------------
 // Pair terms of the edge length alone (smx_kernels_pair.hip)

@@ -76,7 +76,7 @@ __global__ void k_nl_bin_fill(int N, const int* atom_bin, const int* bin_start, 
 
 // One thread per receiver walks every image shift and the bins that the cutoff sphere of the shifted
 // receiver can touch.  FILL = false counts, FILL = true writes the keys sender * num_shifts + shift index
-// (in whatever order the bins deliver them: k_nl_emit sorts).
+// (in whatever order the bins deliver them: k_nl_sort orders them).
 template <bool FILL>
 __global__ void k_nl_search(const double* pos, int N, NlGrid g, const int* bin_start, const int* bin_atoms,
                             int num_shifts, const double* shift_vec, int zero_shift, double r_cut, double r2cut,
@@ -117,33 +117,59 @@ __global__ void k_nl_search(const double* pos, int N, NlGrid g, const int* bin_s
     if (!FILL) count[i] = c;
 }
 
-// One wavefront per receiver: rank of every key among the receiver's keys (they are distinct), then the
-// edge arrays written at first[i] + rank.
-__global__ __launch_bounds__(256) void k_nl_emit(const double* pos, const int* types, int N, const int* first,
-                                                 const long long* keys, int num_shifts, const double* shift_vec,
-                                                 const int* shift_int, int* num_neigh, int* neigh_indices,
-                                                 int* neigh_types, int* neigh_shift, double* xyz, double* r)
+// One wavefront per receiver: rank of every key among the receiver's keys (they are distinct); the keys are
+// rewritten in ascending order, which is the canonical edge order of the receiver.
+__global__ __launch_bounds__(256) void k_nl_sort(int N, const int* cfirst, const long long* keys, long long* sorted)
 {
     const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     if (i >= N) return;
-    const int e0 = first[i], n = first[i + 1] - e0;
-    if (lane == 0) num_neigh[i] = n;
+    const int e0 = cfirst[i], n = cfirst[i + 1] - e0;
     for (int a = lane; a < n; a += 64) {
         const long long key = keys[e0 + a];
         int rank = 0;
         for (int b = 0; b < n; ++b) rank += keys[e0 + b] < key ? 1 : 0;
-        const int j = (int)(key / num_shifts), s = (int)(key % num_shifts);
-        const Cand cd = displacement(pos, i, j, shift_vec + 3 * s);
-        const size_t e = (size_t)e0 + rank;
-        neigh_indices[e] = j;
-        neigh_types[e] = types ? types[j] : 0;
-        if (neigh_shift) {
+        sorted[(size_t)e0 + rank] = key;
+    }
+}
+
+// One wavefront per receiver walks its sorted candidates with the current positions and keeps those inside
+// the cutoff, in order.  EMIT = false counts; EMIT = true writes the edge arrays at first[i] + (number kept before).
+template <bool EMIT>
+__global__ __launch_bounds__(256) void k_nl_filter(const double* pos, const int* types, int N, const int* cfirst,
+                                                   const long long* sorted, int num_shifts, const double* shift_vec,
+                                                   const int* shift_int, double r2cut, int* count, const int* first,
+                                                   int* neigh_indices, int* neigh_types, int* neigh_shift, double* xyz,
+                                                   double* r)
+{
+    const int i = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    if (i >= N) return;
+    const int c0 = cfirst[i], n = cfirst[i + 1] - c0;
+    int kept = 0;
+    const size_t e0 = EMIT ? (size_t)first[i] : 0;
+    for (int a0 = 0; a0 < n; a0 += 64) {
+        const int a = a0 + lane;
+        bool pass = false;
+        int j = 0, s = 0;
+        Cand cd{};
+        if (a < n) {
+            const long long key = sorted[(size_t)c0 + a];
+            j = (int)(key / num_shifts); s = (int)(key % num_shifts);
+            cd = displacement(pos, i, j, shift_vec + 3 * s);
+            pass = cd.r2 < r2cut;
+        }
+        const unsigned long long mask = __ballot(pass);
+        if (EMIT && pass) {
+            const size_t e = e0 + kept + __popcll(mask & ((1ull << lane) - 1ull));
+            neigh_indices[e] = j;
+            neigh_types[e] = types ? types[j] : 0;
             neigh_shift[3 * e] = shift_int[3 * s]; neigh_shift[3 * e + 1] = shift_int[3 * s + 1];
             neigh_shift[3 * e + 2] = shift_int[3 * s + 2];
+            xyz[3 * e] = cd.d0; xyz[3 * e + 1] = cd.d1; xyz[3 * e + 2] = cd.d2;
+            r[e] = __dsqrt_rn(cd.r2);
         }
-        xyz[3 * e] = cd.d0; xyz[3 * e + 1] = cd.d1; xyz[3 * e + 2] = cd.d2;
-        r[e] = __dsqrt_rn(cd.r2);
+        kept += __popcll(mask);
     }
+    if (!EMIT && lane == 0) count[i] = kept;
 }
 
 }  // namespace
@@ -178,14 +204,24 @@ hipError_t launch_nl_search(bool fill, const double* pos, int N, const NlGrid& g
                            num_shifts, shift_vec, zero_shift, r_cut, r2cut, count, first, keys);
     return hipGetLastError();
 }
-hipError_t launch_nl_emit(const double* pos, const int* types, int N, const int* first, const long long* keys,
-                          int num_shifts, const double* shift_vec, const int* shift_int, int* num_neigh,
-                          int* neigh_indices, int* neigh_types, int* neigh_shift, double* xyz, double* r,
-                          hipStream_t s)
+hipError_t launch_nl_sort(int N, const int* cfirst, const long long* keys, long long* sorted, hipStream_t s)
 {
-    if (N > 0)
-        hipLaunchKernelGGL(k_nl_emit, dim3((N + 3) / 4), dim3(256), 0, s, pos, types, N, first, keys, num_shifts,
-                           shift_vec, shift_int, num_neigh, neigh_indices, neigh_types, neigh_shift, xyz, r);
+    if (N > 0) hipLaunchKernelGGL(k_nl_sort, dim3((N + 3) / 4), dim3(256), 0, s, N, cfirst, keys, sorted);
+    return hipGetLastError();
+}
+hipError_t launch_nl_filter(bool emit, const double* pos, const int* types, int N, const int* cfirst,
+                            const long long* sorted, int num_shifts, const double* shift_vec, const int* shift_int,
+                            double r_cut, int* count, const int* first, int* neigh_indices, int* neigh_types,
+                            int* neigh_shift, double* xyz, double* r, hipStream_t s)
+{
+    if (N <= 0) return hipSuccess;
+    const double r2cut = r_cut * r_cut;
+    if (emit)
+        hipLaunchKernelGGL(k_nl_filter<true>, dim3((N + 3) / 4), dim3(256), 0, s, pos, types, N, cfirst, sorted, num_shifts,
+                           shift_vec, shift_int, r2cut, count, first, neigh_indices, neigh_types, neigh_shift, xyz, r);
+    else
+        hipLaunchKernelGGL(k_nl_filter<false>, dim3((N + 3) / 4), dim3(256), 0, s, pos, types, N, cfirst, sorted, num_shifts,
+                           shift_vec, shift_int, r2cut, count, first, neigh_indices, neigh_types, neigh_shift, xyz, r);
     return hipGetLastError();
 }
 

@@ -210,20 +210,36 @@ class DeviceNeighborList:
         except Exception:
             pass
 
-    def build(self, num_atoms, positions_ptr, types_ptr, cell, r_cut, pbc=(True, True, True), stream=0):
+    _names = ("num_neigh", "first_neigh", "neigh_indices", "neigh_types", "neigh_shift", "xyz", "r")
+
+    def _refresh(self, E):
         C = self._C
-        ints, vecs = image_shifts(cell, r_cut, pbc)
+        self.num_edges = int(E)
+        out = [C.c_void_p(0) for _ in self._names]
+        self._lib.check(self._L.smx_nlist_arrays(C.c_void_p(self._h), *[C.byref(o) for o in out]))
+        self.ptr = {n: (o.value or 0) for n, o in zip(self._names, out)}
+        return self.num_edges
+
+    def build(self, num_atoms, positions_ptr, types_ptr, cell, r_cut, pbc=(True, True, True), skin=0.0, stream=0):
+        """New search: pairs within r_cut + skin are remembered, edges are the pairs within r_cut."""
+        C = self._C
+        r_list = float(r_cut) + float(skin)
+        ints, vecs = image_shifts(cell, r_list, pbc)
         E = C.c_long(0)
         self._lib.check(self._L.smx_nlist_build(
             C.c_void_p(self._h), int(num_atoms), C.c_void_p(positions_ptr), C.c_void_p(types_ptr or 0), len(ints),
-            ints.ctypes.data_as(C.POINTER(C.c_int)), vecs.ctypes.data_as(C.POINTER(C.c_double)), C.c_double(r_cut),
-            C.c_void_p(stream), C.byref(E)))
-        self.num_atoms, self.num_edges = int(num_atoms), int(E.value)
-        names = ("num_neigh", "first_neigh", "neigh_indices", "neigh_types", "neigh_shift", "xyz", "r")
-        out = [C.c_void_p(0) for _ in names]
-        self._lib.check(self._L.smx_nlist_arrays(C.c_void_p(self._h), *[C.byref(o) for o in out]))
-        self.ptr = {n: (o.value or 0) for n, o in zip(names, out)}
-        return self.num_edges
+            ints.ctypes.data_as(C.POINTER(C.c_int)), vecs.ctypes.data_as(C.POINTER(C.c_double)), C.c_double(r_list),
+            C.c_double(r_cut), C.c_void_p(stream), C.byref(E)))
+        self.num_atoms = int(num_atoms)
+        return self._refresh(E.value)
+
+    def update(self, positions_ptr, types_ptr, r_cut, stream=0):
+        """Edges within r_cut at new positions, from the pairs remembered by the last build (no new search)."""
+        C = self._C
+        E = C.c_long(0)
+        self._lib.check(self._L.smx_nlist_update(C.c_void_p(self._h), C.c_void_p(positions_ptr), C.c_void_p(types_ptr or 0),
+                                                 C.c_double(r_cut), C.c_void_p(stream), C.byref(E)))
+        return self._refresh(E.value)
 
     def to_host(self):
         C = self._C

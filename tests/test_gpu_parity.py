@@ -374,6 +374,33 @@ def test_device_neighbor_list_is_bit_identical_to_the_host_builder(case):
 
 
 @pytest.mark.gpu
+def test_device_neighbor_list_update_equals_fresh_build():
+    """Skin list + per-step cutoff filter at moved positions against a fresh host build at the moved positions."""
+    import torch
+    from symmetrix_amd import neighbors
+    rng = np.random.default_rng(3)
+    cell = np.array([[12.0, 0.0, 0.0], [1.0, 11.0, 0.0], [0.5, -1.0, 12.5]])
+    pos = rng.uniform(0, 1, size=(400, 3)) @ cell
+    types = rng.integers(0, 4, size=len(pos)).astype(np.int32)
+    rc, skin = 4.5, 1.0
+    dnl = neighbors.DeviceNeighborList()
+    dty = torch.from_numpy(types).cuda()
+    dpos = torch.from_numpy(pos).cuda()
+    dnl.build(len(pos), dpos.data_ptr(), dty.data_ptr(), cell, rc, skin=skin)
+    for step in range(3):
+        pos = pos + rng.uniform(-0.15, 0.15, size=pos.shape)      # total drift stays below skin / 2
+        dpos = torch.from_numpy(pos).cuda()
+        print(f"update step {step}", flush=True)
+        E = dnl.update(dpos.data_ptr(), dty.data_ptr(), rc)
+        got, ref = dnl.to_host(), neighbors.neighbor_list(pos, cell, rc)
+        assert E == len(ref["r"])
+        for k in ("i", "j", "S", "xyz", "r", "first_neigh"):
+            assert np.array_equal(got[k], ref[k].reshape(got[k].shape)), k
+    with pytest.raises(ValueError):
+        dnl.update(dpos.data_ptr(), dty.data_ptr(), rc + 2 * skin)
+
+
+@pytest.mark.gpu
 def test_device_resident_loop_positions_to_forces(gpu, tmp_models):
     """positions on the device -> device neighbour list -> compute_device -> per-atom forces, against the host path."""
     import torch

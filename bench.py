@@ -64,20 +64,154 @@ def algorithmic_bytes(stage, N, E, K, s, n_LM, n_e):
     return table.get(stage)
 
 
+def run_capacity(args):
+    """Capacity run: the l <= 1 water model on a box of about --atoms atoms, MD-style steps.
+
+    Every step moves all atoms by N(0, 0.01^2) on the device, refreshes the edge list on the device (a new search
+    with a skin every --rebuild-every steps, the cutoff filter of the remembered pairs otherwise) and evaluates
+    energies and edge forces.  Nothing but the edge count crosses to the host.  The box is a small random water box
+    repeated 4 x 4 x 4 times, so that before the first move every copy of an atom must get the same energy and
+    force: that is checked at full size and reported.
+    """
+    import torch
+    from symmetrix_amd import modelgen, neighbors, systems
+    from symmetrix_amd.mace import MACE
+
+    dev = torch.device("cuda:0")
+    cfg = dict(modelgen.CONFIGS["off_medium"])
+    cfg["pair_dependent_radial"] = False
+    model_path = os.path.join(args.model_dir, "smx_bench_off_medium.json")
+    if not os.path.exists(model_path):
+        modelgen.write_model(model_path, **cfg)
+    reps = 4
+    n_mol = max(4, -(-args.atoms // (3 * reps ** 3)))
+    bpos, bcell, bsp = systems.water_box(n_mol, seed=0)
+    nb = len(bpos)
+    offs = np.array([[a, b, c] for a in range(reps) for b in range(reps) for c in range(reps)], dtype=np.float64) * bcell
+    pos = (offs[:, None, :] + bpos[None, :, :]).reshape(-1, 3)
+    species = np.tile(bsp, reps ** 3).astype(np.int32)
+    cell = bcell * reps
+    N = len(pos)
+    r_cut, skin = cfg["r_cut"], args.skin
+    dpos = torch.from_numpy(np.ascontiguousarray(pos)).to(dev)
+    dty = torch.from_numpy(species).to(dev)
+    del pos
+    eng = MACE(model_path, args.dtype)
+    nl = neighbors.DeviceNeighborList()
+    stream = torch.cuda.current_stream().cuda_stream
+    out_E = torch.zeros(N, dtype=torch.float64, device=dev)
+    out_F = None
+
+    def evaluate(E):
+        nonlocal out_F
+        if out_F is None or out_F.numel() < 3 * E:
+            out_F = torch.zeros(int(3 * E * 1.05), dtype=torch.float64, device=dev)
+        p = nl.ptr
+        eng.compute_device(N, dty.data_ptr(), p["num_neigh"], p["neigh_indices"], p["neigh_types"], p["xyz"], p["r"], E,
+                           out_E.data_ptr(), out_F.data_ptr(), stream)
+
+    # ---- before any move: all 64 copies of the small box must agree
+    E = nl.build(N, dpos.data_ptr(), dty.data_ptr(), cell, r_cut, skin=skin)
+    evaluate(E)
+    torch.cuda.synchronize()
+    num_neigh = torch.empty(N, dtype=torch.int32, device=dev)
+    neigh = torch.empty(E, dtype=torch.int32, device=dev)
+
+    class DeviceInts:   # zero-copy view of a device array of the list object
+        def __init__(self, ptr, n):
+            self.__cuda_array_interface__ = dict(shape=(n,), typestr="<i4", data=(ptr, False), version=2)
+
+    num_neigh.copy_(torch.as_tensor(DeviceInts(nl.ptr["num_neigh"], N), device=dev))
+    neigh.copy_(torch.as_tensor(DeviceInts(nl.ptr["neigh_indices"], E), device=dev))
+    recv = torch.repeat_interleave(torch.arange(N, device=dev), num_neigh.long())
+    f = out_F[:3 * E].view(E, 3)
+    fa = torch.zeros(N, 3, dtype=torch.float64, device=dev)
+    fa.index_add_(0, neigh.long(), f)
+    fa.index_add_(0, recv, -f)
+    e_rep = out_E.view(reps ** 3, nb)
+    f_rep = fa.view(reps ** 3, nb, 3)
+    e_dev = float((e_rep - e_rep[0]).abs().max().item())
+    f_dev = float((f_rep - f_rep[0]).abs().max().item())
+    e_scale = float(e_rep[0].abs().max().item())
+    energy0 = float(out_E.sum().item())
+    del num_neigh, neigh, recv, fa, f, e_rep, f_rep
+    torch.cuda.empty_cache()
+
+    # ---- MD-style steps
+    gen = torch.Generator(device=dev)
+    gen.manual_seed(0)
+    t_list_build, t_list_update, t_eval, t_step = [], [], [], []
+    edges = []
+    total = args.warmup + args.steps
+    for it in range(total):
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dpos.add_(torch.randn(dpos.shape, dtype=torch.float64, device=dev, generator=gen), alpha=0.01)
+        rebuild = it % args.rebuild_every == 0
+        if rebuild:
+            E = nl.build(N, dpos.data_ptr(), dty.data_ptr(), cell, r_cut, skin=skin)
+        else:
+            E = nl.update(dpos.data_ptr(), dty.data_ptr(), r_cut)
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        evaluate(E)
+        torch.cuda.synchronize()
+        t2 = time.perf_counter()
+        if it >= args.warmup:
+            (t_list_build if rebuild else t_list_update).append(t1 - t0)
+            t_eval.append(t2 - t1)
+            t_step.append(t2 - t0)
+            edges.append(E)
+        if it % 10 == 0:
+            print(f"[capacity] step {it}/{total} edges={E} step={1e3 * (t2 - t0):.1f} ms", file=sys.stderr, flush=True)
+    free_b, total_b = torch.cuda.mem_get_info()
+    ms = 1e3 * float(np.mean(t_step))
+    K, L_max = cfg["num_channels"], cfg["L_max"]
+    line = {
+        "metric": "atom-steps/s per MI355X (energy+forces)", "value": N / (ms * 1e-3), "unit": "atom-steps/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None,
+        "dtype": "f64" if args.dtype == "float64" else "f32-features/f64-accumulation", "data": "synthetic",
+        "config": {
+            "workload": f"water_capacity: {N} atoms ({reps}^3 copies of a {nb}-atom water box, moved by N(0, 0.01^2) A every "
+                        f"step), about {int(np.mean(edges))} edges, K={K}, L_max={L_max}, r_cut={r_cut}, device neighbour list "
+                        f"with skin {skin} A searched anew every {args.rebuild_every} steps and filtered every step",
+            "atoms": N, "edges_mean": float(np.mean(edges)), "channels": K, "L_max": L_max,
+        },
+        "step_breakdown_ms": {
+            "evaluation": 1e3 * float(np.mean(t_eval)),
+            "move_and_list_search": 1e3 * float(np.mean(t_list_build)) if t_list_build else None,
+            "move_and_list_filter": 1e3 * float(np.mean(t_list_update)) if t_list_update else None,
+        },
+        "evaluation_only_value": N / float(np.mean(t_eval)),
+        "hbm_in_use_GB": (total_b - free_b) / 1e9,
+        "copies_check": {"energy_max_abs_diff": e_dev, "energy_scale": e_scale, "atom_force_max_abs_diff": f_dev,
+                         "note": "64 periodic copies of the small box before the first move: equal up to summation order"},
+        "energy_first": energy0,
+    }
+    print(json.dumps(line))
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="off_small", choices=["tiny", "off_small", "off_medium", "mp_medium"])
+    ap.add_argument("--workload", default="off_small", choices=["tiny", "off_small", "off_medium", "mp_medium", "water_capacity"])
+    ap.add_argument("--atoms", type=int, default=1000000, help="water_capacity: target atom count")
+    ap.add_argument("--rebuild-every", type=int, default=10, help="water_capacity: steps between neighbour searches")
+    ap.add_argument("--skin", type=float, default=0.6, help="water_capacity: list radius minus cutoff (Angstrom)")
     ap.add_argument("--scale", type=float, default=1.0, help="shrink the atom count (tests)")
-    ap.add_argument("--dtype", default="float64", choices=["float64", "float32"])
+    ap.add_argument("--dtype", default=None, choices=["float64", "float32"],
+                    help="default: float64, and float32 features for water_capacity")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-atoms", type=int, default=0, help="atoms in the CPU sample (0 = whole workload)")
     ap.add_argument("--model-dir", default=tempfile.gettempdir())
     ap.add_argument("--calibrate-copy", action="store_true",
                     help="also launch one device-to-device copy of 1 GiB (a kernel of known traffic for counter runs)")
     args = ap.parse_args()
+    if args.dtype is None:
+        args.dtype = "float32" if args.workload == "water_capacity" else "float64"
     if args.gpus != 1:
         print("bench.py: this build runs on exactly one GPU (no collectives exist in it); use --gpus 1", file=sys.stderr)
         sys.exit(2)
@@ -90,6 +224,8 @@ def main():
         print("bench.py: no GPU visible", file=sys.stderr)
         sys.exit(1)
     dev = torch.device("cuda:0")
+    if args.workload == "water_capacity":
+        return run_capacity(args)
 
     # ---- model file (seeded, random-init) and synthetic system
     cfg = dict(modelgen.CONFIGS[args.workload])

@@ -145,6 +145,12 @@ int smx_compute_readouts(smx_model* m, int num_nodes, const int* node_types);   
 int smx_get_array(smx_model* m, const char* name, double* out, long cap, long* n);
 int smx_set_array(smx_model* m, const char* name, const double* in, long n);
 
+/* Upper bound in bytes (default 32 GiB) for the buffer that stages the per-edge adjoint messages of reverse_Phi1
+ * (mace.cpp:579-604) in models with l <= 1 hidden features.  Longer edge lists are processed in receiver chunks that
+ * reuse the buffer; results do not depend on the limit.  No counterpart in the reference, which holds no per-edge
+ * staging. */
+int smx_set_staging_limit(smx_model* m, long bytes);
+
 /* Per-stage timing with HIP events on the stream the kernels run on.  When
  * enabled, every stage of the next compute is bracketed by events;
  * smx_get_stage_times synchronises and returns elapsed milliseconds per stage.

@@ -62,11 +62,18 @@ struct DVec {
     void reserve(size_t m, hipStream_t s, bool keep)
     {
         if (m <= cap) return;
-        size_t newcap = m + m / 8 + 64;
+        // headroom against regrowth when the edge count drifts: an eighth, a sixty-fourth for buffers beyond 1 GiB
+        const size_t newcap = m + (m * sizeof(T) > ((size_t)1 << 30) ? m / 64 : m / 8) + 64;
         T* q = nullptr;
+        if (p && !(keep && n)) {
+            // nothing to carry over: release first, so that the two sizes never coexist
+            HIPCHK(hipStreamSynchronize(s));
+            HIPCHK(hipFree(p));
+            p = nullptr; cap = 0;
+        }
         HIPCHK(hipMalloc(&q, newcap * sizeof(T)));
         if (p) {
-            if (keep && n) HIPCHK(hipMemcpyAsync(q, p, n * sizeof(T), hipMemcpyDeviceToDevice, s));
+            HIPCHK(hipMemcpyAsync(q, p, n * sizeof(T), hipMemcpyDeviceToDevice, s));
             HIPCHK(hipStreamSynchronize(s));
             HIPCHK(hipFree(p));
         }
@@ -112,6 +119,7 @@ struct EngineBase {
     hipEvent_t ev0[ST_COUNT] = {}, ev1[ST_COUNT] = {};
     bool ev_used[ST_COUNT] = {};
     int H1_rows_override = -1;
+    size_t msg_limit_bytes = (size_t)32 << 30;   // staging buffer of the layer-1 adjoint messages
 
     virtual void compute(int N, const int* node_types, const int* num_neigh, const int* neigh_indices,
                          const int* neigh_types, const double* xyz, const double* r, long E, bool on_device,
@@ -715,6 +723,13 @@ struct Engine : EngineBase {
         need(xyz, "xyz"); need(r, "r"); need(neigh_indices, "neigh_indices");
         const int k = K(), nlm = NLM();
         node_forces.resize((size_t)3 * E, stream);
+        H1_adj.resize(H1.n, stream);
+        const int rows = (int)(H1.n / ((size_t)nlm * k));
+        const size_t row_bytes = (size_t)nlm * k * sizeof(F);
+        if (!slice_CH1 && (size_t)E * row_bytes > msg_limit_bytes) {
+            agg1_bwd_chunked(N, rows, zero_dxyz, zero_H1_adj);
+            return;
+        }
         msg.size_to((size_t)E * nlm * k, stream);
         stage_begin(ST_AGG1B);
         if (slice_CH1) {
@@ -732,14 +747,58 @@ struct Engine : EngineBase {
             p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
             agg_bwd_general(hm.L_max, p, ST_AGG1B, ST_FSUM1);
         }
-        // edges beyond the first N receivers carry no layer-1 adjoint
-        const long EN = E;  // first_neigh[N] == E whenever the list covers exactly N receivers
-        (void)EN;
         stage_begin(ST_SRED);
-        H1_adj.resize(H1.n, stream);
-        const int rows = (int)(H1.n / ((size_t)nlm * k));
         if (sender_rows != rows) build_sender_lists(rows);
-        HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, stream));
+        HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, 0, E, stream));
+        stage_end(ST_SRED);
+    }
+    // The same stage for edge lists whose messages do not fit the staging buffer: receivers are taken in
+    // chunks, each chunk's messages are added to the sender rows before the next chunk overwrites them.  Every
+    // sender still receives its messages in ascending edge order, so the result does not depend on the chunking.
+    void agg1_bwd_chunked(int N, int rows, bool zero_dxyz, bool zero_H1_adj)
+    {
+        const int k = K(), nlm = NLM();
+        const size_t row_bytes = (size_t)nlm * k * sizeof(F);
+        const long max_rows = (long)std::max<size_t>(msg_limit_bytes / row_bytes, 1);
+        // receiver boundaries: equal receiver counts, then halved until every chunk's edges fit (read back from the CSR)
+        int nchunks = (int)std::min<long>(N, (E + max_rows - 1) / max_rows + 1);
+        std::vector<int> bnd, fe;
+        for (;;) {
+            bnd.assign((size_t)nchunks + 1, 0); fe.assign((size_t)nchunks + 1, 0);
+            for (int c = 0; c <= nchunks; ++c) {
+                bnd[c] = (int)((long)N * c / nchunks);
+                HIPCHK(hipMemcpyAsync(&fe[c], first_neigh.p + bnd[c], sizeof(int), hipMemcpyDeviceToHost, stream));
+            }
+            HIPCHK(hipStreamSynchronize(stream));
+            long worst = 0;
+            for (int c = 0; c < nchunks; ++c) worst = std::max<long>(worst, (long)fe[c + 1] - fe[c]);
+            if (worst <= max_rows || nchunks >= N) {
+                if (worst > max_rows)
+                    throw Error(SMX_ENOMEM, "one receiver's messages exceed the staging limit (smx_set_staging_limit)");
+                msg.size_to((size_t)worst * nlm * k, stream);
+                break;
+            }
+            nchunks = (int)std::min<long>(N, 2L * nchunks);
+        }
+        const int groups = agg_bwd_groups<F>(hm.L_max, k);
+        if (groups > 1) fpart.size_to((size_t)groups * 3 * E, stream);
+        if (sender_rows != rows) build_sender_lists(rows);
+        stage_begin(ST_AGG1B);
+        for (int c = 0; c < nchunks; ++c) {
+            auto p = agg_params(1, bnd[c + 1]);
+            p.node_begin = bnd[c]; p.msg_edge_begin = fe[c];
+            p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
+            p.fpart = groups > 1 ? fpart.p : nullptr;
+            HIPCHK(launch_agg_bwd<F>(hm.L_max, p, stream));
+            HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p,
+                                           (c == 0 && zero_H1_adj) ? 1 : 0, fe[c], fe[c + 1], stream));
+        }
+        stage_end(ST_AGG1B);
+        stage_begin(ST_FSUM1);
+        if (groups > 1)
+            HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
+        stage_end(ST_FSUM1);
+        stage_begin(ST_SRED);
         stage_end(ST_SRED);
     }
     void st_agg0_bwd(int N)
@@ -1443,6 +1502,13 @@ int smx_set_profiling(smx_model* m, int enabled)
         auto& e = E(m);
         e.profiling = enabled != 0;
         for (int i = 0; i < smx::ST_COUNT; ++i) e.ev_used[i] = false;
+    });
+}
+int smx_set_staging_limit(smx_model* m, long bytes)
+{
+    return guarded([&] {
+        if (bytes <= 0) throw smx::Error(SMX_EINVAL, "the staging limit must be positive");
+        E(m).msg_limit_bytes = (size_t)bytes;
     });
 }
 const char* smx_stage_names(void) { return smx::kStageNames; }

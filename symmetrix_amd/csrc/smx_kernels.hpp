@@ -45,6 +45,10 @@ struct AggParams {
     double* fpart;            // bwd: [channel groups][E][3] partial forces, needed when agg_bwd_groups() > 1
     long num_edges;
     int num_terms;            // entries of B_lm1 / B_c
+    // bwd, general kernel only: receivers [node_begin, num_nodes) are processed and the message of edge e goes to
+    // row e - msg_edge_begin of msg (edge lists too long for one staging buffer are taken in receiver chunks)
+    int node_begin;
+    long msg_edge_begin;
 };
 
 template <typename F> hipError_t launch_agg_fwd(int L_max_H, const AggParams<F>& p, hipStream_t s);
@@ -81,9 +85,10 @@ hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double*
                                hipStream_t s);
 
 // H1_adj[j] (+)= sum over edges with sender j of msg[e], in ascending edge order.
+// H_adj[j] (+)= sum of msg[e - e_lo] over the edges e of sender j with e_lo <= e < e_hi, in ascending edge order
 template <typename F>
-hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg,
-                                F* H_adj, int zero_first, hipStream_t s);
+hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg, F* H_adj,
+                                int zero_first, long e_lo, long e_hi, hipStream_t s);
 
 // ---------------------------------------------------------------------------
 // Neighbour list on the device (smx_kernels_nlist.hip)

@@ -200,7 +200,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
     __syncthreads();
 
     const int K = a.K;
-    const int i = blockIdx.x * 4 + wave;
+    const int i = a.node_begin + blockIdx.x * 4 + wave;
     if (i >= a.num_nodes) return;
     const int k0 = (blockIdx.y * 64 + lane) * CPL;
     const bool active = k0 < K;
@@ -315,7 +315,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                     });
                 });
                 if (a.msg) {
-                    F* mrow = a.msg + (size_t)(eb + le) * NLM * K + k0;
+                    F* mrow = a.msg + (size_t)(eb + le - a.msg_edge_begin) * NLM * K + k0;
 #pragma unroll
                     for (int q = 0; q < NLM; ++q) *reinterpret_cast<Vec<F, CPL>*>(mrow + q * K) = mg[q];
                 }
@@ -341,7 +341,9 @@ hipError_t launch_agg_t(const AggParams<F>& p, hipStream_t s)
     if (p.K % CPL != 0) return hipErrorInvalidValue;
     if (BWD && groups > 1 && !p.fpart) return hipErrorInvalidValue;
     const size_t lds = WL::lists(p.num_terms) + 4 * WL::per_wave(EC);
-    dim3 grid((p.num_nodes + 3) / 4, groups);
+    if (!BWD && (p.node_begin != 0 || p.msg_edge_begin != 0)) return hipErrorInvalidValue;
+    if (p.node_begin < 0 || p.node_begin > p.num_nodes) return hipErrorInvalidValue;
+    dim3 grid((p.num_nodes - p.node_begin + 3) / 4, groups);
     if (grid.x == 0) return hipSuccess;
     void (*kern)(const AggParams<F>, const int);
     if constexpr (BWD) kern = k_agg_bwd<F, LMAXH, CPL, EC>;
@@ -417,13 +419,17 @@ template int agg_bwd_groups<float>(int, int);
 namespace {
 template <typename F>
 __global__ void k_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg,
-                                F* H_adj, int zero_first)
+                                F* H_adj, int zero_first, long e_lo, long e_hi)
 {
     const int j = blockIdx.x;
-    const int s0 = sstart[j], s1 = sstart[j + 1];
+    int s0 = sstart[j], s1 = sstart[j + 1];
+    // the sender's edges are listed in ascending order: narrow to those inside [e_lo, e_hi)
+    while (s0 < s1 && slist[s0] < e_lo) ++s0;
+    while (s1 > s0 && slist[s1 - 1] >= e_hi) --s1;
+    if (s0 == s1 && !zero_first) return;
     for (int q = threadIdx.x; q < width; q += blockDim.x) {
         F acc = zero_first ? F(0) : H_adj[(size_t)j * width + q];
-        for (int t = s0; t < s1; ++t) acc += msg[(size_t)slist[t] * width + q];
+        for (int t = s0; t < s1; ++t) acc += msg[(size_t)(slist[t] - e_lo) * width + q];
         H_adj[(size_t)j * width + q] = acc;
     }
 }
@@ -431,15 +437,16 @@ __global__ void k_sender_reduce(int rows, int width, const int* sstart, const in
 
 template <typename F>
 hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg,
-                                F* H_adj, int zero_first, hipStream_t s)
+                                F* H_adj, int zero_first, long e_lo, long e_hi, hipStream_t s)
 {
     if (rows <= 0) return hipSuccess;
     const int bs = width <= 64 ? 64 : (width <= 128 ? 128 : 256);
-    hipLaunchKernelGGL(k_sender_reduce<F>, dim3(rows), dim3(bs), 0, s, rows, width, sstart, slist, msg, H_adj, zero_first);
+    hipLaunchKernelGGL(k_sender_reduce<F>, dim3(rows), dim3(bs), 0, s, rows, width, sstart, slist, msg, H_adj, zero_first,
+                       e_lo, e_hi);
     return hipGetLastError();
 }
-template hipError_t launch_sender_reduce<double>(int, int, const int*, const int*, const double*, double*, int, hipStream_t);
-template hipError_t launch_sender_reduce<float>(int, int, const int*, const int*, const float*, float*, int, hipStream_t);
+template hipError_t launch_sender_reduce<double>(int, int, const int*, const int*, const double*, double*, int, long, long, hipStream_t);
+template hipError_t launch_sender_reduce<float>(int, int, const int*, const int*, const float*, float*, int, long, long, hipStream_t);
 
 // ---------------------------------------------------------------------------
 namespace {

@@ -113,6 +113,10 @@ class MACE:
     def synchronize(self):
         _lib.check(self._L.smx_synchronize(self._h))
 
+    def set_staging_limit(self, nbytes):
+        """Bound for the buffer of per-edge adjoint messages; longer edge lists are taken in receiver chunks."""
+        _lib.check(self._L.smx_set_staging_limit(self._h, C.c_long(int(nbytes))))
+
     def set_profiling(self, enabled):
         _lib.check(self._L.smx_set_profiling(self._h, int(bool(enabled))))
 

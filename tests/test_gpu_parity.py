@@ -422,3 +422,27 @@ def test_device_resident_loop_positions_to_forces(gpu, tmp_models):
                        oE.data_ptr(), oF.data_ptr(), torch.cuda.current_stream().cuda_stream)
     torch.cuda.synchronize()
     assert np.array_equal(oE.cpu().numpy(), e_ref) and np.array_equal(oF.cpu().numpy(), f_ref)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+def test_receiver_chunks_of_the_layer1_adjoint_change_nothing(gpu, tmp_models, dtype):
+    """A staging limit far below the message volume (many chunks, down to a few receivers each) gives the same bits."""
+    model = H.tiny_model(K=16, L_max=1, n_pts=48, seed=9)
+    path = H.write_model(model, tmp_models / "chunks.json")
+    pos, cell, sp = H.small_system(60, seed=4)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    eng = gpu(path, dtype)
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    e_ref, f_ref, h_ref = eng.node_energies.copy(), eng.node_forces.copy(), np.array(eng.H1_adj)
+    row_bytes = 4 * 16 * (8 if dtype == "float64" else 4)
+    for limit in (len(ea["r"]) * row_bytes // 3, 200 * row_bytes, int(ea["num_neigh"].max()) * row_bytes):
+        eng.set_staging_limit(limit)
+        print(f"staging limit {limit} bytes", flush=True)
+        eng.compute_node_energies_forces(*H.call_args(ea))
+        assert np.array_equal(eng.node_energies, e_ref)
+        assert np.array_equal(eng.node_forces, f_ref)
+        assert np.array_equal(np.array(eng.H1_adj), h_ref)
+    eng.set_staging_limit(row_bytes)          # below one receiver's messages
+    with pytest.raises(RuntimeError):
+        eng.compute_node_energies_forces(*H.call_args(ea))

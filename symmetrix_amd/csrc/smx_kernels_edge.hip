@@ -53,6 +53,13 @@ __device__ __forceinline__ void pin(F& v)
     asm volatile("" : "+v"(v));
 }
 
+// v is final here, and what is addressed through off afterwards is not loaded before
+template <typename F>
+__device__ __forceinline__ void tie(F& v, int& off)
+{
+    asm volatile("" : "+v"(v), "+v"(off));
+}
+
 template <typename F, int CPL>
 __device__ __forceinline__ Vec<F, CPL> ldv(const F* p)
 {
@@ -280,7 +287,16 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                         R[c] = cf.v[0] + x * (cf.v[1] + x * (cf.v[2] + x * cf.v[3]));
                         Rd[c] = cf.v[1] + x * (F(2) * cf.v[2] + F(3) * x * cf.v[3]);
                     }
-                    // rows m of B in groups of MG; a fence after each group bounds the LDS values in flight
+                    // Sum over the rows m first: u[m2][comp] = sum_m d[m] * (B, dB/dx, dB/dy, dB/dz)[m][m2], then one
+                    // product with the sender feature per m2.  Rows are taken in groups of MG; the fence after each
+                    // group bounds the LDS values in flight.
+                    F u[CPL][n2][4];
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c)
+#pragma unroll
+                        for (int m2 = 0; m2 < n2; ++m2)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) u[c][m2][t] = F(0);
                     constexpr int MG = n2 == 1 ? 2 * l + 1 : 3;
                     static_for<0, (2 * l + 1 + MG - 1) / MG>([&](auto gc) {
                         constexpr int m0 = decltype(gc)::value * MG;
@@ -294,25 +310,38 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
 #pragma unroll
                             for (int m = m0; m < m1; ++m) {
                                 const F dd = d[c][lme0 + m * es];
-                                const F t = dd * R[c];
-                                F z = F(0), zx = F(0), zy = F(0), zz = F(0);
 #pragma unroll
                                 for (int m2 = 0; m2 < n2; ++m2) {
-                                    const F h = H[l2 * l2 + m2].v[c];
                                     const Vec<F, 4>& bb = b4[(m - m0) * n2 + m2];
-                                    z += bb.v[0] * h; zx += bb.v[1] * h; zy += bb.v[2] * h; zz += bb.v[3] * h;
-                                    mg[l2 * l2 + m2].v[c] += t * bb.v[0];
+#pragma unroll
+                                    for (int t = 0; t < 4; ++t) u[c][m2][t] += dd * bb.v[t];
                                 }
-                                srad += dd * Rd[c] * z;
-                                gx += t * zx; gy += t * zy; gz += t * zz;
                             }
                         }
-                        order_after(gx, gy, gz, srad, roff, boffs);
 #pragma unroll
-                        for (int m2 = 0; m2 < n2; ++m2)
+                        for (int c = 0; c < CPL; ++c)
 #pragma unroll
-                            for (int c = 0; c < CPL; ++c) pin(mg[l2 * l2 + m2].v[c]);
+                            for (int m2 = 0; m2 < n2; ++m2)
+#pragma unroll
+                                for (int t = 0; t < 4; ++t) tie(u[c][m2][t], boffs);
                     });
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) {
+                        F s0 = F(0), s1 = F(0), s2 = F(0), s3 = F(0);
+#pragma unroll
+                        for (int m2 = 0; m2 < n2; ++m2) {
+                            const F h = H[l2 * l2 + m2].v[c];
+                            s0 += u[c][m2][0] * h; s1 += u[c][m2][1] * h; s2 += u[c][m2][2] * h; s3 += u[c][m2][3] * h;
+                            mg[l2 * l2 + m2].v[c] += R[c] * u[c][m2][0];
+                        }
+                        srad += Rd[c] * s0;
+                        gx += R[c] * s1; gy += R[c] * s2; gz += R[c] * s3;
+                    }
+                    order_after(gx, gy, gz, srad, roff, boffs);
+#pragma unroll
+                    for (int m2 = 0; m2 < n2; ++m2)
+#pragma unroll
+                        for (int c = 0; c < CPL; ++c) pin(mg[l2 * l2 + m2].v[c]);
                 });
                 if (a.msg) {
                     F* mrow = a.msg + (size_t)(eb + le - a.msg_edge_begin) * NLM * K + k0;

@@ -39,11 +39,11 @@ struct WaveLds {
     }
 };
 
-// Everything computed from roff or boffs after this point is scheduled after the four sums are final.
+// Everything addressed through boffs after this point is scheduled after the four sums are final.
 template <typename F>
-__device__ __forceinline__ void order_after(F& gx, F& gy, F& gz, F& srad, size_t& roff, int& boffs)
+__device__ __forceinline__ void order_after(F& gx, F& gy, F& gz, F& srad, int& boffs)
 {
-    asm volatile("" : "+v"(gx), "+v"(gy), "+v"(gz), "+v"(srad), "+v"(roff), "+v"(boffs));
+    asm volatile("" : "+v"(gx), "+v"(gy), "+v"(gz), "+v"(srad), "+v"(boffs));
 }
 
 // The value is final here: keeps an accumulation from drifting past the fences (its operands would stay live).
@@ -256,16 +256,28 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
             *reinterpret_cast<Vec<F, 4>*>(Bs + ((size_t)le * NBP + b) * 4) = o;
         }
         wave_lds_sync();
+        // Spline coefficients of one edge: P x CPL 16-byte loads from the channel-major table.  In single
+        // precision the next edge's coefficients are requested while the current edge is worked on (40
+        // registers in flight); in double precision they are requested together at the start of the edge.
+        constexpr bool AHEAD = sizeof(F) == 4;
+        Vec<F, 4> cf[P][CPL];
+        auto load_cf = [&](int le_) {
+            const int row = __builtin_amdgcn_readfirstlane(rows[le_]);
+            const F* rowp = a.tabK + ((size_t)row * K + k0) * (4 * P);
+#pragma unroll
+            for (int q = 0; q < P; ++q)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) cf[q][c] = ldv<F, 4>(rowp + (c * P + q) * 4);
+        };
+        if (AHEAD && active && nE > 0) load_cf(0);
         for (int le = 0; le < nE; ++le) {
             F srad = F(0), gx = F(0), gy = F(0), gz = F(0);
             if (active) {
                 const F x = (F)xs[le];
-                const int row = __builtin_amdgcn_readfirstlane(rows[le]);
                 const int grow = __builtin_amdgcn_readfirstlane(grows[le]);
-                // element offsets of this edge's table row and of its B block; they pass through the
-                // fence at the end of every path, which keeps the loads of a path behind the arithmetic
-                // of the path before it (all loads at once would need several hundred registers)
-                size_t roff = ((size_t)row * K + k0) * (4 * P);
+                // element offset of this edge's B block; it passes through the fences below, which keep the
+                // LDS reads of a group behind the arithmetic of the group before it (all reads at once would
+                // need several hundred registers)
                 int boffs = le * 4 * NBP;
                 const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
                 Vec<F, CPL> H[NLM], mg[NLM];
@@ -275,18 +287,24 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
 #pragma unroll
                     for (int c = 0; c < CPL; ++c) mg[q].v[c] = F(0);
                 }
+                if (!AHEAD) load_cf(le);
+                F Rv[P][CPL], Rdv[P][CPL];
+#pragma unroll
+                for (int q = 0; q < P; ++q)
+#pragma unroll
+                    for (int c = 0; c < CPL; ++c) {
+                        const Vec<F, 4> k4 = cf[q][c];
+                        Rv[q][c] = k4.v[0] + x * (k4.v[1] + x * (k4.v[2] + x * k4.v[3]));
+                        Rdv[q][c] = k4.v[1] + x * (F(2) * k4.v[2] + F(3) * x * k4.v[3]);
+                    }
+                if (AHEAD && le + 1 < nE) load_cf(le + 1);
                 static_for<0, P>([&](auto pc) {
                     constexpr int p = decltype(pc)::value;
                     constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
-                    constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1, nb = (2 * l + 1) * n2;
-                    const F* rowp = a.tabK + roff;
+                    constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1;
                     F R[CPL], Rd[CPL];
 #pragma unroll
-                    for (int c = 0; c < CPL; ++c) {
-                        const Vec<F, 4> cf = ldv<F, 4>(rowp + (c * P + p) * 4);
-                        R[c] = cf.v[0] + x * (cf.v[1] + x * (cf.v[2] + x * cf.v[3]));
-                        Rd[c] = cf.v[1] + x * (F(2) * cf.v[2] + F(3) * x * cf.v[3]);
-                    }
+                    for (int c = 0; c < CPL; ++c) { R[c] = Rv[p][c]; Rd[c] = Rdv[p][c]; }
                     // Sum over the rows m first: u[m2][comp] = sum_m d[m] * (B, dB/dx, dB/dy, dB/dz)[m][m2], then one
                     // product with the sender feature per m2.  Rows are taken in groups of MG; the fence after each
                     // group bounds the LDS values in flight.
@@ -337,7 +355,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                         srad += Rd[c] * s0;
                         gx += R[c] * s1; gy += R[c] * s2; gz += R[c] * s3;
                     }
-                    order_after(gx, gy, gz, srad, roff, boffs);
+                    order_after(gx, gy, gz, srad, boffs);
 #pragma unroll
                     for (int m2 = 0; m2 < n2; ++m2)
 #pragma unroll

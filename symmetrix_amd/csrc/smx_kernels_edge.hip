@@ -39,6 +39,51 @@ struct WaveLds {
     }
 };
 
+// The steps in which the adjoint kernel walks the coupling block B[path][m][m2] of an edge: all rows m of a path
+// with a scalar sender feature, three rows at a time of a path with a vector one (at most nine entries).
+template <int LMAXH>
+struct BwdSteps {
+    using PT = Paths<LMAXH>;
+    static constexpr int rows(int p) { return 2 * PT::l(p) + 1; }
+    static constexpr int group(int p) { return PT::l2(p) == 0 ? rows(p) : 3; }
+    static constexpr int groups(int p) { return (rows(p) + group(p) - 1) / group(p); }
+    static constexpr int count()
+    {
+        int n = 0;
+        for (int p = 0; p < PT::P; ++p) n += groups(p);
+        return n;
+    }
+    static constexpr int path(int s)
+    {
+        for (int p = 0; p < PT::P; ++p) {
+            if (s < groups(p)) return p;
+            s -= groups(p);
+        }
+        return -1;
+    }
+    static constexpr int m0(int s)
+    {
+        for (int p = 0; p < PT::P; ++p) {
+            if (s < groups(p)) return s * group(p);
+            s -= groups(p);
+        }
+        return -1;
+    }
+    static constexpr int m1(int s)
+    {
+        const int p = path(s), e = m0(s) + group(p);
+        return e < rows(p) ? e : rows(p);
+    }
+    static constexpr int len(int s) { return (m1(s) - m0(s)) * (2 * PT::l2(path(s)) + 1); }
+    static constexpr int max_len()
+    {
+        int n = 0;
+        for (int s = 0; s < count(); ++s) n = len(s) > n ? len(s) : n;
+        return n;
+    }
+    static constexpr int MAXLEN = max_len();
+};
+
 // Everything addressed through boffs after this point is scheduled after the four sums are final.
 template <typename F>
 __device__ __forceinline__ void order_after(F& gx, F& gy, F& gz, F& srad, int& boffs)
@@ -298,68 +343,76 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                         Rdv[q][c] = k4.v[1] + x * (F(2) * k4.v[2] + F(3) * x * k4.v[3]);
                     }
                 if (AHEAD && le + 1 < nE) load_cf(le + 1);
-                static_for<0, P>([&](auto pc) {
-                    constexpr int p = decltype(pc)::value;
-                    constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
+                // The B block of the edge is walked in steps (a few rows m of one path each).  Per path, the rows
+                // are summed first, u[m2][comp] = sum_m d[m] * (B, dB/dx, dB/dy, dB/dz)[m][m2], then one product
+                // with the sender feature per m2.  In single precision the LDS reads of the next step are issued
+                // before the arithmetic of the current one (two register buffers); the fence after each step keeps
+                // reads further ahead from being issued (all at once would need several hundred registers).
+                using ST = BwdSteps<LMAXH>;
+                constexpr bool LOOKAHEAD = sizeof(F) == 4;
+                Vec<F, 4> buf[LOOKAHEAD ? 2 : 1][ST::MAXLEN];
+                F u[CPL][2 * LMAXH + 1][4];
+                auto load_step = [&](auto sc, Vec<F, 4>* dst) {
+                    constexpr int s = decltype(sc)::value, p = ST::path(s), n2 = 2 * PT::l2(p) + 1;
+                    const F* B4 = Bs + boffs + (PT::boff(p) + ST::m0(s) * n2) * 4;
+#pragma unroll
+                    for (int q = 0; q < ST::len(s); ++q) dst[q] = ldv<F, 4>(B4 + 4 * q);
+                };
+                if constexpr (LOOKAHEAD) load_step(std::integral_constant<int, 0>{}, buf[0]);
+                static_for<0, ST::count()>([&](auto sc) {
+                    constexpr int s = decltype(sc)::value, p = ST::path(s), m0 = ST::m0(s), m1 = ST::m1(s);
+                    constexpr int l = PT::l(p), l2 = PT::l2(p);
                     constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1;
-                    F R[CPL], Rd[CPL];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c) { R[c] = Rv[p][c]; Rd[c] = Rdv[p][c]; }
-                    // Sum over the rows m first: u[m2][comp] = sum_m d[m] * (B, dB/dx, dB/dy, dB/dz)[m][m2], then one
-                    // product with the sender feature per m2.  Rows are taken in groups of MG; the fence after each
-                    // group bounds the LDS values in flight.
-                    F u[CPL][n2][4];
-#pragma unroll
-                    for (int c = 0; c < CPL; ++c)
-#pragma unroll
-                        for (int m2 = 0; m2 < n2; ++m2)
-#pragma unroll
-                            for (int t = 0; t < 4; ++t) u[c][m2][t] = F(0);
-                    constexpr int MG = n2 == 1 ? 2 * l + 1 : 3;
-                    static_for<0, (2 * l + 1 + MG - 1) / MG>([&](auto gc) {
-                        constexpr int m0 = decltype(gc)::value * MG;
-                        constexpr int m1 = m0 + MG < 2 * l + 1 ? m0 + MG : 2 * l + 1;
-                        const F* B4 = Bs + boffs + (bo + m0 * n2) * 4;
-                        Vec<F, 4> b4[(m1 - m0) * n2];
-#pragma unroll
-                        for (int q = 0; q < (m1 - m0) * n2; ++q) b4[q] = ldv<F, 4>(B4 + 4 * q);
-#pragma unroll
-                        for (int c = 0; c < CPL; ++c) {
-#pragma unroll
-                            for (int m = m0; m < m1; ++m) {
-                                const F dd = d[c][lme0 + m * es];
-#pragma unroll
-                                for (int m2 = 0; m2 < n2; ++m2) {
-                                    const Vec<F, 4>& bb = b4[(m - m0) * n2 + m2];
-#pragma unroll
-                                    for (int t = 0; t < 4; ++t) u[c][m2][t] += dd * bb.v[t];
-                                }
-                            }
-                        }
+                    Vec<F, 4>* b4 = buf[LOOKAHEAD ? (s & 1) : 0];
+                    if constexpr (!LOOKAHEAD) load_step(sc, b4);
+                    else if constexpr (s + 1 < ST::count()) load_step(std::integral_constant<int, s + 1>{}, buf[(s + 1) & 1]);
+                    if constexpr (m0 == 0) {
 #pragma unroll
                         for (int c = 0; c < CPL; ++c)
 #pragma unroll
                             for (int m2 = 0; m2 < n2; ++m2)
 #pragma unroll
-                                for (int t = 0; t < 4; ++t) tie(u[c][m2][t], boffs);
-                    });
+                                for (int t = 0; t < 4; ++t) u[c][m2][t] = F(0);
+                    }
 #pragma unroll
                     for (int c = 0; c < CPL; ++c) {
-                        F s0 = F(0), s1 = F(0), s2 = F(0), s3 = F(0);
 #pragma unroll
-                        for (int m2 = 0; m2 < n2; ++m2) {
-                            const F h = H[l2 * l2 + m2].v[c];
-                            s0 += u[c][m2][0] * h; s1 += u[c][m2][1] * h; s2 += u[c][m2][2] * h; s3 += u[c][m2][3] * h;
-                            mg[l2 * l2 + m2].v[c] += R[c] * u[c][m2][0];
+                        for (int m = m0; m < m1; ++m) {
+                            const F dd = d[c][lme0 + m * es];
+#pragma unroll
+                            for (int m2 = 0; m2 < n2; ++m2) {
+                                const Vec<F, 4>& bb = b4[(m - m0) * n2 + m2];
+#pragma unroll
+                                for (int t = 0; t < 4; ++t) u[c][m2][t] += dd * bb.v[t];
+                            }
                         }
-                        srad += Rd[c] * s0;
-                        gx += R[c] * s1; gy += R[c] * s2; gz += R[c] * s3;
                     }
-                    order_after(gx, gy, gz, srad, boffs);
 #pragma unroll
-                    for (int m2 = 0; m2 < n2; ++m2)
+                    for (int c = 0; c < CPL; ++c)
 #pragma unroll
-                        for (int c = 0; c < CPL; ++c) pin(mg[l2 * l2 + m2].v[c]);
+                        for (int m2 = 0; m2 < n2; ++m2)
+#pragma unroll
+                            for (int t = 0; t < 4; ++t) tie(u[c][m2][t], boffs);
+                    if constexpr (m1 == 2 * l + 1) {
+#pragma unroll
+                        for (int c = 0; c < CPL; ++c) {
+                            const F R = Rv[p][c], Rd = Rdv[p][c];
+                            F s0 = F(0), s1 = F(0), s2 = F(0), s3 = F(0);
+#pragma unroll
+                            for (int m2 = 0; m2 < n2; ++m2) {
+                                const F h = H[l2 * l2 + m2].v[c];
+                                s0 += u[c][m2][0] * h; s1 += u[c][m2][1] * h; s2 += u[c][m2][2] * h; s3 += u[c][m2][3] * h;
+                                mg[l2 * l2 + m2].v[c] += R * u[c][m2][0];
+                            }
+                            srad += Rd * s0;
+                            gx += R * s1; gy += R * s2; gz += R * s3;
+                        }
+                        order_after(gx, gy, gz, srad, boffs);
+#pragma unroll
+                        for (int m2 = 0; m2 < n2; ++m2)
+#pragma unroll
+                            for (int c = 0; c < CPL; ++c) pin(mg[l2 * l2 + m2].v[c]);
+                    }
                 });
                 if (a.msg) {
                     F* mrow = a.msg + (size_t)(eb + le - a.msg_edge_begin) * NLM * K + k0;

@@ -366,14 +366,6 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                     Vec<F, 4>* b4 = buf[LOOKAHEAD ? (s & 1) : 0];
                     if constexpr (!LOOKAHEAD) load_step(sc, b4);
                     else if constexpr (s + 1 < ST::count()) load_step(std::integral_constant<int, s + 1>{}, buf[(s + 1) & 1]);
-                    if constexpr (m0 == 0) {
-#pragma unroll
-                        for (int c = 0; c < CPL; ++c)
-#pragma unroll
-                            for (int m2 = 0; m2 < n2; ++m2)
-#pragma unroll
-                                for (int t = 0; t < 4; ++t) u[c][m2][t] = F(0);
-                    }
 #pragma unroll
                     for (int c = 0; c < CPL; ++c) {
 #pragma unroll
@@ -383,7 +375,8 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                             for (int m2 = 0; m2 < n2; ++m2) {
                                 const Vec<F, 4>& bb = b4[(m - m0) * n2 + m2];
 #pragma unroll
-                                for (int t = 0; t < 4; ++t) u[c][m2][t] += dd * bb.v[t];
+                                for (int t = 0; t < 4; ++t)   // the first row of a path starts the sums
+                                    u[c][m2][t] = m == 0 ? dd * bb.v[t] : u[c][m2][t] + dd * bb.v[t];
                             }
                         }
                     }

@@ -510,7 +510,9 @@ template int agg_bwd_groups<float>(int, int);
 
 // ---------------------------------------------------------------------------
 namespace {
-template <typename F>
+// V consecutive elements per thread (16-byte accesses when the row width allows); four messages are requested
+// before the first is added, the additions keep the ascending edge order
+template <typename F, int V>
 __global__ void k_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg,
                                 F* H_adj, int zero_first, long e_lo, long e_hi)
 {
@@ -520,10 +522,30 @@ __global__ void k_sender_reduce(int rows, int width, const int* sstart, const in
     while (s0 < s1 && slist[s0] < e_lo) ++s0;
     while (s1 > s0 && slist[s1 - 1] >= e_hi) --s1;
     if (s0 == s1 && !zero_first) return;
-    for (int q = threadIdx.x; q < width; q += blockDim.x) {
-        F acc = zero_first ? F(0) : H_adj[(size_t)j * width + q];
-        for (int t = s0; t < s1; ++t) acc += msg[(size_t)(slist[t] - e_lo) * width + q];
-        H_adj[(size_t)j * width + q] = acc;
+    for (int q = threadIdx.x * V; q < width; q += blockDim.x * V) {
+        Vec<F, V> acc;
+        if (zero_first) {
+#pragma unroll
+            for (int c = 0; c < V; ++c) acc.v[c] = F(0);
+        } else {
+            acc = ldv<F, V>(H_adj + (size_t)j * width + q);
+        }
+        int t = s0;
+        for (; t + 4 <= s1; t += 4) {
+            Vec<F, V> m[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) m[i] = ldv<F, V>(msg + (size_t)(slist[t + i] - e_lo) * width + q);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int c = 0; c < V; ++c) acc.v[c] += m[i].v[c];
+        }
+        for (; t < s1; ++t) {
+            const Vec<F, V> m = ldv<F, V>(msg + (size_t)(slist[t] - e_lo) * width + q);
+#pragma unroll
+            for (int c = 0; c < V; ++c) acc.v[c] += m.v[c];
+        }
+        *reinterpret_cast<Vec<F, V>*>(H_adj + (size_t)j * width + q) = acc;
     }
 }
 }  // namespace
@@ -533,9 +555,17 @@ hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const in
                                 F* H_adj, int zero_first, long e_lo, long e_hi, hipStream_t s)
 {
     if (rows <= 0) return hipSuccess;
-    const int bs = width <= 64 ? 64 : (width <= 128 ? 128 : 256);
-    hipLaunchKernelGGL(k_sender_reduce<F>, dim3(rows), dim3(bs), 0, s, rows, width, sstart, slist, msg, H_adj, zero_first,
-                       e_lo, e_hi);
+    constexpr int V = 16 / (int)sizeof(F);
+    if (width % V == 0) {
+        const int lanes = width / V;
+        const int bs = lanes <= 64 ? 64 : (lanes <= 128 ? 128 : 256);
+        hipLaunchKernelGGL((k_sender_reduce<F, V>), dim3(rows), dim3(bs), 0, s, rows, width, sstart, slist, msg, H_adj,
+                           zero_first, e_lo, e_hi);
+    } else {
+        const int bs = width <= 64 ? 64 : (width <= 128 ? 128 : 256);
+        hipLaunchKernelGGL((k_sender_reduce<F, 1>), dim3(rows), dim3(bs), 0, s, rows, width, sstart, slist, msg, H_adj,
+                           zero_first, e_lo, e_hi);
+    }
     return hipGetLastError();
 }
 template hipError_t launch_sender_reduce<double>(int, int, const int*, const int*, const double*, double*, int, long, long, hipStream_t);

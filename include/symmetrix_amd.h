@@ -88,6 +88,23 @@ int smx_compute_device(smx_model* m, int num_nodes,
                        const double* d_xyz, const double* d_r, long num_edges,
                        double* d_node_energies, double* d_node_forces, void* stream);
 
+/* The same computation for a caller that holds ghost atoms as extra nodes, the mode no_mpi_message_passing of the
+ * pair style (pair_symmetrix_mace.cpp:557-748): the first num_local_nodes nodes are evaluated in full, the
+ * num_ghost_nodes nodes after them go through layer 0 only (R0, A0, M0, H1 and their adjoints, :674-698), so that
+ * neigh_indices of local receivers may point at ghost nodes.  Arrays are laid out as for
+ * smx_compute_node_energies_forces over all num_local_nodes + num_ghost_nodes nodes, local nodes and their edges
+ * first; neigh_indices of edges that belong to ghost receivers are not read.  Results: node_energies[num_local_nodes],
+ * node_forces[3*num_edges] (ghost receivers' edges carry their layer-0 share).  The device variant needs the number of
+ * edges of the local receivers as well, writes d_node_energies[num_local_nodes] and d_node_forces[3*num_edges] when
+ * they are not NULL, and does not synchronise. */
+int smx_compute_ghosted(smx_model* m, int num_local_nodes, int num_ghost_nodes, const int* node_types,
+                        const int* num_neigh, const int* neigh_indices, const int* neigh_types, const double* xyz,
+                        const double* r, long num_edges);
+int smx_compute_ghosted_device(smx_model* m, int num_local_nodes, int num_ghost_nodes, const int* d_node_types,
+                               const int* d_num_neigh, const int* d_neigh_indices, const int* d_neigh_types,
+                               const double* d_xyz, const double* d_r, long num_edges, long num_local_edges,
+                               double* d_node_energies, double* d_node_forces, void* stream);
+
 /* Number of rows of H1 a following layer-1 call may index (ghost rows of the
  * LAMMPS modes, pair_symmetrix_mace.cpp:462-471, 674-698).  Defaults to the
  * num_nodes of the last compute_H1. */

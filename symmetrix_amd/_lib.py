@@ -22,7 +22,7 @@ ERROR_NAMES = {-1: "SMX_EINVAL", -2: "SMX_EFILE", -3: "SMX_EUNSUPPORTED", -4: "S
 EXPORTS = [
     "smx_last_error", "smx_model_load", "smx_model_free", "smx_model_get_int", "smx_model_get_double",
     "smx_model_get_atomic_numbers", "smx_model_get_atomic_energies", "smx_compute_node_energies_forces",
-    "smx_compute_device", "smx_set_num_H1_rows", "smx_compute_Y", "smx_compute_R0", "smx_compute_R1",
+    "smx_compute_device", "smx_compute_ghosted", "smx_compute_ghosted_device", "smx_set_num_H1_rows", "smx_compute_Y", "smx_compute_R0", "smx_compute_R1",
     "smx_compute_A0", "smx_reverse_A0", "smx_compute_A0_scaled", "smx_reverse_A0_scaled", "smx_compute_A1_scaled",
     "smx_reverse_A1_scaled", "smx_compute_M0", "smx_reverse_M0", "smx_compute_H1", "smx_reverse_H1",
     "smx_compute_Phi1", "smx_reverse_Phi1", "smx_compute_A1", "smx_reverse_A1", "smx_compute_M1",

@@ -123,7 +123,7 @@ struct EngineBase {
 
     virtual void compute(int N, const int* node_types, const int* num_neigh, const int* neigh_indices,
                          const int* neigh_types, const double* xyz, const double* r, long E, bool on_device,
-                         double* d_energies, double* d_forces) = 0;
+                         double* d_energies, double* d_forces, int N_local, long E_local) = 0;
     virtual void stage(const char* name, int N, const int* node_types, const int* num_neigh,
                        const int* neigh_indices, const int* neigh_types, const double* xyz, const double* r,
                        long E, int flag_a, int flag_b) = 0;
@@ -179,6 +179,7 @@ struct Engine : EngineBase {
     const int *node_types = nullptr, *num_neigh = nullptr, *neigh_indices = nullptr, *neigh_types = nullptr;
     const double *xyz = nullptr, *r = nullptr;
     long E = 0;
+    long E1 = 0;   // leading edges whose receivers take part in layer 1 (all of them unless ghost nodes follow)
     int N_geo = 0;
     DVec<int> first_neigh, recv_order, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
     int sender_rows = 0;
@@ -407,7 +408,7 @@ struct Engine : EngineBase {
             if (x) { g_xyz.upload(x, 3 * E_, s); xyz = g_xyz.p; }
             if (rr) { g_r.upload(rr, E_, s); r = g_r.p; }
         }
-        if (E_ >= 0) E = E_;
+        if (E_ >= 0) { E = E_; E1 = E_; }
     }
     void build_first_neigh(int N)
     {
@@ -431,9 +432,9 @@ struct Engine : EngineBase {
     {
         hipStream_t s = stream;
         s_count.size_to((size_t)2 * rows, s); s_start.size_to((size_t)rows + 1, s);
-        s_list.size_to((size_t)E, s);
+        s_list.size_to((size_t)E1, s);
         scan_tmp.size_to((size_t)rows / 1024 + 2, s);
-        HIPCHK(launch_sender_lists(neigh_indices, (int)E, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p,
+        HIPCHK(launch_sender_lists(neigh_indices, (int)E1, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p,
                                    counters_zeroed ? 1 : 0, s));
         counters_zeroed = false;
         sender_rows = rows;
@@ -446,7 +447,7 @@ struct Engine : EngineBase {
         HIPCHK(hipMemsetAsync(flags.p, 0, sizeof(int), s));
         HIPCHK(launch_check_range(node_types, N, hm.T, flags.p, s));
         HIPCHK(launch_check_range(neigh_types, E, hm.T, flags.p, s));
-        HIPCHK(launch_check_range(neigh_indices, E, rows, flags.p, s));
+        HIPCHK(launch_check_range(neigh_indices, E1, rows, flags.p, s));
         HIPCHK(launch_check_r(r, E, hm.r_cut, flags.p, s));
         int f = 0;
         HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, s));
@@ -726,11 +727,11 @@ struct Engine : EngineBase {
         H1_adj.resize(H1.n, stream);
         const int rows = (int)(H1.n / ((size_t)nlm * k));
         const size_t row_bytes = (size_t)nlm * k * sizeof(F);
-        if (!slice_CH1 && (size_t)E * row_bytes > msg_limit_bytes) {
+        if (!slice_CH1 && (size_t)E1 * row_bytes > msg_limit_bytes) {
             agg1_bwd_chunked(N, rows, zero_dxyz, zero_H1_adj);
             return;
         }
-        msg.size_to((size_t)E * nlm * k, stream);
+        msg.size_to((size_t)E1 * nlm * k, stream);
         stage_begin(ST_AGG1B);
         if (slice_CH1) {
             auto sp = slice_params(1, N);
@@ -740,16 +741,16 @@ struct Engine : EngineBase {
             HIPCHK(launch_slice_bwd<F>(sp, stream));
             stage_end(ST_AGG1B);
             stage_begin(ST_FSUM1);
-            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
+            HIPCHK(launch_fpart_reduce(E1, E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
             stage_end(ST_FSUM1);
         } else {
             auto p = agg_params(1, N);
             p.d_out = dPhi1.p; p.forces = node_forces.p; p.accumulate_forces = zero_dxyz ? 0 : 1; p.msg = msg.p;
-            agg_bwd_general(hm.L_max, p, ST_AGG1B, ST_FSUM1);
+            agg_bwd_general(hm.L_max, p, E1, ST_AGG1B, ST_FSUM1);
         }
         stage_begin(ST_SRED);
         if (sender_rows != rows) build_sender_lists(rows);
-        HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, 0, E, stream));
+        HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, 0, E1, stream));
         stage_end(ST_SRED);
     }
     // The same stage for edge lists whose messages do not fit the staging buffer: receivers are taken in
@@ -761,7 +762,7 @@ struct Engine : EngineBase {
         const size_t row_bytes = (size_t)nlm * k * sizeof(F);
         const long max_rows = (long)std::max<size_t>(msg_limit_bytes / row_bytes, 1);
         // receiver boundaries: equal receiver counts, then halved until every chunk's edges fit (read back from the CSR)
-        int nchunks = (int)std::min<long>(N, (E + max_rows - 1) / max_rows + 1);
+        int nchunks = (int)std::min<long>(N, (E1 + max_rows - 1) / max_rows + 1);
         std::vector<int> bnd, fe;
         for (;;) {
             bnd.assign((size_t)nchunks + 1, 0); fe.assign((size_t)nchunks + 1, 0);
@@ -796,7 +797,7 @@ struct Engine : EngineBase {
         stage_end(ST_AGG1B);
         stage_begin(ST_FSUM1);
         if (groups > 1)
-            HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
+            HIPCHK(launch_fpart_reduce(E1, E, groups, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
         stage_end(ST_FSUM1);
         stage_begin(ST_SRED);
         stage_end(ST_SRED);
@@ -814,17 +815,17 @@ struct Engine : EngineBase {
             HIPCHK(launch_slice_bwd<F>(sp, stream));
             stage_end(ST_AGG0B);
             stage_begin(ST_FSUM0);
-            HIPCHK(launch_fpart_reduce(E, S, fpart.p, node_forces.p, 1, forces_copy, stream));
+            HIPCHK(launch_fpart_reduce(E, E, S, fpart.p, node_forces.p, 1, forces_copy, stream));
             forces_copy = nullptr;
             stage_end(ST_FSUM0);
             return;
         }
         auto p = agg_params(0, N);
         p.d_out = Phi0.p; p.forces = node_forces.p; p.accumulate_forces = 1; p.msg = nullptr;
-        agg_bwd_general(0, p, ST_AGG0B, ST_FSUM0);
+        agg_bwd_general(0, p, E, ST_AGG0B, ST_FSUM0);
     }
     // general adjoint kernel; wide models are cut into channel groups whose partial forces are added in order
-    void agg_bwd_general(int L_max_H, AggParams<F>& p, int st_kernel, int st_sum)
+    void agg_bwd_general(int L_max_H, AggParams<F>& p, long edges, int st_kernel, int st_sum)
     {
         const int groups = agg_bwd_groups<F>(L_max_H, K());
         if (groups > 1) {
@@ -836,16 +837,26 @@ struct Engine : EngineBase {
         stage_end(st_kernel);
         if (groups > 1) {
             stage_begin(st_sum);
-            HIPCHK(launch_fpart_reduce(E, groups, fpart.p, node_forces.p, p.accumulate_forces, nullptr, stream));
+            HIPCHK(launch_fpart_reduce(edges, E, groups, fpart.p, node_forces.p, p.accumulate_forces, nullptr, stream));
             stage_end(st_sum);
         }
     }
 
     // ------------------------------------------------------------------
     void compute(int N, const int* nt, const int* nn, const int* ni, const int* nty, const double* x,
-                 const double* rr, long E_, bool on_device, double* d_energies, double* d_forces) override
+                 const double* rr, long E_, bool on_device, double* d_energies, double* d_forces, int N_local,
+                 long E_local) override
     {
         if (N < 0 || E_ < 0) throw Error(SMX_EINVAL, "negative num_nodes or num_edges");
+        // ghost nodes (the last N - N1 nodes and their edges) go through layer 0 only: their H1 rows feed the
+        // local receivers, their adjoint comes back through H1_adj (pair_symmetrix_mace.cpp:662-698)
+        const int N1 = N_local < 0 ? N : N_local;
+        if (N1 > N || E_local > E_) throw Error(SMX_EINVAL, "more local nodes or edges than nodes or edges");
+        if (N1 < N && E_local < 0) {
+            if (on_device) throw Error(SMX_EINVAL, "the number of local edges is needed with ghost nodes");
+            E_local = 0;
+            for (int i = 0; i < N1; ++i) E_local += nn[i];
+        }
         if (!on_device) edges_from_counts_check(N, nn, E_);
         if (N == 0) {
             if (E_ != 0) throw Error(SMX_EINVAL, "edges without nodes");
@@ -855,6 +866,7 @@ struct Engine : EngineBase {
         }
         stage_begin(ST_PREP);
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, on_device);
+        if (N1 < N) E1 = E_local;
         // range checks come before any kernel that uses these integers as indices
         if (on_device && N <= 65536) {
             // one launch for first_neigh, degree order, species groups and the cleared sender counters
@@ -876,42 +888,49 @@ struct Engine : EngineBase {
         build_sender_lists(N);
         stage_end(ST_PREP);
 
-        node_energies.size_to((size_t)N, stream);
+        node_energies.size_to((size_t)N1, stream);
         node_forces.size_to((size_t)3 * E, stream);
         if (N == 0) return;
 
         energies_copy = d_energies; forces_copy = d_forces;
         // Terms that add to the forces before the layer-1 adjoint writes them (mace.cpp:27-35, 56): with any of
         // them the force array starts at zero and every later stage accumulates.
-        const bool early_forces = hm.has_zbl || hm.A1_scaled;
+        const bool early_forces = hm.has_zbl || hm.A1_scaled || N1 < N;
         if (early_forces) HIPCHK(launch_fill<double>(node_forces.p, 3 * E, 0.0, stream));
         if (hm.has_zbl) {
-            HIPCHK(launch_fill<double>(node_energies.p, (long)N, 0.0, stream));
-            st_zbl(N);
+            HIPCHK(launch_fill<double>(node_energies.p, (long)N1, 0.0, stream));
+            st_zbl(N1);
         }
         stage_begin(ST_AGG0F); st_agg0_fwd(N); stage_end(ST_AGG0F);
         stage_begin(ST_A0LIN); st_A0_lin(N, false); stage_end(ST_A0LIN);
         st_scale(0, N, false);
         stage_begin(ST_M0); st_poly(N, false); stage_end(ST_M0);
         stage_begin(ST_H1); st_H1(N, false); stage_end(ST_H1);
-        stage_begin(ST_AGG1F); st_agg1_fwd(N); stage_end(ST_AGG1F);
-        stage_begin(ST_A1); st_A1(N, false); stage_end(ST_A1);
-        st_scale(1, N, false);
-        stage_begin(ST_M1); st_poly(N, true); stage_end(ST_M1);
-        stage_begin(ST_H2); st_H2(N); stage_end(ST_H2);
-        stage_begin(ST_READOUT); st_readouts(N, !hm.has_zbl); stage_end(ST_READOUT);
-        stage_begin(ST_REVH2); st_reverse_H2(N, false); stage_end(ST_REVH2);
-        stage_begin(ST_REVM1); st_reverse_M1(N); stage_end(ST_REVM1);
-        st_scale(1, N, true);
-        stage_begin(ST_REVA1); st_A1(N, true); stage_end(ST_REVA1);
-        st_agg1_bwd(N, !early_forces, false);
+        // per-species node groups and the degree order of the receivers cover the nodes of the current stages
+        auto node_lists_for = [&](int n) {
+            build_type_groups(n);
+            HIPCHK(launch_degree_order(n, first_neigh.p, recv_order.p, stream));
+        };
+        if (N1 < N) node_lists_for(N1);
+        stage_begin(ST_AGG1F); st_agg1_fwd(N1); stage_end(ST_AGG1F);
+        stage_begin(ST_A1); st_A1(N1, false); stage_end(ST_A1);
+        st_scale(1, N1, false);
+        stage_begin(ST_M1); st_poly(N1, true); stage_end(ST_M1);
+        stage_begin(ST_H2); st_H2(N1); stage_end(ST_H2);
+        stage_begin(ST_READOUT); st_readouts(N1, !hm.has_zbl); stage_end(ST_READOUT);
+        stage_begin(ST_REVH2); st_reverse_H2(N1, false); stage_end(ST_REVH2);
+        stage_begin(ST_REVM1); st_reverse_M1(N1); stage_end(ST_REVM1);
+        st_scale(1, N1, true);
+        stage_begin(ST_REVA1); st_A1(N1, true); stage_end(ST_REVA1);
+        st_agg1_bwd(N1, !early_forces, false);
+        if (N1 < N) node_lists_for(N);
         stage_begin(ST_REVH1); st_H1(N, true); stage_end(ST_REVH1);
         stage_begin(ST_REVM0); st_reverse_M0(N); stage_end(ST_REVM0);
         st_scale(0, N, true);
         stage_begin(ST_REVA0LIN); st_A0_lin(N, true); stage_end(ST_REVA0LIN);
         st_agg0_bwd(N);
 
-        if (energies_copy) HIPCHK(hipMemcpyAsync(energies_copy, node_energies.p, (size_t)N * sizeof(double), hipMemcpyDeviceToDevice, stream));
+        if (energies_copy) HIPCHK(hipMemcpyAsync(energies_copy, node_energies.p, (size_t)N1 * sizeof(double), hipMemcpyDeviceToDevice, stream));
         if (forces_copy && E) HIPCHK(hipMemcpyAsync(forces_copy, node_forces.p, (size_t)3 * E * sizeof(double), hipMemcpyDeviceToDevice, stream));
         energies_copy = nullptr; forces_copy = nullptr;
         // the reference throws from CubicSpline::evaluate for an edge beyond the normalisation spline
@@ -1353,7 +1372,7 @@ int smx_compute_node_energies_forces(smx_model* m, int num_nodes, const int* nod
         if (num_nodes > 0 && (!node_types || !num_neigh)) throw smx::Error(SMX_EINVAL, "null node array");
         if (num_edges > 0 && (!neigh_indices || !neigh_types || !xyz || !r)) throw smx::Error(SMX_EINVAL, "null edge array");
         e.stream = nullptr;
-        e.compute(num_nodes, node_types, num_neigh, neigh_indices, neigh_types, xyz, r, num_edges, false, nullptr, nullptr);
+        e.compute(num_nodes, node_types, num_neigh, neigh_indices, neigh_types, xyz, r, num_edges, false, nullptr, nullptr, -1, -1);
         HIPCHK(hipStreamSynchronize(e.stream));
     });
 }
@@ -1368,7 +1387,41 @@ int smx_compute_device(smx_model* m, int num_nodes, const int* d_node_types, con
         if (num_edges > 0 && (!d_neigh_indices || !d_neigh_types || !d_xyz || !d_r)) throw smx::Error(SMX_EINVAL, "null edge array");
         e.stream = static_cast<hipStream_t>(stream);
         e.compute(num_nodes, d_node_types, d_num_neigh, d_neigh_indices, d_neigh_types, d_xyz, d_r, num_edges, true,
-                  d_node_energies, d_node_forces);
+                  d_node_energies, d_node_forces, -1, -1);
+    });
+}
+
+int smx_compute_ghosted(smx_model* m, int num_local_nodes, int num_ghost_nodes, const int* node_types,
+                        const int* num_neigh, const int* neigh_indices, const int* neigh_types, const double* xyz,
+                        const double* r, long num_edges)
+{
+    return guarded([&] {
+        auto& e = E(m);
+        if (num_local_nodes < 0 || num_ghost_nodes < 0) throw smx::Error(SMX_EINVAL, "negative node count");
+        const int n = num_local_nodes + num_ghost_nodes;
+        if (n > 0 && (!node_types || !num_neigh)) throw smx::Error(SMX_EINVAL, "null node array");
+        if (num_edges > 0 && (!neigh_indices || !neigh_types || !xyz || !r)) throw smx::Error(SMX_EINVAL, "null edge array");
+        e.stream = nullptr;
+        e.compute(n, node_types, num_neigh, neigh_indices, neigh_types, xyz, r, num_edges, false, nullptr, nullptr,
+                  num_local_nodes, -1);
+        HIPCHK(hipStreamSynchronize(e.stream));
+    });
+}
+
+int smx_compute_ghosted_device(smx_model* m, int num_local_nodes, int num_ghost_nodes, const int* d_node_types,
+                               const int* d_num_neigh, const int* d_neigh_indices, const int* d_neigh_types,
+                               const double* d_xyz, const double* d_r, long num_edges, long num_local_edges,
+                               double* d_node_energies, double* d_node_forces, void* stream)
+{
+    return guarded([&] {
+        auto& e = E(m);
+        if (num_local_nodes < 0 || num_ghost_nodes < 0 || num_local_edges < 0) throw smx::Error(SMX_EINVAL, "negative count");
+        const int n = num_local_nodes + num_ghost_nodes;
+        if (n > 0 && (!d_node_types || !d_num_neigh)) throw smx::Error(SMX_EINVAL, "null node array");
+        if (num_edges > 0 && (!d_neigh_indices || !d_neigh_types || !d_xyz || !d_r)) throw smx::Error(SMX_EINVAL, "null edge array");
+        e.stream = static_cast<hipStream_t>(stream);
+        e.compute(n, d_node_types, d_num_neigh, d_neigh_indices, d_neigh_types, d_xyz, d_r, num_edges, true,
+                  d_node_energies, d_node_forces, num_local_nodes, num_local_edges);
     });
 }
 

@@ -81,8 +81,8 @@ template <typename F> hipError_t launch_slice_fwd(const SliceParams<F>& p, hipSt
 template <typename F> hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s);
 // forces (+)= sum over slices of fpart, slices added in ascending order
 // (`copy`, if not null, receives the same sums: the caller's output array of the whole-pipeline call)
-hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, double* copy,
-                               hipStream_t s);
+hipError_t launch_fpart_reduce(long edges, long E, int nslices, const double* fpart, double* forces, int accumulate,
+                               double* copy, hipStream_t s);
 
 // H1_adj[j] (+)= sum over edges with sender j of msg[e], in ascending edge order.
 // H_adj[j] (+)= sum of msg[e - e_lo] over the edges e of sender j with e_lo <= e < e_hi, in ascending edge order

@@ -311,12 +311,13 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     }
 }
 
-__global__ void k_fpart_reduce(long n3, int nslices, const double* fpart, double* forces, int accumulate, double* copy)
+__global__ void k_fpart_reduce(long n3, long stride3, int nslices, const double* fpart, double* forces, int accumulate,
+                               double* copy)
 {
     const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n3) return;
     double s = accumulate ? forces[t] : 0.0;
-    for (int q = 0; q < nslices; ++q) s += fpart[(size_t)q * n3 + t];
+    for (int q = 0; q < nslices; ++q) s += fpart[(size_t)q * stride3 + t];
     forces[t] = s;
     if (copy) copy[t] = s;
 }
@@ -394,13 +395,13 @@ template hipError_t launch_slice_fwd<float>(const SliceParams<float>&, hipStream
 template hipError_t launch_slice_bwd<double>(const SliceParams<double>&, hipStream_t);
 template hipError_t launch_slice_bwd<float>(const SliceParams<float>&, hipStream_t);
 
-hipError_t launch_fpart_reduce(long E, int nslices, const double* fpart, double* forces, int accumulate, double* copy,
-                               hipStream_t s)
+hipError_t launch_fpart_reduce(long edges, long E, int nslices, const double* fpart, double* forces, int accumulate,
+                               double* copy, hipStream_t s)
 {
-    const long n3 = 3 * E;
-    if (n3 <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_fpart_reduce, dim3((unsigned)((n3 + 255) / 256)), dim3(256), 0, s, n3, nslices, fpart, forces,
-                       accumulate, copy);
+    const long n3 = 3 * edges;
+    if (n3 <= 0 || edges > E) return n3 <= 0 ? hipSuccess : hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_fpart_reduce, dim3((unsigned)((n3 + 255) / 256)), dim3(256), 0, s, n3, 3 * E, nslices, fpart,
+                       forces, accumulate, copy);
     return hipGetLastError();
 }
 

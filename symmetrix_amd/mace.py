@@ -102,6 +102,18 @@ class MACE:
         _lib.check(self._L.smx_compute_node_energies_forces(
             self._h, int(num_nodes), _pi(nt), _pi(nn), _pi(ni), _pi(nty), _pd(x), _pd(rr), C.c_long(len(rr))))
 
+    def compute_ghosted(self, num_local_nodes, num_ghost_nodes, node_types, num_neigh, neigh_indices, neigh_types, xyz, r):
+        """Ghost atoms as extra nodes that go through layer 0 only: the no_mpi_message_passing mode of the pair
+        style (pair_symmetrix/pair_symmetrix_mace.cpp:557-748).  Local nodes and their edges come first."""
+        nt, nn, ni, nty = _i(node_types), _i(num_neigh), _i(neigh_indices), _i(neigh_types)
+        x, rr = _d(xyz).reshape(-1), _d(r)
+        n = int(num_local_nodes) + int(num_ghost_nodes)
+        if len(nt) < n or len(nn) < n or len(ni) != len(rr) or len(nty) != len(rr) or len(x) != 3 * len(rr):
+            raise ValueError("array lengths do not match the node and edge counts")
+        _lib.check(self._L.smx_compute_ghosted(
+            self._h, int(num_local_nodes), int(num_ghost_nodes), _pi(nt), _pi(nn), _pi(ni), _pi(nty), _pd(x), _pd(rr),
+            C.c_long(len(rr))))
+
     def compute_device(self, num_nodes, node_types, num_neigh, neigh_indices, neigh_types, xyz, r, num_edges,
                        node_energies=0, node_forces=0, stream=0):
         """Device-resident variant: every argument is a device address (int)."""
@@ -109,6 +121,14 @@ class MACE:
             self._h, int(num_nodes), C.c_void_p(node_types), C.c_void_p(num_neigh), C.c_void_p(neigh_indices),
             C.c_void_p(neigh_types), C.c_void_p(xyz), C.c_void_p(r), C.c_long(num_edges),
             C.c_void_p(node_energies), C.c_void_p(node_forces), C.c_void_p(stream)))
+
+    def compute_ghosted_device(self, num_local_nodes, num_ghost_nodes, node_types, num_neigh, neigh_indices, neigh_types,
+                               xyz, r, num_edges, num_local_edges, node_energies=0, node_forces=0, stream=0):
+        """compute_ghosted with every array a device address (int); does not synchronise."""
+        _lib.check(self._L.smx_compute_ghosted_device(
+            self._h, int(num_local_nodes), int(num_ghost_nodes), C.c_void_p(node_types), C.c_void_p(num_neigh),
+            C.c_void_p(neigh_indices), C.c_void_p(neigh_types), C.c_void_p(xyz), C.c_void_p(r), C.c_long(num_edges),
+            C.c_long(num_local_edges), C.c_void_p(node_energies), C.c_void_p(node_forces), C.c_void_p(stream)))
 
     def synchronize(self):
         _lib.check(self._L.smx_synchronize(self._h))

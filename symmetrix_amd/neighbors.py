@@ -164,6 +164,44 @@ def edge_arrays(nl, species_index, num_nodes=None):
     )
 
 
+def ghost_edge_arrays(nl, species_index):
+    """The same periodic system with ghost atoms as explicit nodes, as the pair style lays it out in its
+    no_mpi_message_passing mode (pair_symmetrix/pair_symmetrix_mace.cpp:557-658).
+
+    Local nodes 0..N-1 come first; every periodic image (j, S != 0) that neighbours a local atom becomes a ghost
+    node, ordered by (j, S).  Edges of local receivers point at local or ghost nodes; a ghost node carries the
+    edge list of its owner atom (only species, xyz and r of those edges are used).  sender_atom[edge] and
+    receiver_atom[node] name the owners for the force scatter f[i] -= f_ij, f[j] += f_ij (:700-716).
+    """
+    i, j, S = nl["i"], nl["j"], np.asarray(nl["S"]).reshape(-1, 3)
+    species_index = np.asarray(species_index, dtype=np.int32)
+    N = len(species_index)
+    first = np.asarray(nl["first_neigh"])
+    xyz = np.asarray(nl["xyz"], dtype=np.float64).reshape(-1, 3)
+    r = np.asarray(nl["r"], dtype=np.float64)
+    is_img = np.any(S != 0, axis=1)
+    keys = np.concatenate([j[is_img, None].astype(np.int64), S[is_img].astype(np.int64)], axis=1)
+    ghosts, inverse = (np.unique(keys, axis=0, return_inverse=True) if len(keys) else (np.zeros((0, 4), np.int64), np.zeros(0, np.int64)))
+    G = len(ghosts)
+    neigh_local = j.astype(np.int32).copy()
+    neigh_local[is_img] = N + np.asarray(inverse).reshape(-1).astype(np.int32)
+    owner = ghosts[:, 0].astype(np.int64)
+    counts = (first[1:] - first[:-1]).astype(np.int64)
+    g_edges = np.concatenate([np.arange(first[o], first[o + 1]) for o in owner]) if G else np.zeros(0, np.int64)
+    return dict(
+        num_local_nodes=N, num_ghost_nodes=G,
+        node_types=np.concatenate([species_index, species_index[owner]]).astype(np.int32),
+        num_neigh=np.concatenate([counts, counts[owner]]).astype(np.int32),
+        neigh_indices=np.concatenate([neigh_local, np.zeros(len(g_edges), np.int32)]).astype(np.int32),
+        neigh_types=np.concatenate([species_index[j], species_index[j[g_edges]]]).astype(np.int32),
+        xyz=np.ascontiguousarray(np.concatenate([xyz, xyz[g_edges]])).reshape(-1),
+        r=np.ascontiguousarray(np.concatenate([r, r[g_edges]])),
+        sender_atom=np.concatenate([j, j[g_edges]]).astype(np.int32),
+        receiver_atom=np.concatenate([np.arange(N), owner]).astype(np.int32),
+        ghost_owner=owner.astype(np.int32),
+    )
+
+
 def image_shifts(cell, r_cut, pbc=(True, True, True)):
     """Integer cell shifts (lexicographic order) and their Cartesian vectors, as neighbor_list forms them."""
     cell = np.asarray(cell, dtype=np.float64)

@@ -446,3 +446,63 @@ def test_receiver_chunks_of_the_layer1_adjoint_change_nothing(gpu, tmp_models, d
     eng.set_staging_limit(row_bytes)          # below one receiver's messages
     with pytest.raises(RuntimeError):
         eng.compute_node_energies_forces(*H.call_args(ea))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("L_max,dtype", [(0, "float64"), (1, "float64"), (0, "float32"), (1, "float32")])
+def test_pair_style_modes_agree(gpu, tmp_models, L_max, dtype):
+    """The three ways the pair style feeds the engine on one rank give one answer (the reference's
+    tests/test_pair_symmetrix_mace.py:28-39): owners as senders (no_domain_decomposition), ghost nodes that go
+    through layer 0 (no_mpi_message_passing, one call), and ghost rows of H1 filled by a forward copy with the
+    adjoint summed back (mpi_message_passing, stage calls as pair_symmetrix_mace.cpp:372-550 issues them)."""
+    from symmetrix_amd import neighbors
+    model = H.tiny_model(K=16, L_max=L_max, n_pts=48, seed=12, zbl=(dtype == "float32"), density=(L_max == 1))
+    path = H.write_model(model, tmp_models / f"modes{L_max}{dtype}.json")
+    pos, cell, sp = H.small_system(36, seed=21)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    N = len(sp)
+    eng = gpu(path, dtype)
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    e_ref = eng.node_energies.copy()
+    f_ref = eng.reduce_forces(N, ea["neigh_indices"])
+    ga = neighbors.ghost_edge_arrays(nl, sp)
+    Nl, Ng = ga["num_local_nodes"], ga["num_ghost_nodes"]
+    assert Ng > 0
+    print(f"ghost mode: {Nl} local + {Ng} ghost nodes, {len(ga['r'])} edges", flush=True)
+    eng.compute_ghosted(Nl, Ng, ga["node_types"], ga["num_neigh"], ga["neigh_indices"], ga["neigh_types"], ga["xyz"], ga["r"])
+    e_g = eng.node_energies.copy()
+    f_g = eng.reduce_forces(N, ga["sender_atom"], ga["receiver_atom"])
+    assert e_g.shape == (Nl,)
+    ftol = 1e-11 if dtype == "float64" else 2e-5
+    assert np.array_equal(e_g, e_ref)      # same edges in the same order for every local receiver
+    assert np.abs(f_g - f_ref).max() <= ftol * max(1.0, np.abs(f_ref).max())
+
+    # message-passing mode: local nodes only; H1 of the ghosts copied from their owners, H1_adj summed back
+    El = int(ga["num_neigh"][:Nl].sum())
+    nt, nn = ga["node_types"][:Nl], ga["num_neigh"][:Nl]
+    ni, nty, x, r = ga["neigh_indices"][:El], ga["neigh_types"][:El], ga["xyz"][:3 * El], ga["r"][:El]
+    eng2 = gpu(path, dtype)
+    eng2.node_energies = np.zeros(Nl); eng2.node_forces = np.zeros(3 * El)
+    if model["has_zbl"]:
+        return      # the stage calls hold no separate ZBL step; the two whole-pipeline modes above cover it
+    eng2.compute_Y(x)
+    eng2.compute_R0(Nl, nt, nn, nty, r); eng2.compute_A0(Nl, nt, nn, nty); eng2.compute_A0_scaled(Nl, nt, nn, nty, r)
+    eng2.compute_M0(Nl, nt); eng2.compute_H1(Nl)
+    nlm_k = eng2.H1.size // Nl
+    H1 = np.array(eng2.H1).reshape(Nl, nlm_k)
+    eng2.H1 = np.concatenate([H1, H1[ga["ghost_owner"]]]).reshape(-1)          # forward_comm
+    eng2.compute_R1(Nl, nt, nn, nty, r); eng2.compute_Phi1(Nl, nn, ni); eng2.compute_A1(Nl)
+    eng2.compute_A1_scaled(Nl, nt, nn, nty, r); eng2.compute_M1(Nl, nt); eng2.compute_H2(Nl, nt)
+    eng2.compute_readouts(Nl, nt)
+    eng2.reverse_H2(Nl, nt, False); eng2.reverse_M1(Nl, nt)
+    eng2.reverse_A1_scaled(Nl, nt, nn, nty, x, r, False); eng2.reverse_A1(Nl)
+    eng2.reverse_Phi1(Nl, nn, ni, x, r, False, False)
+    Hadj = np.array(eng2.H1_adj).reshape(Nl + Ng, nlm_k)
+    np.add.at(Hadj, ga["ghost_owner"], Hadj[Nl:])                                # reverse_comm
+    eng2.H1_adj = Hadj[:Nl].reshape(-1).copy()
+    eng2.reverse_H1(Nl); eng2.reverse_M0(Nl, nt); eng2.reverse_A0_scaled(Nl, nt, nn, nty, x, r)
+    eng2.reverse_A0(Nl, nt, nn, nty, x, r)
+    etol = 1e-12 if dtype == "float64" else 1e-6
+    assert np.abs(eng2.node_energies - e_ref).max() <= etol * max(1.0, np.abs(e_ref).max())
+    f_m = eng2.reduce_forces(N, ga["sender_atom"][:El])
+    assert np.abs(f_m - f_ref).max() <= ftol * 10 * max(1.0, np.abs(f_ref).max())

@@ -692,20 +692,12 @@ struct Engine : EngineBase {
         node_energies.resize((size_t)N, stream);
         H1_adj.size_to(H1.n, stream);
         H2_adj.size_to(H2.n, stream);
-        hidden.size_to((size_t)N * 16, stream);
         const int rows = (int)(H1.n / ((size_t)nlm * k));
-        HIPCHK(launch_seed_H1_adj<F>(rows, N, nlm, k, ro1.p, H1_adj.p, stream));
-        auto g1 = gemm_base<double, double, double>(N, false);
-        g1.nprob = 1;
-        g1.prob[0] = gemm_prob<double, double, double>(H2.p, k, 0, 0, hidden.p, 16, 0, 0, ro2_w1.p, 0, 0, 1, 0, k, 16, 1);
-        HIPCHK((launch_gemm<double, double, double>(g1, stream)));
-        HIPCHK(launch_readout<F>(N, k, nlm, node_types, E0.p, ro1.p, H1.p, hidden.p, ro2_w2.p, hm.readout_2_scale,
-                                 node_energies.p, zero_energies ? 1 : 0, energies_copy, stream));
+        if (rows < N || H2.n < (size_t)N * k) throw Error(SMX_EINVAL, "readouts called before H1 and H2 exist for these nodes");
+        HIPCHK(launch_readout_fused<F>(N, rows, k, nlm, node_types, E0.p, ro1.p, ro2_w1.p, ro2_w2.p, hm.readout_2_scale,
+                                       H1.p, H2.p, H2_adj.p, H1_adj.p, node_energies.p, zero_energies ? 1 : 0,
+                                       energies_copy, stream));
         energies_copy = nullptr;
-        auto g2 = gemm_base<double, double, double>(N, false);
-        g2.nprob = 1;
-        g2.prob[0] = gemm_prob<double, double, double>(hidden.p, 16, 0, 0, H2_adj.p, k, 0, 0, ro2_w1.p, 0, 0, 0, 0, 16, k, 1);
-        HIPCHK((launch_gemm<double, double, double>(g2, stream)));
     }
     void st_reverse_M1(int N)
     {

@@ -213,18 +213,14 @@ template <typename TA, typename TC, typename CT>
 hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p, hipStream_t s);
 
 // ---------------------------------------------------------------------------
-// Readout tail (MACE::compute_readouts, mace.cpp:876-903) after the two MFMA
-// products: hidden[N][16] = H2 . W1^T has been formed; this applies the scaled
-// SiLU, adds E0 + w1.H1[l=0] + w2.act to the node energy and leaves
-// g[N][16] = w2 * act' for the product g . W1 that yields H2_adj.
+// Readout tail (MACE::compute_readouts, mace.cpp:876-903) in one launch: node_energies[i] (+)= E0[type] +
+// w1 . H1[i, l=0] + MLP_{K->16->1}(H2[i]) with W1[16][K], H2_adj = gradient of the network, H1_adj[rows][num_LM][K]
+// seeded with w1 in the scalar block of the first N rows and zero elsewhere.
 template <typename F>
-hipError_t launch_readout(int N, int K, int num_LM, const int* node_types, const double* atomic_energies,
-                          const double* w1, const F* H1, double* hidden_g, const double* w2, double scale,
-                          double* node_energies, int zero_energies, double* energies_copy, hipStream_t s);
-// H1_adj: zero everywhere (rows x num_LM x K), l=0 block of the first N rows = readout_1 weights
-template <typename F>
-hipError_t launch_seed_H1_adj(int rows, int N, int num_LM, int K, const double* w1, F* H1_adj, hipStream_t s);
-
+hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
+                                const double* w1, const double* W1, const double* w2, double scale, const F* H1,
+                                const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
+                                double* energies_copy, hipStream_t s);
 template <typename T> hipError_t launch_fill(T* p, long n, T v, hipStream_t s);
 template <typename TS, typename TD> hipError_t launch_convert(const TS* src, TD* dst, long n, hipStream_t s);
 

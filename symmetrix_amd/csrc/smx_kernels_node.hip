@@ -516,70 +516,89 @@ template hipError_t launch_poly_reverse<float>(int, int, int, const float*, cons
 
 // ===========================================================================
 // Readout tail
+// The whole readout tail in one launch (mace.cpp:876-903, multilayer_perceptron.cpp:76-150): the K -> 16 -> 1
+// network on H2 with its gradient (H2_adj), the linear readout of H1's scalar block, the atomic energy, and the
+// seed of H1_adj (readout weights in the scalar block of the first N rows, zero elsewhere).  A block serves 16
+// nodes; thread (node, hidden unit) forms one hidden activation with the K products taken in ascending order.
 namespace {
 template <typename F>
-__global__ void k_readout(int N, int K, int num_LM, const int* node_types, const double* E0, const double* w1,
-                          const F* H1, double* hidden_g, const double* w2, double scale, double* node_energies,
-                          int zero_energies, double* energies_copy)
+__global__ __launch_bounds__(256) void k_readout_fused(int N, int rows, int K, int num_LM, const int* node_types,
+                                                       const double* E0, const double* w1, const double* W1,
+                                                       const double* w2, double scale, const F* H1, const double* H2,
+                                                       double* H2_adj, F* H1_adj, double* node_energies,
+                                                       int zero_energies, double* energies_copy)
 {
-    // 16 threads per node: thread h owns hidden unit h
-    const int i = blockIdx.x * (blockDim.x / 16) + threadIdx.x / 16;
-    const int h = threadIdx.x & 15;
-    if (i >= N) return;
-    // multilayer_perceptron.cpp:107-113: scaled SiLU and its derivative
-    const double x = hidden_g[(size_t)i * 16 + h];
-    const double sig = 1.0 / (1.0 + exp(-x));
-    const double act = scale * x * sig;
-    const double dact = scale * sig + scale * x * sig * (1 - sig);
-    double e = w2[h] * act;
-    hidden_g[(size_t)i * 16 + h] = w2[h] * dact;
-    // first readout: w1 . H1[i, l=0, :]
-    const F* H = H1 + (size_t)i * num_LM * K;
-    for (int k = h; k < K; k += 16) e += w1[k] * (double)H[k];
+    extern __shared__ double rsm[];
+    const int ldw = K + 1;                 // rows of W1 start two banks apart
+    double* W = rsm;                       // [16][K + 1]
+    double* hg = W + 16 * ldw;             // [16 nodes][16]
+    double* X = hg + 256;                  // [16 nodes][K]: the block's rows of H2
+    for (int t = threadIdx.x; t < 16 * K; t += 256) {
+        W[(t / K) * ldw + t % K] = W1[t];
+        const size_t src = (size_t)blockIdx.x * 16 * K + t;
+        X[t] = src < (size_t)N * K ? H2[src] : 0.0;
+    }
+    __syncthreads();
+    const int n = threadIdx.x >> 4, h = threadIdx.x & 15;
+    const int i = blockIdx.x * 16 + n;
+    double e = 0.0, g = 0.0;
+    if (i < N) {
+        const double* h2 = X + n * K;
+        double s = 0.0;
+        for (int k = 0; k < K; ++k) s += W[h * ldw + k] * h2[k];
+        // multilayer_perceptron.cpp:107-113: scaled SiLU and its derivative
+        const double sig = 1.0 / (1.0 + exp(-s));
+        e = w2[h] * (scale * s * sig);
+        g = w2[h] * (scale * sig + scale * s * sig * (1 - sig));
+        const F* Hs = H1 + (size_t)i * num_LM * K;
+        for (int k = h; k < K; k += 16) e += w1[k] * (double)Hs[k];
+    }
 #pragma unroll
     for (int off = 8; off >= 1; off >>= 1) e += __shfl_xor(e, off, 64);
-    if (h == 0) {
-        const double base = zero_energies ? 0.0 : node_energies[i];
-        const double en = base + E0[node_types[i]] + e;
+    hg[threadIdx.x] = g;
+    if (h == 0 && i < N) {
+        const double en = (zero_energies ? 0.0 : node_energies[i]) + E0[node_types[i]] + e;
         node_energies[i] = en;
         if (energies_copy) energies_copy[i] = en;
     }
-}
-template <typename F>
-__global__ void k_seed_H1_adj(long total, int N, int num_LM, int K, const double* w1, F* H1_adj)
-{
-    const long idx = (long)blockIdx.x * blockDim.x + threadIdx.x;
-    if (idx >= total) return;
-    const int k = (int)(idx % K);
-    const long t = idx / K;
-    const int lm = (int)(t % num_LM);
-    const long i = t / num_LM;
-    H1_adj[idx] = (lm == 0 && i < N) ? (F)w1[k] : F(0);
+    __syncthreads();
+    for (int t = threadIdx.x; t < 16 * K; t += 256) {
+        const int n2 = t / K, k = t - n2 * K;
+        const int i2 = blockIdx.x * 16 + n2;
+        if (i2 < N) {
+            double s = 0.0;
+#pragma unroll
+            for (int q = 0; q < 16; ++q) s += hg[n2 * 16 + q] * W[q * ldw + k];
+            H2_adj[(size_t)i2 * K + k] = s;
+        }
+    }
+    const int width = num_LM * K;
+    for (int t = threadIdx.x; t < 16 * width; t += 256) {
+        const int n2 = t / width, c = t - n2 * width;
+        const int row = blockIdx.x * 16 + n2;
+        if (row < rows) H1_adj[(size_t)row * width + c] = (c < K && row < N) ? (F)w1[c] : F(0);
+    }
 }
 }  // namespace
 
 template <typename F>
-hipError_t launch_readout(int N, int K, int num_LM, const int* node_types, const double* atomic_energies,
-                          const double* w1, const F* H1, double* hidden_g, const double* w2, double scale,
-                          double* node_energies, int zero_energies, double* energies_copy, hipStream_t s)
+hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
+                                const double* w1, const double* W1, const double* w2, double scale, const F* H1,
+                                const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
+                                double* energies_copy, hipStream_t s)
 {
-    if (N > 0)
-        hipLaunchKernelGGL(k_readout<F>, dim3(nblk((long)N * 16, 256)), dim3(256), 0, s, N, K, num_LM, node_types,
-                           atomic_energies, w1, H1, hidden_g, w2, scale, node_energies, zero_energies, energies_copy);
+    if (rows < N) return hipErrorInvalidValue;
+    if (rows <= 0) return hipSuccess;
+    const size_t lds = ((size_t)16 * (K + 1) + 256 + (size_t)16 * K) * sizeof(double);
+    if (lds > 64 * 1024) return hipErrorInvalidValue;
+    hipLaunchKernelGGL(k_readout_fused<F>, dim3((rows + 15) / 16), dim3(256), lds, s, N, rows, K, num_LM, node_types,
+                       atomic_energies, w1, W1, w2, scale, H1, H2, H2_adj, H1_adj, node_energies, zero_energies,
+                       energies_copy);
     return hipGetLastError();
 }
-template hipError_t launch_readout<double>(int, int, int, const int*, const double*, const double*, const double*, double*, const double*, double, double*, int, double*, hipStream_t);
-template hipError_t launch_readout<float>(int, int, int, const int*, const double*, const double*, const float*, double*, const double*, double, double*, int, double*, hipStream_t);
+template hipError_t launch_readout_fused<double>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const double*, const double*, double*, double*, double*, int, double*, hipStream_t);
+template hipError_t launch_readout_fused<float>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const float*, const double*, double*, float*, double*, int, double*, hipStream_t);
 
-template <typename F>
-hipError_t launch_seed_H1_adj(int rows, int N, int num_LM, int K, const double* w1, F* H1_adj, hipStream_t s)
-{
-    const long total = (long)rows * num_LM * K;
-    if (total > 0) hipLaunchKernelGGL(k_seed_H1_adj<F>, dim3(nblk(total, 256)), dim3(256), 0, s, total, N, num_LM, K, w1, H1_adj);
-    return hipGetLastError();
-}
-template hipError_t launch_seed_H1_adj<double>(int, int, int, int, const double*, double*, hipStream_t);
-template hipError_t launch_seed_H1_adj<float>(int, int, int, int, const double*, float*, hipStream_t);
 
 // ===========================================================================
 // Caller-side reductions: per-edge forces -> per-atom forces (each atom sums its

@@ -38,12 +38,17 @@ STAGE_KERNEL = {
 }
 
 # HBM bytes per launch from rocprofv3 counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the factors read off a
-# 1 GiB copy in the same runs), full-size off_small workload only: profiles/edge_kernels_off_small_hbm_traffic.txt
+# 1 GiB copy in the same runs), full-size workloads only: profiles/edge_kernels_off_small_hbm_traffic.txt and
+# profiles/edge_kernels_mp_medium_hbm_traffic.txt
 MEASURED_TRAFFIC = {
-    ("off_small", "float64"): {"agg0_fwd": 78.9e6, "agg1_fwd": 106.1e6, "agg1_bwd": 434.8e6, "agg0_bwd": 258.0e6,
-                               "sender_reduce": 93.2e6},
-    ("off_small", "float32"): {"agg0_fwd": 58.9e6, "agg1_fwd": 84.2e6, "agg1_bwd": 243.5e6, "agg0_bwd": 148.8e6,
-                               "sender_reduce": 47.4e6},
+    ("off_small", "float64"): {"agg0_fwd": 78.9e6, "agg1_fwd": 106.0e6, "agg1_bwd": 436.8e6, "agg0_bwd": 257.9e6,
+                               "sender_reduce": 93.6e6},
+    ("off_small", "float32"): {"agg0_fwd": 58.8e6, "agg1_fwd": 86.2e6, "agg1_bwd": 247.3e6, "agg0_bwd": 151.8e6,
+                               "sender_reduce": 47.7e6},
+    ("mp_medium", "float32"): {"agg0_fwd": 1700.6e6, "agg1_fwd": 9676.8e6, "agg1_bwd": 16227.3e6, "agg0_bwd": 4480.1e6,
+                               "sender_reduce": 8257.2e6},
+    ("mp_medium", "float64"): {"agg0_fwd": 2099.7e6, "agg1_fwd": 20267.6e6, "agg1_bwd": 46609.2e6, "agg0_bwd": 7626.2e6,
+                               "sender_reduce": 16442.4e6},
 }
 
 
@@ -377,7 +382,7 @@ def main():
             "bound": "hbm", "kernel": STAGE_KERNEL[dom][0 if L_max == 0 else 1], "stage": dom,
             "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
             "frac": achieved / (HBM_PEAK / 1e9),
-            "traffic": MEASURED_TRAFFIC.get((args.workload, args.dtype), {}).get(dom) if args.scale == 1.0 else None,
+            "traffic": MEASURED_TRAFFIC.get((args.workload, args.dtype), {}).get(dom) if args.scale == 1.0 and not args.ghosts else None,
             "algorithmic_bytes_per_launch": dom_bytes,
             "whole_step_algorithmic_bytes": total_bytes,
             "whole_step_frac": (total_bytes / HBM_PEAK) / (res["ms"] * 1e-3),

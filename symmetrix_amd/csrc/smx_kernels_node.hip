@@ -545,6 +545,7 @@ __global__ __launch_bounds__(256) void k_readout_fused(int N, int rows, int K, i
     if (i < N) {
         const double* h2 = X + n * K;
         double s = 0.0;
+#pragma unroll 8
         for (int k = 0; k < K; ++k) s += W[h * ldw + k] * h2[k];
         // multilayer_perceptron.cpp:107-113: scaled SiLU and its derivative
         const double sig = 1.0 / (1.0 + exp(-s));

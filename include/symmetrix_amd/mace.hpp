@@ -70,6 +70,19 @@ public:
         pull("node_energies", node_energies);
         pull("node_forces", node_forces);
     }
+    // Ghost atoms as extra nodes that go through layer 0 only: the stage sequence of
+    // PairSymmetrixMACE::compute_no_mpi_message_passing (pair_symmetrix_mace.cpp:660-698) as one call.
+    // No counterpart among the reference's methods.
+    void compute_node_energies_forces_ghosted(const int num_local_nodes, const int num_ghost_nodes,
+                                              std::span<const int> node_types, std::span<const int> num_neigh,
+                                              std::span<const int> neigh_indices, std::span<const int> neigh_types,
+                                              std::span<const double> xyz, std::span<const double> r)
+    {
+        check(smx_compute_ghosted(m_, num_local_nodes, num_ghost_nodes, node_types.data(), num_neigh.data(),
+                                  neigh_indices.data(), neigh_types.data(), xyz.data(), r.data(), (long)r.size()));
+        pull("node_energies", node_energies);
+        pull("node_forces", node_forces);
+    }
     void compute_R0(const int num_nodes, std::span<const int> node_types, std::span<const int> num_neigh,
                     std::span<const int> neigh_types, std::span<const double> r)
     { check(smx_compute_R0(m_, num_nodes, node_types.data(), num_neigh.data(), neigh_types.data(), r.data(), (long)r.size())); }

@@ -188,6 +188,9 @@ int smx_synchronize(smx_model* m);
  * compute.  Outputs are host arrays. */
 int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const int* receiver_atom,
                       double* atom_forces, double* virial);
+/* The same with sender_atom a device array (e.g. neigh_indices of smx_nlist_arrays) and receiver i = atom i. */
+int smx_reduce_forces_device(smx_model* m, int num_atoms, const int* d_sender_atom, double* atom_forces,
+                             double* virial);
 
 /* Full neighbour list built on the device, counterpart of the edge construction of
  * pair_symmetrix_mace.cpp:246-315 (ghost images, r^2 < r_cut^2) and of the ASE caller's
@@ -213,6 +216,14 @@ int smx_nlist_build(smx_nlist* nl, int num_atoms, const double* d_positions, con
  * as no pair outside r_list at build time has come inside r_cut since. */
 int smx_nlist_update(smx_nlist* nl, const double* d_positions, const int* d_types, double r_cut, void* stream,
                      long* num_edges);
+/* Variants for callers that hold positions and species in host memory (the ASE calculator,
+ * symmetrix_calc.py:72-83): the list object keeps device copies (smx_nlist_inputs returns their addresses, to be
+ * handed to smx_compute_device as node_types) and the calls synchronise.  An update reuses the species of the
+ * last build. */
+int smx_nlist_build_host(smx_nlist* nl, int num_atoms, const double* positions, const int* types, int num_shifts,
+                         const int* shift_int, const double* shift_vec, double r_list, double r_cut, long* num_edges);
+int smx_nlist_update_host(smx_nlist* nl, const double* positions, double r_cut, long* num_edges);
+int smx_nlist_inputs(smx_nlist* nl, const double** d_positions, const int** d_types);
 int smx_nlist_arrays(smx_nlist* nl, const int** num_neigh, const int** first_neigh, const int** neigh_indices,
                      const int** neigh_types, const int** neigh_shift, const double** xyz, const double** r);
 int smx_nlist_copy_to_host(smx_nlist* nl, int* num_neigh, int* neigh_indices, int* neigh_types, int* neigh_shift,

@@ -3,7 +3,10 @@ configuration, the work of `Symmetrix.calculate`
 (symmetrix/source/symmetrix/symmetrix_calc.py:72-102), without requiring ASE.
 
 `SymmetrixCalculator.compute(positions, cell, atomic_numbers)` builds the
-canonical neighbour list, calls the engine and reduces per-edge forces to atoms
+canonical neighbour list on the device (the counterpart of the
+neighbor_list('ijdD') call at symmetrix_calc.py:77-83; bit-identical to the
+numpy builder of this package, which `neighbor_list="host"` selects), calls the
+engine on the device-resident edge arrays and reduces per-edge forces to atoms
 on the device.  When ASE is importable, `Symmetrix` is an
 `ase.calculators.calculator.Calculator` with the reference's constructor
 signature and `implemented_properties`.
@@ -19,12 +22,15 @@ from .mace import MACE
 class SymmetrixCalculator:
     implemented_properties = ["energy", "free_energy", "energies", "forces", "stress"]
 
-    def __init__(self, model_file, dtype="float64"):
+    def __init__(self, model_file, dtype="float64", neighbor_list="device"):
         if dtype not in ("float32", "float64"):
             raise ValueError(f"Unsupported dtype '{dtype}'. Supported dtypes are 'float64' and 'float32'.")
+        if neighbor_list not in ("device", "host"):
+            raise ValueError("neighbor_list is 'device' or 'host'")
         self.evaluator = MACE(str(model_file), dtype)
         self.cutoff = self.evaluator.r_cut
         self.results = {}
+        self._nlist = neighbors.DeviceNeighborList() if neighbor_list == "device" else None
 
     def compute(self, positions, cell, atomic_numbers, pbc=(True, True, True)):
         Z = [int(z) for z in atomic_numbers]
@@ -33,14 +39,26 @@ class SymmetrixCalculator:
             species = np.array([table.index(z) for z in Z], dtype=np.int32)
         except ValueError as exc:
             raise ValueError("an atom's element is not in the model") from exc
-        nl = neighbors.neighbor_list(positions, cell, self.cutoff, pbc)
-        ea = neighbors.edge_arrays(nl, species)
         ev = self.evaluator
-        ev.compute_node_energies_forces(ea["num_nodes"], ea["node_types"], ea["num_neigh"], ea["neigh_indices"],
-                                        ea["neigh_types"], ea["xyz"], ea["r"])
-        energies = ev.node_energies
         n_atoms = len(Z)
-        forces, virial = ev.reduce_forces(n_atoms, nl["j"], virial=True)
+        if self._nlist is not None:
+            E = self._nlist.build_host(positions, species, cell, self.cutoff, pbc)
+            p = self._nlist.ptr
+            ev.compute_device(n_atoms, p["node_types"], p["num_neigh"], p["neigh_indices"], p["neigh_types"], p["xyz"],
+                              p["r"], E)
+            ev.synchronize()
+            energies = ev.node_energies
+            if E:
+                forces, virial = ev.reduce_forces_device(n_atoms, p["neigh_indices"], virial=True)
+            else:
+                forces, virial = np.zeros((n_atoms, 3)), np.zeros(6)
+        else:
+            nl = neighbors.neighbor_list(positions, cell, self.cutoff, pbc)
+            ea = neighbors.edge_arrays(nl, species)
+            ev.compute_node_energies_forces(ea["num_nodes"], ea["node_types"], ea["num_neigh"], ea["neigh_indices"],
+                                            ea["neigh_types"], ea["xyz"], ea["r"])
+            energies = ev.node_energies
+            forces, virial = ev.reduce_forces(n_atoms, nl["j"], virial=True)
         cell = np.asarray(cell, dtype=np.float64)
         volume = abs(np.linalg.det(np.diag(cell) if cell.shape == (3,) else cell))
         # symmetrix_calc.py:102: stress = -(pair_forces^T xyz)/V in Voigt order xx,yy,zz,yz,xz,xy

@@ -130,7 +130,7 @@ struct EngineBase {
     virtual void get_array(const char* name, double* out, long cap, long* n) = 0;
     virtual void set_array(const char* name, const double* in, long n) = 0;
     virtual void reduce_forces(int num_atoms, const int* sender_atom, const int* receiver_atom,
-                               double* atom_forces, double* virial) = 0;
+                               double* atom_forces, double* virial, bool sender_on_device) = 0;
 
     void stage_begin(int st)
     {
@@ -1060,7 +1060,7 @@ struct Engine : EngineBase {
     DVec<int> rf_send, rf_recv, rf_count, rf_sstart, rf_cursor, rf_slist, rf_rstart, rf_rlist;
     DVec<double> rf_out;
     void reduce_forces(int num_atoms, const int* sender_atom, const int* receiver_atom, double* atom_forces,
-                       double* virial) override
+                       double* virial, bool sender_on_device) override
     {
         hipStream_t s = stream;
         need(node_forces.p, "node_forces");
@@ -1068,12 +1068,13 @@ struct Engine : EngineBase {
         if (atom_forces) {
             if (num_atoms <= 0) throw Error(SMX_EINVAL, "num_atoms must be positive");
             if (!sender_atom) throw Error(SMX_EINVAL, "sender_atom is required");
-            rf_send.upload(sender_atom, (size_t)E, s);
+            const int* send = sender_atom;
+            if (!sender_on_device) { rf_send.upload(sender_atom, (size_t)E, s); send = rf_send.p; }
             rf_count.size_to(num_atoms, s); rf_cursor.size_to(num_atoms, s);
             rf_sstart.size_to((size_t)num_atoms + 1, s); rf_slist.size_to((size_t)E, s);
             scan_tmp.size_to((size_t)num_atoms / 1024 + 2, s);
             HIPCHK(hipMemsetAsync(flags.p, 0, sizeof(int), s));
-            HIPCHK(launch_check_range(rf_send.p, E, num_atoms, flags.p, s));
+            HIPCHK(launch_check_range(send, E, num_atoms, flags.p, s));
             {
                 int f = 0;
                 HIPCHK(hipMemcpyAsync(&f, flags.p, sizeof(int), hipMemcpyDeviceToHost, s));
@@ -1108,7 +1109,7 @@ struct Engine : EngineBase {
                 HIPCHK(hipStreamSynchronize(s));
                 rstart = rf_rstart.p;
             }
-            HIPCHK(launch_sender_lists(rf_send.p, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, 0, s));
+            HIPCHK(launch_sender_lists(send, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, 0, s));
             rf_out.size_to((size_t)3 * num_atoms, s);
             HIPCHK(launch_force_scatter(num_atoms, rstart, rlist, rf_sstart.p, rf_slist.p, node_forces.p, rf_out.p, s));
             HIPCHK(hipMemcpyAsync(atom_forces, rf_out.p, (size_t)3 * num_atoms * sizeof(double), hipMemcpyDeviceToHost, s));
@@ -1191,6 +1192,8 @@ struct NeighborList {
     DVec<int> shift_int, atom_bin, bin_count, bin_start, bin_atoms, count, cfirst, first, num_neigh, neigh_indices,
         neigh_types, neigh_shift, scan_tmp;
     DVec<long long> keys, sorted;
+    DVec<double> pos_dev;     // copies of host inputs (smx_nlist_build_host / smx_nlist_update_host)
+    DVec<int> types_dev;
     int N = 0, num_shifts = 0;
     long E = 0, num_candidates = 0;
     double r_list = 0.0;
@@ -1576,7 +1579,11 @@ int smx_synchronize(smx_model* m)
 int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const int* receiver_atom,
                       double* atom_forces, double* virial)
 {
-    return guarded([&] { E(m).reduce_forces(num_atoms, sender_atom, receiver_atom, atom_forces, virial); });
+    return guarded([&] { E(m).reduce_forces(num_atoms, sender_atom, receiver_atom, atom_forces, virial, false); });
+}
+int smx_reduce_forces_device(smx_model* m, int num_atoms, const int* d_sender_atom, double* atom_forces, double* virial)
+{
+    return guarded([&] { E(m).reduce_forces(num_atoms, d_sender_atom, nullptr, atom_forces, virial, true); });
 }
 
 smx_nlist* smx_nlist_create(void)
@@ -1606,6 +1613,45 @@ int smx_nlist_update(smx_nlist* nl, const double* d_positions, const int* d_type
         if (!nl) throw smx::Error(SMX_EINVAL, "null argument");
         const long e = reinterpret_cast<smx::NeighborList*>(nl)->update(d_positions, d_types, r_cut, (hipStream_t)stream);
         if (num_edges) *num_edges = e;
+    });
+}
+int smx_nlist_build_host(smx_nlist* nl, int num_atoms, const double* positions, const int* types, int num_shifts,
+                         const int* shift_int, const double* shift_vec, double r_list, double r_cut, long* num_edges)
+{
+    return guarded([&] {
+        if (!nl || !shift_int || !shift_vec || num_atoms < 0 || (num_atoms > 0 && (!positions || !types)))
+            throw smx::Error(SMX_EINVAL, "null argument");
+        if (!(r_cut > 0.0) || r_cut > r_list) throw smx::Error(SMX_EINVAL, "neighbour list: need 0 < r_cut <= r_list");
+        require_device();
+        auto& n = *reinterpret_cast<smx::NeighborList*>(nl);
+        n.pos_dev.upload(positions, (size_t)3 * num_atoms, nullptr);
+        n.types_dev.upload(types, (size_t)num_atoms, nullptr);
+        n.build(num_atoms, n.pos_dev.p, num_shifts, shift_int, shift_vec, r_list, nullptr);
+        const long e = n.update(n.pos_dev.p, n.types_dev.p, r_cut, nullptr);
+        HIPCHK(hipStreamSynchronize(nullptr));
+        if (num_edges) *num_edges = e;
+    });
+}
+int smx_nlist_update_host(smx_nlist* nl, const double* positions, double r_cut, long* num_edges)
+{
+    return guarded([&] {
+        if (!nl) throw smx::Error(SMX_EINVAL, "null argument");
+        auto& n = *reinterpret_cast<smx::NeighborList*>(nl);
+        if (n.types_dev.n != (size_t)n.N || (n.N > 0 && !positions))
+            throw smx::Error(SMX_EINVAL, "neighbour list: update from host positions needs a build from host positions first");
+        n.pos_dev.upload(positions, (size_t)3 * n.N, nullptr);
+        const long e = n.update(n.pos_dev.p, n.types_dev.p, r_cut, nullptr);
+        HIPCHK(hipStreamSynchronize(nullptr));
+        if (num_edges) *num_edges = e;
+    });
+}
+int smx_nlist_inputs(smx_nlist* nl, const double** d_positions, const int** d_types)
+{
+    return guarded([&] {
+        if (!nl) throw smx::Error(SMX_EINVAL, "null argument");
+        auto& n = *reinterpret_cast<smx::NeighborList*>(nl);
+        if (d_positions) *d_positions = n.pos_dev.p;
+        if (d_types) *d_types = n.types_dev.p;
     });
 }
 int smx_nlist_arrays(smx_nlist* nl, const int** num_neigh, const int** first_neigh, const int** neigh_indices,

@@ -156,6 +156,14 @@ class MACE:
                                              _pd(F), _pd(V) if virial else None))
         return (F, V) if virial else F
 
+    def reduce_forces_device(self, num_atoms, sender_atom_ptr, virial=False):
+        """reduce_forces with the per-edge sender atoms in a device array (receiver i = atom i)."""
+        F = np.zeros((num_atoms, 3))
+        V = np.zeros(6)
+        _lib.check(self._L.smx_reduce_forces_device(self._h, int(num_atoms), C.c_void_p(sender_atom_ptr), _pd(F),
+                                                    _pd(V) if virial else None))
+        return (F, V) if virial else F
+
     # --- stages --------------------------------------------------------------
     def compute_Y(self, xyz):
         x = _d(xyz).reshape(-1)

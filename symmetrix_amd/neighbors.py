@@ -256,6 +256,9 @@ class DeviceNeighborList:
         out = [C.c_void_p(0) for _ in self._names]
         self._lib.check(self._L.smx_nlist_arrays(C.c_void_p(self._h), *[C.byref(o) for o in out]))
         self.ptr = {n: (o.value or 0) for n, o in zip(self._names, out)}
+        dp, dt = C.c_void_p(0), C.c_void_p(0)
+        self._lib.check(self._L.smx_nlist_inputs(C.c_void_p(self._h), C.byref(dp), C.byref(dt)))
+        self.ptr["positions"], self.ptr["node_types"] = dp.value or 0, dt.value or 0
         return self.num_edges
 
     def build(self, num_atoms, positions_ptr, types_ptr, cell, r_cut, pbc=(True, True, True), skin=0.0, stream=0):
@@ -269,6 +272,35 @@ class DeviceNeighborList:
             ints.ctypes.data_as(C.POINTER(C.c_int)), vecs.ctypes.data_as(C.POINTER(C.c_double)), C.c_double(r_list),
             C.c_double(r_cut), C.c_void_p(stream), C.byref(E)))
         self.num_atoms = int(num_atoms)
+        return self._refresh(E.value)
+
+    def build_host(self, positions, types, cell, r_cut, pbc=(True, True, True), skin=0.0):
+        """build() from numpy positions [N][3] and species indices [N]; device copies are kept in the list object
+        (addresses in .ptr["positions"], .ptr["node_types"])."""
+        C = self._C
+        pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
+        ty = np.ascontiguousarray(types, dtype=np.int32)
+        if len(ty) != len(pos):
+            raise ValueError("positions and types differ in length")
+        r_list = float(r_cut) + float(skin)
+        ints, vecs = image_shifts(cell, r_list, pbc)
+        E = C.c_long(0)
+        self._lib.check(self._L.smx_nlist_build_host(
+            C.c_void_p(self._h), len(pos), pos.ctypes.data_as(C.POINTER(C.c_double)), ty.ctypes.data_as(C.POINTER(C.c_int)),
+            len(ints), ints.ctypes.data_as(C.POINTER(C.c_int)), vecs.ctypes.data_as(C.POINTER(C.c_double)),
+            C.c_double(r_list), C.c_double(r_cut), C.byref(E)))
+        self.num_atoms = len(pos)
+        return self._refresh(E.value)
+
+    def update_host(self, positions, r_cut):
+        """update() from numpy positions, with the species of the last build_host."""
+        C = self._C
+        pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
+        if len(pos) != self.num_atoms:
+            raise ValueError("the number of atoms differs from the last build")
+        E = C.c_long(0)
+        self._lib.check(self._L.smx_nlist_update_host(C.c_void_p(self._h), pos.ctypes.data_as(C.POINTER(C.c_double)),
+                                                      C.c_double(r_cut), C.byref(E)))
         return self._refresh(E.value)
 
     def update(self, positions_ptr, types_ptr, r_cut, stream=0):

@@ -321,6 +321,10 @@ def test_calculator_energy_forces_stress(gpu, tmp_models):
     orc.compute_node_energies_forces(*H.call_args(ea))
     assert res["energy"] == pytest.approx(orc.node_energies.sum(), rel=1e-10)
     assert np.allclose(res["forces"], H.atom_forces(nl, orc.node_forces, len(pos)), atol=1e-8)
+    # the list built on the device (default) and the numpy builder give the same bits
+    res_h = SymmetrixCalculator(path, neighbor_list="host").compute(pos, cell, Z)
+    assert res_h["energy"] == res["energy"] and np.array_equal(res_h["energies"], res["energies"])
+    assert np.array_equal(res_h["forces"], res["forces"]) and np.array_equal(res_h["stress"], res["stress"])
     F, e0 = res["forces"].copy(), res["energy"]
     h = 1e-5
     for a, c in ((0, 0), (3, 1), (7, 2)):
@@ -398,6 +402,14 @@ def test_device_neighbor_list_update_equals_fresh_build():
             assert np.array_equal(got[k], ref[k].reshape(got[k].shape)), k
     with pytest.raises(ValueError):
         dnl.update(dpos.data_ptr(), dty.data_ptr(), rc + 2 * skin)
+    # the same through host arrays
+    hnl = neighbors.DeviceNeighborList()
+    hnl.build_host(pos, types, cell, rc, skin=skin)
+    pos2 = pos + rng.uniform(-0.1, 0.1, size=pos.shape)
+    E = hnl.update_host(pos2, rc)
+    got, ref = hnl.to_host(), neighbors.neighbor_list(pos2, cell, rc)
+    assert E == len(ref["r"]) and np.array_equal(got["j"], ref["j"]) and np.array_equal(got["r"], ref["r"])
+    assert np.array_equal(got["neigh_types"], types[ref["j"]])
 
 
 @pytest.mark.gpu

@@ -278,7 +278,7 @@ def test_invalid_inputs_raise(gpu, tmp_models):
     eng.compute_node_energies_forces(*ok)   # still usable afterwards
 
 
-@pytest.mark.parametrize("workload", ["off_small"])
+@pytest.mark.parametrize("workload", ["off_small", "mp_medium"])
 def test_full_size_properties(gpu, tmp_models, workload):
     """At the benchmark's full size: properties that do not need the oracle."""
     from symmetrix_amd import modelgen, neighbors, systems
@@ -518,3 +518,32 @@ def test_pair_style_modes_agree(gpu, tmp_models, L_max, dtype):
     assert np.abs(eng2.node_energies - e_ref).max() <= etol * max(1.0, np.abs(e_ref).max())
     f_m = eng2.reduce_forces(N, ga["sender_atom"][:El])
     assert np.abs(f_m - f_ref).max() <= ftol * 10 * max(1.0, np.abs(f_ref).max())
+
+
+@pytest.mark.gpu
+def test_rotation_and_replication_through_the_calculator(tmp_models):
+    """A rigid rotation of positions and cell leaves the energy alone and rotates the forces; a cell repeated along
+    an axis repeats energies and forces.  Both go through the device neighbour list with general triclinic cells."""
+    from symmetrix_amd.calc import SymmetrixCalculator
+    model = H.tiny_model(K=16, L_max=1, n_pts=64, seed=31, zbl=True, density=True)
+    path = H.write_model(model, tmp_models / "rot.json")
+    calc = SymmetrixCalculator(path)
+    pos, cell, sp = H.small_system(24, density=0.08, seed=13)
+    Z = np.array(model["atomic_numbers"])[sp]
+    cell = np.diag(cell)
+    res = calc.compute(pos, cell, Z)
+    e0, f0, en0 = res["energy"], res["forces"].copy(), res["energies"].copy()
+    rng = np.random.default_rng(5)
+    Q, _ = np.linalg.qr(rng.normal(size=(3, 3)))
+    if np.linalg.det(Q) < 0:
+        Q[:, 0] = -Q[:, 0]
+    rot = calc.compute(pos @ Q.T, cell @ Q.T, Z)
+    assert abs(rot["energy"] - e0) <= 1e-10 * abs(e0)
+    assert np.abs(rot["forces"] - f0 @ Q.T).max() <= 1e-8 * max(1.0, np.abs(f0).max())
+    pos2 = np.concatenate([pos, pos + cell[0]])
+    cell2 = cell.copy(); cell2[0] *= 2
+    rep = calc.compute(pos2, cell2, np.concatenate([Z, Z]))
+    assert np.abs(rep["energies"][:len(pos)] - en0).max() <= 1e-10 * max(1.0, np.abs(en0).max())
+    assert np.abs(rep["energies"][len(pos):] - en0).max() <= 1e-10 * max(1.0, np.abs(en0).max())
+    assert np.abs(rep["forces"][:len(pos)] - f0).max() <= 1e-8 * max(1.0, np.abs(f0).max())
+    assert np.abs(rep["stress"] - res["stress"]).max() <= 1e-9 * max(1.0, np.abs(res["stress"]).max())

@@ -69,7 +69,7 @@ struct DVec {
             // nothing to carry over: release first, so that the two sizes never coexist
             HIPCHK(hipStreamSynchronize(s));
             HIPCHK(hipFree(p));
-            p = nullptr; cap = 0;
+            p = nullptr; cap = 0; n = 0;
         }
         HIPCHK(hipMalloc(&q, newcap * sizeof(T)));
         if (p) {

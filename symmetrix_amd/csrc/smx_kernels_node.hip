@@ -591,7 +591,12 @@ hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* n
     if (rows < N) return hipErrorInvalidValue;
     if (rows <= 0) return hipSuccess;
     const size_t lds = ((size_t)16 * (K + 1) + 256 + (size_t)16 * K) * sizeof(double);
-    if (lds > 64 * 1024) return hipErrorInvalidValue;
+    if (lds > 160 * 1024) return hipErrorInvalidValue;    // K beyond about 630 channels
+    if (lds > 64 * 1024) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_readout_fused<F>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+    }
     hipLaunchKernelGGL(k_readout_fused<F>, dim3((rows + 15) / 16), dim3(256), lds, s, N, rows, K, num_LM, node_types,
                        atomic_energies, w1, W1, w2, scale, H1, H2, H2_adj, H1_adj, node_energies, zero_energies,
                        energies_copy);

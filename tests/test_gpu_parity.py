@@ -52,6 +52,8 @@ CASES = [
     # K, L_max, atoms, pair-dependent radial
     (32, 0, 40, True), (32, 1, 40, True), (96, 0, 48, False), (128, 1, 36, True), (48, 1, 24, True),
     (20, 0, 17, True), (64, 1, 30, False), (128, 0, 30, True),
+    # wider than one block of channels: several channel groups, column tiles and slices
+    (256, 0, 20, False), (192, 1, 16, False),
 ]
 
 

@@ -245,8 +245,8 @@ struct Engine : EngineBase {
             size_t o = 0;
             for (auto& t : tables)
                 for (int n = 0; n < R; ++n)
-                    for (int k = 0; k < Kc; ++k)
-                        for (int pth = 0; pth < Pn; ++pth)
+                    for (int pth = 0; pth < Pn; ++pth)
+                        for (int k = 0; k < Kc; ++k)
                             for (int q = 0; q < 4; ++q) out[o++] = t[((size_t)n * 4 + q) * nspl + pth * Kc + k];
             upload_as(dst, out, s);
         };

@@ -178,7 +178,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
             const F x = (F)xs[le];
             const int row = __builtin_amdgcn_readfirstlane(rows[le]);
             const int grow = __builtin_amdgcn_readfirstlane(grows[le]);
-            const F* rowp = a.tabK + ((size_t)row * K + k0) * (4 * P);
+            const F* rowp = a.tabK + ((size_t)row * P * K + k0) * 4;
             const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
             const F* B = Bs + le * NBP;
             Vec<F, CPL> H[NLM];
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
                 constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1;
                 Vec<F, 4> cf[CPL];
 #pragma unroll
-                for (int c = 0; c < CPL; ++c) cf[c] = ldv<F, 4>(rowp + (c * P + p) * 4);
+                for (int c = 0; c < CPL; ++c) cf[c] = ldv<F, 4>(rowp + ((size_t)p * K + c) * 4);
                 F Bv[(2 * l + 1) * n2];
 #pragma unroll
                 for (int q = 0; q < (2 * l + 1) * n2; ++q) Bv[q] = B[bo + q];
@@ -308,11 +308,11 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
         Vec<F, 4> cf[P][CPL];
         auto load_cf = [&](int le_) {
             const int row = __builtin_amdgcn_readfirstlane(rows[le_]);
-            const F* rowp = a.tabK + ((size_t)row * K + k0) * (4 * P);
+            const F* rowp = a.tabK + ((size_t)row * P * K + k0) * 4;
 #pragma unroll
             for (int q = 0; q < P; ++q)
 #pragma unroll
-                for (int c = 0; c < CPL; ++c) cf[q][c] = ldv<F, 4>(rowp + (c * P + q) * 4);
+                for (int c = 0; c < CPL; ++c) cf[q][c] = ldv<F, 4>(rowp + ((size_t)q * K + c) * 4);
         };
         if (AHEAD && active && nE > 0) load_cf(0);
         for (int le = 0; le < nE; ++le) {

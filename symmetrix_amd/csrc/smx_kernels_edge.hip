@@ -174,37 +174,55 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
         }
         wave_lds_sync();
         if (!active) continue;
-        for (int le = 0; le < nE; ++le) {
-            const F x = (F)xs[le];
-            const int row = __builtin_amdgcn_readfirstlane(rows[le]);
-            const int grow = __builtin_amdgcn_readfirstlane(grows[le]);
+        // Spline coefficients (P x CPL 16-byte loads, contiguous across the lanes for one path) and the sender
+        // row of an edge.  In single precision those of the next edge are requested while the current edge is
+        // worked on; in double precision there are no registers for that.
+        constexpr bool AHEAD = sizeof(F) == 4 && (CPL == 1 || LMAXH == 0);
+        Vec<F, 4> cf[P][CPL];
+        Vec<F, CPL> H[NLM];
+        auto request = [&](int le_) {
+            const int row = __builtin_amdgcn_readfirstlane(rows[le_]);
+            const int grow = __builtin_amdgcn_readfirstlane(grows[le_]);
             const F* rowp = a.tabK + ((size_t)row * P * K + k0) * 4;
             const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
-            const F* B = Bs + le * NBP;
-            Vec<F, CPL> H[NLM];
 #pragma unroll
             for (int q = 0; q < NLM; ++q) H[q] = ldv<F, CPL>(Hp + q * K);
+#pragma unroll
+            for (int q = 0; q < P; ++q)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) cf[q][c] = ldv<F, 4>(rowp + ((size_t)q * K + c) * 4);
+        };
+        if (AHEAD && nE > 0) request(0);
+        for (int le = 0; le < nE; ++le) {
+            const F x = (F)xs[le];
+            const F* B = Bs + le * NBP;
+            if (!AHEAD) request(le);
+            // radial value times sender feature for every path and sender component
+            F w[P][CPL][2 * LMAXH + 1];
+#pragma unroll
+            for (int q = 0; q < P; ++q)
+#pragma unroll
+                for (int c = 0; c < CPL; ++c) {
+                    const Vec<F, 4> k4 = cf[q][c];
+                    const F R = k4.v[0] + x * (k4.v[1] + x * (k4.v[2] + x * k4.v[3]));
+#pragma unroll
+                    for (int m2 = 0; m2 < 2 * PT::l2(q) + 1; ++m2) w[q][c][m2] = R * H[PT::l2(q) * PT::l2(q) + m2].v[c];
+                }
+            if (AHEAD && le + 1 < nE) request(le + 1);
             static_for<0, P>([&](auto pc) {
                 constexpr int p = decltype(pc)::value;
                 constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
                 constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1;
-                Vec<F, 4> cf[CPL];
-#pragma unroll
-                for (int c = 0; c < CPL; ++c) cf[c] = ldv<F, 4>(rowp + ((size_t)p * K + c) * 4);
                 F Bv[(2 * l + 1) * n2];
 #pragma unroll
                 for (int q = 0; q < (2 * l + 1) * n2; ++q) Bv[q] = B[bo + q];
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) {
-                    const F R = cf[c].v[0] + x * (cf[c].v[1] + x * (cf[c].v[2] + x * cf[c].v[3]));
-                    F w[n2];
-#pragma unroll
-                    for (int m2 = 0; m2 < n2; ++m2) w[m2] = R * H[l2 * l2 + m2].v[c];
 #pragma unroll
                     for (int m = 0; m < 2 * l + 1; ++m) {
                         F z = acc[c][lme0 + m * es];
 #pragma unroll
-                        for (int m2 = 0; m2 < n2; ++m2) z += Bv[m * n2 + m2] * w[m2];
+                        for (int m2 = 0; m2 < n2; ++m2) z += Bv[m * n2 + m2] * w[p][c][m2];
                         acc[c][lme0 + m * es] = z;
                     }
                 }
@@ -455,7 +473,7 @@ hipError_t launch_agg_t(const AggParams<F>& p, hipStream_t s)
 template <typename F, int LMAXH, bool BWD>
 int agg_cpl(int K)
 {
-    const bool wide = LMAXH == 0 || (!BWD && sizeof(F) == 4);
+    const bool wide = LMAXH == 0;
     return (wide && K > 64 && K % 2 == 0) ? 2 : 1;
 }
 

@@ -238,8 +238,10 @@ struct Engine : EngineBase {
             upload_as(A1w, all, s);
         }
         build_slices(s);
-        // the general edge kernels read the tables channel-major; layers served by the slice kernels need no copy
-        auto kmajor = [&](const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst) {
+        // the general edge kernels read the tables as [interval][path][channel][4 coefficients]: one load instruction
+        // of a wavefront (one path, consecutive channels) then covers contiguous memory; layers served by the slice
+        // kernels need no copy
+        auto regroup = [&](const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst) {
             const int R = hm.spl_nodes - 1, Kc = hm.K, Pn = nspl / Kc;
             std::vector<double> out((size_t)tables.size() * R * nspl * 4);
             size_t o = 0;
@@ -250,8 +252,8 @@ struct Engine : EngineBase {
                             for (int q = 0; q < 4; ++q) out[o++] = t[((size_t)n * 4 + q) * nspl + pth * Kc + k];
             upload_as(dst, out, s);
         };
-        if (!slice_CH0) kmajor(hm.tables0, hm.nspl0, tabK0);
-        if (!slice_CH1) kmajor(hm.tables1, hm.nspl1, tabK1);
+        if (!slice_CH0) regroup(hm.tables0, hm.nspl0, tabK0);
+        if (!slice_CH1) regroup(hm.tables1, hm.nspl1, tabK1);
         // layer 0 couples Y_lm straight into output slot lm
         {
             std::vector<int> st(17), lm(16);

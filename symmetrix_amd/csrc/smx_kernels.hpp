@@ -28,7 +28,7 @@ struct AggParams {
     const double* r;          // [E]
     const F* Hsrc;            // [rows][NLM][K]
     const F* tab;             // [table][nodes-1][4][P*K]
-    const F* tabK;            // the same numbers channel-major, [table][nodes-1][K][P][4] (general edge kernels)
+    const F* tabK;            // the same numbers with the coefficients of a spline adjacent, [table][nodes-1][P][K][4] (general edge kernels)
     const int* pair_table;    // [T(T+1)/2] -> table
     int T;
     int spl_nodes;

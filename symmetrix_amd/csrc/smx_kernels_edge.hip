@@ -319,7 +319,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
             *reinterpret_cast<Vec<F, 4>*>(Bs + ((size_t)le * NBP + b) * 4) = o;
         }
         wave_lds_sync();
-        // Spline coefficients of one edge: P x CPL 16-byte loads from the channel-major table.  In single
+        // Spline coefficients of one edge: P x CPL 16-byte loads, contiguous across the lanes for one path.  In single
         // precision the next edge's coefficients are requested while the current edge is worked on (40
         // registers in flight); in double precision they are requested together at the start of the edge.
         constexpr bool AHEAD = sizeof(F) == 4;

@@ -45,10 +45,10 @@ MEASURED_TRAFFIC = {
                                "sender_reduce": 93.6e6},
     ("off_small", "float32"): {"agg0_fwd": 58.8e6, "agg1_fwd": 86.2e6, "agg1_bwd": 247.3e6, "agg0_bwd": 151.8e6,
                                "sender_reduce": 47.7e6},
-    ("mp_medium", "float32"): {"agg0_fwd": 1700.6e6, "agg1_fwd": 9676.8e6, "agg1_bwd": 16227.3e6, "agg0_bwd": 4480.1e6,
-                               "sender_reduce": 8257.2e6},
-    ("mp_medium", "float64"): {"agg0_fwd": 2099.7e6, "agg1_fwd": 20267.6e6, "agg1_bwd": 46609.2e6, "agg0_bwd": 7626.2e6,
-                               "sender_reduce": 16442.4e6},
+    ("mp_medium", "float32"): {"agg0_fwd": 1693.3e6, "agg1_fwd": 5003.7e6, "agg1_bwd": 16249.3e6, "agg0_bwd": 4474.9e6,
+                               "sender_reduce": 8256.9e6},
+    ("mp_medium", "float64"): {"agg0_fwd": 2096.3e6, "agg1_fwd": 19989.5e6, "agg1_bwd": 45951.0e6, "agg0_bwd": 7629.8e6,
+                               "sender_reduce": 16442.7e6},
 }
 
 

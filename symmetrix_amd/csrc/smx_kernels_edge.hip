@@ -208,7 +208,9 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
 #pragma unroll
                     for (int m2 = 0; m2 < 2 * PT::l2(q) + 1; ++m2) w[q][c][m2] = R * H[PT::l2(q) * PT::l2(q) + m2].v[c];
                 }
-            if (AHEAD && le + 1 < nE) request(le + 1);
+            // unconditional (the last edge of a chunk asks for its own operands again): a conditional request makes the
+            // values carried round the loop a merge of old and new registers, which costs a register copy per value
+            if (AHEAD) request(le + 1 < nE ? le + 1 : le);
             static_for<0, P>([&](auto pc) {
                 constexpr int p = decltype(pc)::value;
                 constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);

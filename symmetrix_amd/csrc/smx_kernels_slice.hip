@@ -124,7 +124,7 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
             }
             for (int e = e0 + e_sub; e < e1; e += EPR) {
                 const EdgeGeo cu = nx;
-                if (e + EPR < e1) nx = load_edge(a, e + EPR);
+                nx = load_edge(a, min(e + EPR, e1 - 1));   // unconditional: a conditional load costs a register copy per value
                 const int tj = cu.tj;
                 if (p.U > 1 && a.pair_table[pair_index(a.T, ti, tj)] != u) continue;
                 const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
@@ -227,7 +227,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
                 const int e = e0 + it * EPR + e_sub;
                 bool on = e < e1;
                 const EdgeGeo cu = nx;
-                if (e + EPR < e1) nx = load_edge(a, e + EPR);
+                nx = load_edge(a, min(e + EPR, e1 - 1));   // unconditional: a conditional load costs a register copy per value
                 if (on && p.U > 1 && a.pair_table[pair_index(a.T, ti, cu.tj)] != u) on = false;
                 double fx = 0.0, fy = 0.0, fz = 0.0;
                 if (on) {
@@ -351,7 +351,8 @@ hipError_t launch_slice_cfg(const SliceParams<F>& p, hipStream_t s)
 template <typename F, int CH, bool BWD>
 hipError_t launch_slice_t(const SliceParams<F>& p, hipStream_t s)
 {
-    if constexpr (CH % 4 == 0) return launch_slice_cfg<F, CH, 4, 768, BWD>(p, s);
+    if constexpr (CH % 4 == 0 && !BWD && sizeof(F) == 8 && CH == 4) return launch_slice_cfg<F, CH, 4, 1024, BWD>(p, s);
+    else if constexpr (CH % 4 == 0) return launch_slice_cfg<F, CH, 4, 768, BWD>(p, s);
     else return launch_slice_cfg<F, CH, 2, 512, BWD>(p, s);
 }
 

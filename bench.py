@@ -41,14 +41,14 @@ STAGE_KERNEL = {
 # 1 GiB copy in the same runs), full-size workloads only: profiles/edge_kernels_off_small_hbm_traffic.txt and
 # profiles/edge_kernels_mp_medium_hbm_traffic.txt
 MEASURED_TRAFFIC = {
-    ("off_small", "float64"): {"agg0_fwd": 78.9e6, "agg1_fwd": 106.0e6, "agg1_bwd": 436.8e6, "agg0_bwd": 257.9e6,
+    ("off_small", "float64"): {"agg0_fwd": 78.8e6, "agg1_fwd": 106.2e6, "agg1_bwd": 436.0e6, "agg0_bwd": 257.9e6,
                                "sender_reduce": 93.6e6},
     ("off_small", "float32"): {"agg0_fwd": 58.8e6, "agg1_fwd": 86.2e6, "agg1_bwd": 247.3e6, "agg0_bwd": 151.8e6,
                                "sender_reduce": 47.7e6},
-    ("mp_medium", "float32"): {"agg0_fwd": 1693.3e6, "agg1_fwd": 5003.7e6, "agg1_bwd": 16249.3e6, "agg0_bwd": 4474.9e6,
-                               "sender_reduce": 8256.9e6},
-    ("mp_medium", "float64"): {"agg0_fwd": 2096.3e6, "agg1_fwd": 19989.5e6, "agg1_bwd": 45951.0e6, "agg0_bwd": 7629.8e6,
-                               "sender_reduce": 16442.7e6},
+    ("mp_medium", "float32"): {"agg0_fwd": 1736.3e6, "agg1_fwd": 4687.3e6, "agg1_bwd": 16246.2e6, "agg0_bwd": 4489.3e6,
+                               "sender_reduce": 8257.1e6},
+    ("mp_medium", "float64"): {"agg0_fwd": 2300.1e6, "agg1_fwd": 19990.4e6, "agg1_bwd": 45947.7e6, "agg0_bwd": 7632.3e6,
+                               "sender_reduce": 16442.6e6},
 }
 
 

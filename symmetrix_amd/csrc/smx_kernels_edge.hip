@@ -39,13 +39,19 @@ struct WaveLds {
     }
 };
 
-// The steps in which the adjoint kernel walks the coupling block B[path][m][m2] of an edge: all rows m of a path
-// with a scalar sender feature, three rows at a time of a path with a vector one (at most nine entries).
-template <int LMAXH>
+// The steps in which the adjoint kernel walks the coupling block B[path][m][m2] of an edge.  Wide steps (single
+// precision): all rows m of a path with a scalar sender feature, three rows at a time of a path with a vector one
+// (at most nine entries).  Narrow steps (double precision, where an entry takes eight registers): at most three
+// entries, i.e. three rows of a scalar path or one row of a vector path.
+template <int LMAXH, bool NARROW>
 struct BwdSteps {
     using PT = Paths<LMAXH>;
     static constexpr int rows(int p) { return 2 * PT::l(p) + 1; }
-    static constexpr int group(int p) { return PT::l2(p) == 0 ? rows(p) : 3; }
+    static constexpr int group(int p)
+    {
+        if (NARROW) return PT::l2(p) == 0 ? (rows(p) < 3 ? rows(p) : 3) : 1;
+        return PT::l2(p) == 0 ? rows(p) : 3;
+    }
     static constexpr int groups(int p) { return (rows(p) + group(p) - 1) / group(p); }
     static constexpr int count()
     {
@@ -365,11 +371,11 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                 if (AHEAD && le + 1 < nE) load_cf(le + 1);
                 // The B block of the edge is walked in steps (a few rows m of one path each).  Per path, the rows
                 // are summed first, u[m2][comp] = sum_m d[m] * (B, dB/dx, dB/dy, dB/dz)[m][m2], then one product
-                // with the sender feature per m2.  In single precision the LDS reads of the next step are issued
-                // before the arithmetic of the current one (two register buffers); the fence after each step keeps
+                // with the sender feature per m2.  The LDS reads of the next step are issued before the
+                // arithmetic of the current one (two register buffers); the fence after each step keeps
                 // reads further ahead from being issued (all at once would need several hundred registers).
-                using ST = BwdSteps<LMAXH>;
-                constexpr bool LOOKAHEAD = sizeof(F) == 4;
+                using ST = BwdSteps<LMAXH, sizeof(F) == 8>;
+                constexpr bool LOOKAHEAD = true;
                 Vec<F, 4> buf[LOOKAHEAD ? 2 : 1][ST::MAXLEN];
                 F u[CPL][2 * LMAXH + 1][4];
                 auto load_step = [&](auto sc, Vec<F, 4>* dst) {

@@ -266,6 +266,8 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
     int* cg_lm1 = reinterpret_cast<int*>(cg_c + num_terms);
     int* cg_start = cg_lm1 + num_terms;
     unsigned char* base = smem + WL::lists(num_terms) + (size_t)wave * WL::per_wave(EC);
+    // the B block below is read with 4 * sizeof(F)-byte accesses: the doubles in front of it must keep that alignment
+    static_assert((EC * (64 + 4 + 1) * sizeof(double)) % (4 * sizeof(F)) == 0, "chunk size breaks the alignment of the B block");
     double* Yt = reinterpret_cast<double*>(base);                                 // [EC][4][16]: Y, dY/dx, dY/dy, dY/dz
     double* us = Yt + EC * 64;                                                    // [EC][4] unit vector xyz/r
     double* xs = us + EC * 4;                                                     // [EC]

@@ -182,31 +182,36 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
         if (!active) continue;
         // Spline coefficients (P x CPL 16-byte loads, contiguous across the lanes for one path) and the sender
         // row of an edge.  In single precision those of the next edge are requested while the current edge is
-        // worked on; in double precision there are no registers for that.
+        // worked on (AHEAD).  In double precision there are registers for half of that at most (HALF: the first
+        // five paths and the sender row requested an edge ahead, the other five at the start of the edge).
         constexpr bool AHEAD = sizeof(F) == 4 && (CPL == 1 || LMAXH == 0);
+        constexpr bool HALF = false;   // measured slower than requesting all ten at the start of the edge (10.4 against 9.1 ms)
+        constexpr int PA = HALF ? P / 2 : P;     // paths of the first part
         Vec<F, 4> cf[P][CPL];
         Vec<F, CPL> H[NLM];
-        auto request = [&](int le_) {
+        auto request = [&](int le_, auto first, auto last, bool sender) {
+            constexpr int p0 = decltype(first)::value, p1 = decltype(last)::value;
             const int row = __builtin_amdgcn_readfirstlane(rows[le_]);
-            const int grow = __builtin_amdgcn_readfirstlane(grows[le_]);
             const F* rowp = a.tabK + ((size_t)row * P * K + k0) * 4;
-            const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
+            if (sender) {
+                const int grow = __builtin_amdgcn_readfirstlane(grows[le_]);
+                const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
 #pragma unroll
-            for (int q = 0; q < NLM; ++q) H[q] = ldv<F, CPL>(Hp + q * K);
+                for (int q = 0; q < NLM; ++q) H[q] = ldv<F, CPL>(Hp + q * K);
+            }
 #pragma unroll
-            for (int q = 0; q < P; ++q)
+            for (int q = p0; q < p1; ++q)
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) cf[q][c] = ldv<F, 4>(rowp + ((size_t)q * K + c) * 4);
         };
-        if (AHEAD && nE > 0) request(0);
-        for (int le = 0; le < nE; ++le) {
-            const F x = (F)xs[le];
-            const F* B = Bs + le * NBP;
-            if (!AHEAD) request(le);
-            // radial value times sender feature for every path and sender component
-            F w[P][CPL][2 * LMAXH + 1];
+        constexpr std::integral_constant<int, 0> c0{};
+        constexpr std::integral_constant<int, PA> cA{};
+        constexpr std::integral_constant<int, P> cP{};
+        if ((AHEAD || HALF) && nE > 0) request(0, c0, cA, true);
+        F w[P][CPL][2 * LMAXH + 1];   // radial value times sender feature per path and sender component
+        auto products = [&](F x, auto first, auto last) {
 #pragma unroll
-            for (int q = 0; q < P; ++q)
+            for (int q = decltype(first)::value; q < decltype(last)::value; ++q)
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) {
                     const Vec<F, 4> k4 = cf[q][c];
@@ -214,10 +219,11 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
 #pragma unroll
                     for (int m2 = 0; m2 < 2 * PT::l2(q) + 1; ++m2) w[q][c][m2] = R * H[PT::l2(q) * PT::l2(q) + m2].v[c];
                 }
-            // unconditional (the last edge of a chunk asks for its own operands again): a conditional request makes the
-            // values carried round the loop a merge of old and new registers, which costs a register copy per value
-            if (AHEAD) request(le + 1 < nE ? le + 1 : le);
-            static_for<0, P>([&](auto pc) {
+        };
+        for (int le = 0; le < nE; ++le) {
+            const F x = (F)xs[le];
+            const F* B = Bs + le * NBP;
+            auto accumulate = [&](auto pc) {
                 constexpr int p = decltype(pc)::value;
                 constexpr int l = PT::l(p), l2 = PT::l2(p), bo = PT::boff(p);
                 constexpr int lme0 = PT::lme(p, 0), es = PT::num_e(l), n2 = 2 * l2 + 1;
@@ -234,7 +240,21 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
                         acc[c][lme0 + m * es] = z;
                     }
                 }
-            });
+            };
+            // requests for a following edge are unconditional (the last edge of a chunk asks for its own operands
+            // again): a conditional request makes the values carried round the loop a merge of old and new registers,
+            // which costs a register copy per value
+            const int le_next = le + 1 < nE ? le + 1 : le;
+            if (!AHEAD && !HALF) request(le, c0, cP, true);
+            if (HALF) request(le, cA, cP, false);
+            products(x, c0, cA);
+            if (AHEAD) request(le_next, c0, cP, true);
+            static_for<0, PA>(accumulate);
+            if constexpr (HALF) {
+                products(x, cA, cP);
+                request(le_next, c0, cA, true);
+                static_for<PA, P>(accumulate);
+            }
         }
     }
     if (active) {

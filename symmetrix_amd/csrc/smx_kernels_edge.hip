@@ -302,8 +302,10 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
     const int K = a.K;
     const int i = a.node_begin + blockIdx.x * 4 + wave;
     if (i >= a.num_nodes) return;
-    const int k0 = (blockIdx.y * 64 + lane) * CPL;
-    const bool active = k0 < K;
+    // Lanes beyond the last channel work on channel 0 with a zero adjoint (all their sums are zero) and skip the
+    // message store: no branch on the lane's channel inside the edge loop, hence no merges of old and new registers.
+    const bool active = (blockIdx.y * 64 + lane) * CPL < K;
+    const int k0 = active ? (blockIdx.y * 64 + lane) * CPL : 0;
     const int e0 = a.first_neigh[i], e1 = a.first_neigh[i + 1], ti = a.node_types[i];
     double* fout = gridDim.y > 1 ? a.fpart + (size_t)blockIdx.y * 3 * a.num_edges : a.forces;
     const bool add_forces = gridDim.y == 1 && a.accumulate_forces;
@@ -311,8 +313,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
     F d[CPL][NE];
 #pragma unroll
     for (int q = 0; q < NE; ++q) {
-        // lanes beyond K read channel 0 and discard it
-        const Vec<F, CPL> v = ldv<F, CPL>(a.d_out + ((size_t)i * NE + q) * K + (active ? k0 : 0));
+        const Vec<F, CPL> v = ldv<F, CPL>(a.d_out + ((size_t)i * NE + q) * K + k0);
 #pragma unroll
         for (int c = 0; c < CPL; ++c) d[c][q] = active ? v.v[c] : F(0);
     }
@@ -362,10 +363,13 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) cf[q][c] = ldv<F, 4>(rowp + ((size_t)q * K + c) * 4);
         };
-        if (AHEAD && active && nE > 0) load_cf(0);
-        for (int le = 0; le < nE; ++le) {
+        if (AHEAD && nE > 0) load_cf(0);
+        // One edge.  The loop below runs it with the request for the next edge's coefficients for all edges but the
+        // last of the chunk, which runs without: a request under a condition inside one loop body would make the
+        // coefficients carried round the loop a merge of old and new registers (a register copy per value and edge).
+        auto edge = [&](const int le, auto ahead) {
             F srad = F(0), gx = F(0), gy = F(0), gz = F(0);
-            if (active) {
+            {
                 const F x = (F)xs[le];
                 const int grow = __builtin_amdgcn_readfirstlane(grows[le]);
                 // element offset of this edge's B block; it passes through the fences below, which keep the
@@ -390,7 +394,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                         Rv[q][c] = k4.v[0] + x * (k4.v[1] + x * (k4.v[2] + x * k4.v[3]));
                         Rdv[q][c] = k4.v[1] + x * (F(2) * k4.v[2] + F(3) * x * k4.v[3]);
                     }
-                if (AHEAD && le + 1 < nE) load_cf(le + 1);
+                if constexpr (AHEAD && decltype(ahead)::value) load_cf(le + 1);
                 // The B block of the edge is walked in steps (a few rows m of one path each).  Per path, the rows
                 // are summed first, u[m2][comp] = sum_m d[m] * (B, dB/dx, dB/dy, dB/dz)[m][m2], then one product
                 // with the sender feature per m2.  The LDS reads of the next step are issued before the
@@ -455,7 +459,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                             for (int c = 0; c < CPL; ++c) pin(mg[l2 * l2 + m2].v[c]);
                     }
                 });
-                if (a.msg) {
+                if (a.msg && active) {
                     F* mrow = a.msg + (size_t)(eb + le - a.msg_edge_begin) * NLM * K + k0;
 #pragma unroll
                     for (int q = 0; q < NLM; ++q) *reinterpret_cast<Vec<F, CPL>*>(mrow + q * K) = mg[q];
@@ -470,7 +474,9 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                 if (add_forces) { f[0] += fx; f[1] += fy; f[2] += fz; }
                 else { f[0] = fx; f[1] = fy; f[2] = fz; }
             }
-        }
+        };
+        for (int le = 0; le + 1 < nE; ++le) edge(le, std::true_type{});
+        if (nE > 0) edge(nE - 1, std::false_type{});
     }
 }
 

@@ -181,6 +181,15 @@ __device__ __forceinline__ double read_lane(double v, int lane)
     const int hi = __builtin_amdgcn_readlane((int)(b >> 32), lane);
     return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
+__device__ __forceinline__ float read_lane(float v, int lane)
+{
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), lane));
+}
+__device__ __forceinline__ float wave_sum(float v)
+{
+    v = row_sum_strided<1>(v);
+    return (read_lane(v, 0) + read_lane(v, 16)) + (read_lane(v, 32) + read_lane(v, 48));
+}
 // sum over the 64 lanes of the wavefront, the same value (and the same order of additions) in every lane
 __device__ __forceinline__ double wave_sum(double v)
 {

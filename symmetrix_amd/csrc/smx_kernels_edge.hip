@@ -465,10 +465,22 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                     for (int q = 0; q < NLM; ++q) *reinterpret_cast<Vec<F, CPL>*>(mrow + q * K) = mg[q];
                 }
             }
-            const double sr = (double)srad;
-            const double fx = wave_sum(-(us[le * 4] * sr + (double)gx));
-            const double fy = wave_sum(-(us[le * 4 + 1] * sr + (double)gy));
-            const double fz = wave_sum(-(us[le * 4 + 2] * sr + (double)gz));
+            // Sums over the channels of the wavefront (a fixed tree: bit-reproducible).  Double precision: the three
+            // force components are put together per lane and summed.  Single-precision features: the four partial
+            // sums are added across the lanes in single precision (a third of the instructions) and put together in
+            // double afterwards.
+            double fx, fy, fz;
+            if constexpr (sizeof(F) == 8) {
+                const double sr = (double)srad;
+                fx = wave_sum(-(us[le * 4] * sr + (double)gx));
+                fy = wave_sum(-(us[le * 4 + 1] * sr + (double)gy));
+                fz = wave_sum(-(us[le * 4 + 2] * sr + (double)gz));
+            } else {
+                const double sr = (double)wave_sum(srad);
+                fx = -(us[le * 4] * sr + (double)wave_sum(gx));
+                fy = -(us[le * 4 + 1] * sr + (double)wave_sum(gy));
+                fz = -(us[le * 4 + 2] * sr + (double)wave_sum(gz));
+            }
             if (lane == 0) {
                 double* f = fout + 3 * (size_t)(eb + le);
                 if (add_forces) { f[0] += fx; f[1] += fy; f[2] += fz; }

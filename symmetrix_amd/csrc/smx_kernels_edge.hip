@@ -117,6 +117,26 @@ __device__ __forceinline__ Vec<F, CPL> ldv(const F* p)
     return *reinterpret_cast<const Vec<F, CPL>*>(p);
 }
 
+// Entry b of the coupling block, B[b] = sum_t c_t Y[lm1_t], as one lane holds it for the whole kernel: lane L owns the
+// entries L and L + 64.  The first two terms sit in registers (most entries have one or two); further terms, if a
+// model file has them, are read from the lists in LDS.
+struct BlockEntry {
+    double c0, c1;
+    int l0, l1, t2, t_end;
+};
+__device__ __forceinline__ BlockEntry block_entry(int b, int NB, const int* cg_start, const double* cg_c, const int* cg_lm1)
+{
+    BlockEntry e{0.0, 0.0, 0, 0, 0, 0};
+    if (b < NB) {
+        const int s0 = cg_start[b], s1 = cg_start[b + 1];
+        if (s1 > s0) { e.c0 = cg_c[s0]; e.l0 = cg_lm1[s0]; e.l1 = e.l0; }
+        if (s1 > s0 + 1) { e.c1 = cg_c[s0 + 1]; e.l1 = cg_lm1[s0 + 1]; }
+        e.t2 = s0 + 2 < s1 ? s0 + 2 : s1;
+        e.t_end = s1;
+    }
+    return e;
+}
+
 // ---------------------------------------------------------------------------
 template <typename F, int LMAXH, int CPL, int EC>
 __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const int num_terms)
@@ -139,6 +159,15 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
     for (int t = threadIdx.x; t < num_terms; t += 256) { cg_c[t] = a.B_c[t]; cg_lm1[t] = a.B_lm1[t]; }
     for (int t = threadIdx.x; t <= NB; t += 256) cg_start[t] = a.B_start[t];
     __syncthreads();
+    // lane-owned entries of the coupling block: measured faster in double precision; in single precision their
+    // registers cost a wavefront per SIMD and the kernel runs 15 % slower
+    constexpr bool OWNED = sizeof(F) == 8;
+    constexpr int NSLOT = OWNED ? (NB + 63) / 64 : 1;
+    BlockEntry ent[NSLOT];
+    if constexpr (OWNED) {
+#pragma unroll
+        for (int j = 0; j < NSLOT; ++j) ent[j] = block_entry(lane + 64 * j, NB, cg_start, cg_c, cg_lm1);
+    }
 
     const int K = a.K;
     const int i = blockIdx.x * 4 + wave;
@@ -172,11 +201,27 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
             grows[lane] = a.gather[e];
         }
         wave_lds_sync();
-        for (int it = lane; it < nE * NB; it += 64) {
-            const int le = it / NB, b = it - le * NB;
-            double s = 0.0;
-            for (int t = cg_start[b]; t < cg_start[b + 1]; ++t) s += cg_c[t] * Yt[le * 16 + cg_lm1[t]];
-            Bs[le * NBP + b] = (F)s;
+        if constexpr (OWNED) {
+#pragma unroll
+            for (int j = 0; j < NSLOT; ++j) {
+                const int b = lane + 64 * j;
+                if (b < NB) {
+                    const BlockEntry& en = ent[j];
+                    for (int le = 0; le < nE; ++le) {
+                        const double* y = Yt + le * 16;
+                        double s = en.c0 * y[en.l0] + en.c1 * y[en.l1];
+                        for (int t = en.t2; t < en.t_end; ++t) s += cg_c[t] * y[cg_lm1[t]];
+                        Bs[le * NBP + b] = (F)s;
+                    }
+                }
+            }
+        } else {
+            for (int it = lane; it < nE * NB; it += 64) {
+                const int le = it / NB, b = it - le * NB;
+                double s = 0.0;
+                for (int t = cg_start[b]; t < cg_start[b + 1]; ++t) s += cg_c[t] * Yt[le * 16 + cg_lm1[t]];
+                Bs[le * NBP + b] = (F)s;
+            }
         }
         wave_lds_sync();
         if (!active) continue;
@@ -298,6 +343,14 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
     for (int t = threadIdx.x; t < num_terms; t += 256) { cg_c[t] = a.B_c[t]; cg_lm1[t] = a.B_lm1[t]; }
     for (int t = threadIdx.x; t <= NB; t += 256) cg_start[t] = a.B_start[t];
     __syncthreads();
+    // lane-owned entries of the coupling block (registers for them exist in single precision only)
+    constexpr bool OWNED = sizeof(F) == 4;
+    constexpr int NSLOT = OWNED ? (NB + 63) / 64 : 1;
+    BlockEntry ent[NSLOT];
+    if constexpr (OWNED) {
+#pragma unroll
+        for (int j = 0; j < NSLOT; ++j) ent[j] = block_entry(lane + 64 * j, NB, cg_start, cg_c, cg_lm1);
+    }
 
     const int K = a.K;
     const int i = a.node_begin + blockIdx.x * 4 + wave;
@@ -337,6 +390,29 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
             grows[lane] = a.gather[e];
         }
         wave_lds_sync();
+        if constexpr (OWNED) {
+#pragma unroll
+            for (int j = 0; j < NSLOT; ++j) {
+                const int b = lane + 64 * j;
+                if (b < NB) {
+                    const BlockEntry& en = ent[j];
+                    for (int le = 0; le < nE; ++le) {
+                        const double* y0 = Yt + le * 64 + en.l0;
+                        const double* y1 = Yt + le * 64 + en.l1;
+                        double s = en.c0 * y0[0] + en.c1 * y1[0], sx = en.c0 * y0[16] + en.c1 * y1[16];
+                        double sy = en.c0 * y0[32] + en.c1 * y1[32], sz = en.c0 * y0[48] + en.c1 * y1[48];
+                        for (int t = en.t2; t < en.t_end; ++t) {
+                            const double cc = cg_c[t];
+                            const double* y = Yt + le * 64 + cg_lm1[t];
+                            s += cc * y[0]; sx += cc * y[16]; sy += cc * y[32]; sz += cc * y[48];
+                        }
+                        Vec<F, 4> o;
+                        o.v[0] = (F)s; o.v[1] = (F)sx; o.v[2] = (F)sy; o.v[3] = (F)sz;
+                        *reinterpret_cast<Vec<F, 4>*>(Bs + ((size_t)le * NBP + b) * 4) = o;
+                    }
+                }
+            }
+        } else {
         for (int it = lane; it < nE * NB; it += 64) {
             const int le = it / NB, b = it - le * NB;
             double s = 0.0, sx = 0.0, sy = 0.0, sz = 0.0;
@@ -348,6 +424,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
             Vec<F, 4> o;
             o.v[0] = (F)s; o.v[1] = (F)sx; o.v[2] = (F)sy; o.v[3] = (F)sz;
             *reinterpret_cast<Vec<F, 4>*>(Bs + ((size_t)le * NBP + b) * 4) = o;
+        }
         }
         wave_lds_sync();
         // Spline coefficients of one edge: P x CPL 16-byte loads, contiguous across the lanes for one path.  In single

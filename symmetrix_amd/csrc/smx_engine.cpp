@@ -111,7 +111,13 @@ enum Stage { ST_PREP, ST_AGG0F, ST_A0LIN, ST_M0, ST_H1, ST_AGG1F, ST_A1, ST_M1, 
              ST_REVM1, ST_REVA1, ST_AGG1B, ST_SRED, ST_REVH1, ST_REVM0, ST_REVA0LIN, ST_AGG0B, ST_FSUM1, ST_FSUM0, ST_COUNT };
 
 struct EngineBase {
-    virtual ~EngineBase() = default;
+    virtual ~EngineBase()
+    {
+        for (int i = 0; i < ST_COUNT; ++i) {
+            if (ev0[i]) (void)hipEventDestroy(ev0[i]);
+            if (ev1[i]) (void)hipEventDestroy(ev1[i]);
+        }
+    }
     HostModel hm;
     int precision = 0;
     hipStream_t stream = nullptr;   // stream of the current call

@@ -45,10 +45,10 @@ MEASURED_TRAFFIC = {
                                "sender_reduce": 93.6e6},
     ("off_small", "float32"): {"agg0_fwd": 58.8e6, "agg1_fwd": 86.2e6, "agg1_bwd": 247.3e6, "agg0_bwd": 151.8e6,
                                "sender_reduce": 47.7e6},
-    ("mp_medium", "float32"): {"agg0_fwd": 1732.4e6, "agg1_fwd": 4609.2e6, "agg1_bwd": 16229.8e6, "agg0_bwd": 4489.3e6,
+    ("mp_medium", "float32"): {"agg0_fwd": 1733.4e6, "agg1_fwd": 4609.0e6, "agg1_bwd": 16226.3e6, "agg0_bwd": 4490.6e6,
                                "sender_reduce": 8257.2e6},
-    ("mp_medium", "float64"): {"agg0_fwd": 2301.7e6, "agg1_fwd": 20012.3e6, "agg1_bwd": 45823.9e6, "agg0_bwd": 7627.0e6,
-                               "sender_reduce": 16442.5e6},
+    ("mp_medium", "float64"): {"agg0_fwd": 2291.3e6, "agg1_fwd": 20204.2e6, "agg1_bwd": 45819.8e6, "agg0_bwd": 7626.9e6,
+                               "sender_reduce": 16442.6e6},
 }
 
 

@@ -187,7 +187,7 @@ struct Engine : EngineBase {
     long E = 0;
     long E1 = 0;   // leading edges whose receivers take part in layer 1 (all of them unless ghost nodes follow)
     int N_geo = 0;
-    DVec<int> first_neigh, recv_order, scan_tmp, s_count, s_start, s_cursor, s_list, t_count, t_start, t_cursor, t_perm, flags;
+    DVec<int> first_neigh, recv_order, scan_tmp, s_count, s_start, s_list, t_count, t_start, t_cursor, t_perm, flags;
     int sender_rows = 0;
     // pair terms: ZBL constants per species pair, density-normalisation splines, divisors of the last forward pass
     DVec<double> zbl_a, zbl_rmax, zbl_zz, A0spl, A1spl, div0, div1;
@@ -215,7 +215,7 @@ struct Engine : EngineBase {
 
     // ---- state (mace.hpp members)
     DVec<F> Phi0, A0, A0_adj, M0, M0_grad, M0_adj, H1, H1_adj, Phi1, dPhi1, A1, A1_adj, M1, M1_grad, M1_adj, msg;
-    DVec<double> H2, H2_adj, hidden, node_energies, node_forces, scratch_d;
+    DVec<double> H2, H2_adj, node_energies, node_forces, scratch_d;
 
     int K() const { return hm.K; }
     int NLM() const { return hm.num_LM; }

@@ -606,7 +606,10 @@ template <typename F, int LMAXH, bool BWD>
 hipError_t launch_agg_sel(const AggParams<F>& p, hipStream_t s)
 {
     constexpr int EC = LMAXH == 0 ? 16 : (BWD ? (sizeof(F) == 4 ? 8 : 4) : 16);
-    if (agg_cpl<F, LMAXH, BWD>(p.K) == 2) return launch_agg_t<F, LMAXH, 2, EC, BWD>(p, s);
+    // two channels per lane exist for the four-path list only (the ten-path kernels have no registers for them)
+    if constexpr (LMAXH == 0) {
+        if (agg_cpl<F, LMAXH, BWD>(p.K) == 2) return launch_agg_t<F, LMAXH, 2, EC, BWD>(p, s);
+    }
     return launch_agg_t<F, LMAXH, 1, EC, BWD>(p, s);
 }
 

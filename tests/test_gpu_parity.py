@@ -549,3 +549,53 @@ def test_rotation_and_replication_through_the_calculator(tmp_models):
     assert np.abs(rep["energies"][len(pos):] - en0).max() <= 1e-10 * max(1.0, np.abs(en0).max())
     assert np.abs(rep["forces"][:len(pos)] - f0).max() <= 1e-8 * max(1.0, np.abs(f0).max())
     assert np.abs(rep["stress"] - res["stress"]).max() <= 1e-9 * max(1.0, np.abs(res["stress"]).max())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("L_max", [0, 1])
+def test_a_step_captured_in_a_hip_graph_replays_bitwise(gpu, tmp_models, L_max):
+    """Callers that cannot launch from the host each step capture the device-resident call once (after a call at the
+    same sizes, which allocates) and replay it.  Replays are interleaved with eager calls on other inputs and each
+    one is compared with the eager result."""
+    import torch
+    model = H.tiny_model(K=32, L_max=L_max, n_pts=48, seed=17, zbl=True, density=(L_max == 1))
+    path = H.write_model(model, tmp_models / f"graph{L_max}.json")
+    eng = gpu(path, "float64")
+    pos, cell, sp = H.small_system(50, seed=2)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    N, E = len(sp), len(ea["r"])
+    dev = torch.device("cuda:0")
+    t = lambda a, dt: torch.from_numpy(np.ascontiguousarray(a)).to(dev, dtype=dt)
+    d = [t(ea["node_types"], torch.int32), t(ea["num_neigh"], torch.int32), t(ea["neigh_indices"], torch.int32),
+         t(ea["neigh_types"], torch.int32), t(ea["xyz"], torch.float64), t(ea["r"], torch.float64)]
+    xyz0, r0 = d[4].clone(), d[5].clone()
+    oE = torch.zeros(N, dtype=torch.float64, device=dev); oF = torch.zeros(3 * E, dtype=torch.float64, device=dev)
+    s = torch.cuda.Stream()
+
+    def step():
+        eng.compute_device(N, *[x.data_ptr() for x in d], E, oE.data_ptr(), oF.data_ptr(), s.cuda_stream)
+
+    with torch.cuda.stream(s):
+        step()
+    torch.cuda.synchronize()
+    refE, refF = oE.clone(), oF.clone()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        step()
+    torch.cuda.synchronize()
+    rng = np.random.default_rng(0)
+    for rep in range(3):
+        # eager work on other inputs in between: the same geometry scaled, which changes every intermediate
+        scale = 1.0 - 0.01 * (rep + 1)
+        d[4].copy_(xyz0 * scale); d[5].copy_(r0 * scale)
+        with torch.cuda.stream(s):
+            step()
+        torch.cuda.synchronize()
+        assert not torch.equal(oF, refF)
+        d[4].copy_(xyz0); d[5].copy_(r0)
+        oE.zero_(); oF.zero_()
+        torch.cuda.synchronize()
+        print(f"replay {rep}", flush=True)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(oE, refE) and torch.equal(oF, refF)

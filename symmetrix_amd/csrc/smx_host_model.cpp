@@ -153,18 +153,20 @@ PolySpec build_poly(int num_lm, int T, int K, const std::vector<std::vector<int>
         }
         if (ents.size() >= 65535) unsupported("more than 65534 monomials in one symmetric-contraction polynomial");
         const int dummy = (int)ents.size() | (ONE << 16) | (ONE << 24);
-        for (int v = 0; v < 16; ++v) {
-            const int s0 = P.list_start[v], sf = s0 + P.list_nfirst[v], s1 = P.list_start[v + 1];
-            const int bounds[3] = {s0, sf, s1};
-            for (int part = 0; part < 2; ++part) {
-                int n = 0;
-                for (int e = bounds[part]; e < bounds[part + 1]; ++e, ++n)
-                    P.packed.push_back(P.list_mono[e] | (P.list_fa[e] << 16) | (P.list_fb[e] << 24));
-                while (n % 4) { P.packed.push_back(dummy); ++n; }
-                P.chunks.push_back(n / 4);
+        // variables in the order the wavefront groups walk them: group g owns v = g, g + POLY_GROUPS, ...
+        for (int g = 0; g < POLY_GROUPS; ++g)
+            for (int v = g; v < 16; v += POLY_GROUPS) {
+                const int s0 = P.list_start[v], sf = s0 + P.list_nfirst[v], s1 = P.list_start[v + 1];
+                const int bounds[3] = {s0, sf, s1};
+                for (int part = 0; part < 2; ++part) {
+                    int n = 0;
+                    for (int e = bounds[part]; e < bounds[part + 1]; ++e, ++n)
+                        P.packed.push_back(P.list_mono[e] | (P.list_fa[e] << 16) | (P.list_fb[e] << 24));
+                    while (n % 4) { P.packed.push_back(dummy); ++n; }
+                    P.chunks.push_back(n / 4);
+                }
             }
-        }
-        for (int q = 0; q < 4; ++q) P.packed.push_back(dummy);
+        for (int q = 0; q < 4 * POLY_SPARE_CHUNKS; ++q) P.packed.push_back(dummy);
     }
     // one extra all-zero coefficient row per species for the padding entries
     P.coef.assign((size_t)T * (ents.size() + 1) * K, 0.0);

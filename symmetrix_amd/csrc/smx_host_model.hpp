@@ -20,6 +20,8 @@ namespace smx {
 // One polynomial family P[type][k](x_0..x_15): monomials grouped in rows that
 // share their first two factors.  Index 16 denotes the constant 1, so that a
 // monomial (a) is stored as (16,16,a) and (a,b) as (16,a,b).
+constexpr int POLY_GROUPS = 4;         // wavefront groups of the contraction kernel that share one atom group
+constexpr int POLY_SPARE_CHUNKS = 2;   // the kernel reads entries this many chunks ahead
 struct PolySpec {
     int num_entries = 0;                         // distinct monomials
     std::vector<int> row_i0, row_i1, row_start;  // row_start has num_rows+1 entries
@@ -35,9 +37,11 @@ struct PolySpec {
     // Device form of the lists: entries packed as mono | fa << 16 | fb << 24, each
     // half-list (first-factor entries of v, then the rest of v) padded to a
     // multiple of four with entries that point at an all-zero coefficient row
-    // (index num_entries), plus one spare chunk at the end for the prefetch.
-    std::vector<int> packed;                     // [4 * (total chunks + 1)]
-    std::vector<int> chunks;                     // [32]: chunks of (v, first part), (v, rest)
+    // (index num_entries), plus spare chunks at the end for the prefetch.  The
+    // variables follow each other in the order v = g, g + POLY_GROUPS, ... for
+    // g = 0 .. POLY_GROUPS-1, so that each group's chunks are contiguous.
+    std::vector<int> packed;                     // [4 * (total chunks + POLY_SPARE_CHUNKS)]
+    std::vector<int> chunks;                     // [32]: chunks of (v, first part), (v, rest), same order
 };
 
 struct HostModel {

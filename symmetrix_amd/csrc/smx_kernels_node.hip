@@ -1,6 +1,7 @@
 // Node-level kernels for gfx950: symmetric contraction, MFMA channel mixing,
 // readout tail, integer list preparation and caller-side force reduction.
 #include "smx_kernels.hpp"
+#include "smx_host_model.hpp"
 
 namespace smx {
 
@@ -351,6 +352,7 @@ constexpr int POLY_BLOCK = 128;
 // all of them and every loaded coefficient serves them all.  (Twice as many was measured slower: fewer
 // blocks than the chip holds at once.)
 template <typename F> constexpr int poly_nb() { return 16 / (int)sizeof(F); }
+typedef int __attribute__((address_space(4))) ConstInt;
 template <typename F, int N>
 struct alignas(16) PolyVec {
     F v[N];
@@ -360,7 +362,8 @@ struct alignas(16) PolyVec {
 // the variables v = g, g + POLY_VG, ...  A block is latency bound (every list entry needs a coefficient
 // from L2), so spreading the 16 lists of an atom group over four times as many wavefronts shortens the
 // kernel by nearly that factor.
-constexpr int POLY_VG = 4;
+constexpr int POLY_VG = POLY_GROUPS;
+static_assert(16 % POLY_VG == 0 && POLY_BLOCK % 64 == 0 && POLY_SPARE_CHUNKS >= 2, "list layout and the kernel's walk must agree");
 
 template <typename F>
 __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<F> a)
@@ -368,7 +371,10 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
     constexpr int NB = poly_nb<F>();
     __shared__ PolyVec<F, NB> X[17][POLY_BLOCK];
     __shared__ PolyVec<F, NB> fsum[POLY_VG][POLY_BLOCK];
-    const int tid = threadIdx.x % POLY_BLOCK, vg = threadIdx.x / POLY_BLOCK;
+    // the group index is the same for a whole wavefront: as a scalar it keeps the walk through the lists
+    // (indices, chunk counts, coefficient rows) in scalar registers and scalar loads
+    const int tid = threadIdx.x % POLY_BLOCK, vg = __builtin_amdgcn_readfirstlane(threadIdx.x / POLY_BLOCK);
+    constexpr int VPG = 16 / POLY_VG;   // variables per group
     // species segment and group of atoms of this block row
     const int kblocks = (a.K + POLY_BLOCK - 1) / POLY_BLOCK;
     int type = -1, grp = blockIdx.x / kblocks, seg0 = 0, seg_n = 0;
@@ -381,7 +387,7 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
     if (type < 0) return;
     const int k = (blockIdx.x % kblocks) * POLY_BLOCK + tid;
     const bool klive = k < a.K;
-    const int kk = klive ? k : a.K - 1;
+    const unsigned kk = klive ? k : a.K - 1;
     int node[NB];
     bool nlive[NB];
 #pragma unroll
@@ -398,44 +404,69 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
     }
     __syncthreads();
     for (int pl = 0; pl < a.NP; ++pl) {
-        const int4* pk = a.packed[pl];
-        const int* nch = a.chunks[pl];
-        const F* coef = a.coef[pl] + (size_t)type * (a.num_entries[pl] + 1) * a.K + kk;
-        F f[NB];
+        // the lists are read-only model data, the same for every lane: through the constant address space
+        // they are fetched by scalar loads
+        const ConstInt* pki = (const ConstInt*)a.packed[pl];
+        auto pk = [&](int ch) { return make_int4(pki[4 * ch], pki[4 * ch + 1], pki[4 * ch + 2], pki[4 * ch + 3]); };
+        const ConstInt* nch = (const ConstInt*)a.chunks[pl];
+        // scalar base in the global address space; the lane adds kk
+        typedef const F __attribute__((address_space(1))) GlobalF;
+        GlobalF* coef = (GlobalF*)a.coef[pl] + (size_t)type * (a.num_entries[pl] + 1) * a.K;
+        F f[NB], g[NB];
 #pragma unroll
-        for (int b = 0; b < NB; ++b) f[b] = F(0);
-        int c = 0;   // first chunk of variable v
-        for (int v = 0; v < 16; ++v) {
-            const int n0 = nch[2 * v], n1 = nch[2 * v + 1];
-            if (v % POLY_VG == vg) {
-                F g[NB];
+        for (int b = 0; b < NB; ++b) f[b] = g[b] = F(0);
+        // this group's chunks are contiguous: [c, c_end)
+        int c = 0;
+        for (int q = 0; q < 2 * VPG * vg; ++q) c += nch[q];
+        int c_end = c;
+        for (int q = 0; q < 2 * VPG; ++q) c_end += nch[2 * VPG * vg + q];
+        int t = 0, v = vg, done = 0;
+        int n0 = nch[2 * VPG * vg], n1 = nch[2 * VPG * vg + 1];
+        // a finished variable (possibly one without entries) stores its gradient and hands over to the next
+        auto flush = [&]() {
+            while (t < VPG && done == n0 + n1) {
 #pragma unroll
-                for (int b = 0; b < NB; ++b) g[b] = F(0);
-                int4 cur = pk[c];
-                for (int j = 0; j < n0 + n1; ++j) {
-                    const int4 nxt = pk[c + j + 1];   // next chunk's indices are in flight while this one is used
-                    const int e4[4] = {cur.x, cur.y, cur.z, cur.w};
-#pragma unroll
-                    for (int q = 0; q < 4; ++q) {
-                        const int mono = e4[q] & 0xffff, ia = (e4[q] >> 16) & 0xff, ib = (e4[q] >> 24) & 0xff;
-                        const F w = coef[(size_t)mono * a.K];
-                        const PolyVec<F, NB> xa = X[ia][tid], xb = X[ib][tid];
-#pragma unroll
-                        for (int b = 0; b < NB; ++b) g[b] += w * (xa.v[b] * xb.v[b]);
-                    }
-                    cur = nxt;
-                    if (j == n0 - 1) {
-                        // the monomials that start with v are done: their sum times x_v is v's share of P
-                        const PolyVec<F, NB> xv = X[v][tid];
-#pragma unroll
-                        for (int b = 0; b < NB; ++b) f[b] += xv.v[b] * g[b];
-                    }
-                }
-#pragma unroll
-                for (int b = 0; b < NB; ++b)
+                for (int b = 0; b < NB; ++b) {
                     if (klive && nlive[b]) a.M_grad[(((size_t)node[b] * a.NP + pl) * 16 + v) * a.K + k] = g[b];
+                    g[b] = F(0);
+                }
+                ++t; v += POLY_VG; done = 0;
+                if (t < VPG) { n0 = nch[2 * (VPG * vg + t)]; n1 = nch[2 * (VPG * vg + t) + 1]; }
             }
-            c += n0 + n1;
+        };
+        auto weights = [&](const int4& e, F (&w)[4]) {
+            const int e4[4] = {e.x, e.y, e.z, e.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) w[q] = (coef + (size_t)(e4[q] & 0xffff) * a.K)[kk];
+        };
+        flush();
+        // indices two chunks ahead and coefficients one chunk ahead of the arithmetic; the list ends with
+        // spare chunks of padding entries, so nothing here depends on where the group's range stops
+        int4 cur = pk(c), nxt = pk(c + 1);
+        F w[4];
+        weights(cur, w);
+        for (; c < c_end; ++c) {
+            F wn[4];
+            weights(nxt, wn);
+            const int4 nn = pk(c + 2);
+            const int e4[4] = {cur.x, cur.y, cur.z, cur.w};
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                const int ia = (e4[q] >> 16) & 0xff, ib = (e4[q] >> 24) & 0xff;
+                const PolyVec<F, NB> xa = X[ia][tid], xb = X[ib][tid];
+#pragma unroll
+                for (int b = 0; b < NB; ++b) g[b] += w[q] * (xa.v[b] * xb.v[b]);
+            }
+            cur = nxt; nxt = nn;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) w[q] = wn[q];
+            if (++done == n0) {
+                // the monomials that start with v are done: their sum times x_v is v's share of P
+                const PolyVec<F, NB> xv = X[v][tid];
+#pragma unroll
+                for (int b = 0; b < NB; ++b) f[b] += xv.v[b] * g[b];
+            }
+            flush();
         }
         // P = sum of the groups' shares, added in group order
         {

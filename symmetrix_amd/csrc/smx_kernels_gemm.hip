@@ -13,6 +13,8 @@
 // 4*r+L/16 (f64).
 #include "smx_kernels.hpp"
 
+#include <algorithm>
+
 namespace smx {
 
 namespace {
@@ -206,6 +208,225 @@ __global__ __launch_bounds__(256) void k_gemm(const GemmParams<TA, TC, CT> g)
     }
 }
 
+// ---------------------------------------------------------------------------
+// Row-streaming variant for inner sizes up to 128 (every channel mixing of a K <= 128 model except the
+// concatenated ones).  The whole weight block [Kd][GN] sits in LDS for the life of the block, so after
+// one barrier the eight wavefronts never synchronise again: wavefront (s, h) streams 16-row tiles
+// s, s+4, ... of the block's row range straight from global memory into the A-operand registers (a lane
+// loads 32 contiguous bytes per row, i.e. whole 128-byte lines per 16-lane group; the matrix cores see the
+// k index permuted inside groups of KG, which a sum over k allows), keeps the next tile's rows in flight
+// while it multiplies, and owns the column tiles of half h.  The two wavefronts that share a SIMD thus
+// do the same number of matrix instructions.
+template <typename T, int N>
+struct alignas(16) VecN {
+    T v[N];
+};
+template <typename CT> constexpr int rows_vl() { return 32 / (int)sizeof(CT); }   // k values per lane and group
+template <typename CT, int NTW> constexpr int rows_sw() { return 32 * NTW + (sizeof(CT) == 4 ? 2 : 0); }
+constexpr int ROWS_KMAX = 128;
+constexpr int ROWS_MMAX = 8;                     // 16-row tiles per wavefront at most
+constexpr size_t ROWS_OFFS_BYTES = 8 * ROWS_MMAX * 16 * sizeof(int2);
+
+template <typename TA, typename TC, typename CT, int NTW>
+__global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> g, const int m)
+{
+    constexpr int VL = rows_vl<CT>(), KG = 4 * VL, KJ = ROWS_KMAX / KG;
+    constexpr int GN = 32 * NTW, SW = rows_sw<CT, NTW>();
+    extern __shared__ __align__(16) unsigned char smem_raw[];
+    CT* Wl = reinterpret_cast<CT*>(smem_raw);          // [Kp][SW], rows Kd..Kp-1 zero
+    const GemmProb<TA, TC, CT>& pr = g.prob[blockIdx.z];
+    const int Nn = pr.Nn, Kd = pr.Kd, sub = pr.sub;
+    const int col0 = blockIdx.y * GN;
+    if (col0 >= Nn) return;
+    const int chunk_rows = 64 * m;
+    int type = 0, chunk = blockIdx.x, nrows_seg = g.num_nodes * sub, seg_node0 = 0;
+    if (g.perm) {
+        bool found = false;
+        for (int t = 0; t < g.T; ++t) {
+            const int n_t = g.tstart[t + 1] - g.tstart[t];
+            const int chunks = (n_t * sub + chunk_rows - 1) / chunk_rows;
+            if (chunk < chunks) { type = t; nrows_seg = n_t * sub; seg_node0 = g.tstart[t]; found = true; break; }
+            chunk -= chunks;
+        }
+        if (!found) return;
+    } else if ((long)chunk * chunk_rows >= nrows_seg) {
+        return;
+    }
+    const int tid = threadIdx.x;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    const int srow = wave & 3, t0 = (wave >> 2) * NTW;
+    const int r = lane & 15, gq = lane >> 4;
+    const int row_base = chunk * chunk_rows;
+
+    // Row `rr` of the segment as (node, sub-row); beyond the segment the last row with a flag: its A row is
+    // still loaded (so that every load below is unconditional straight-line code the matrix instructions
+    // need not wait for), what it produces is never stored.
+    constexpr int OUTSIDE = 1 << 30;
+    auto row_of = [&](int rr) {
+        const bool inside = rr < nrows_seg;
+        const int rc = inside ? rr : nrows_seg - 1;
+        const int ns = rc / sub, sb = rc - ns * sub;
+        const int node = g.perm ? g.perm[seg_node0 + ns] : ns;
+        return make_int2(node, inside ? sb : sb | OUTSIDE);
+    };
+    auto a_offset = [&](int2 o) { return (long)o.x * pr.a_node_stride + pr.a_off + (long)(o.y & ~OUTSIDE) * pr.a_sub_stride; };
+    auto c_offset = [&](int2 o) {
+        return (o.y & OUTSIDE) ? -1L : (long)o.x * pr.c_node_stride + pr.c_off + (long)o.y * pr.c_sub_stride;
+    };
+    // a run beyond Kd (a multiple of VL) is read from the last run instead: it meets zero rows of Wl
+    auto fetch = [&](long ao, VecN<CT, VL> (&a)[KJ]) {
+#pragma unroll
+        for (int jj = 0; jj < KJ; ++jj) {
+            const int k0 = min(jj * KG + gq * VL, Kd - VL);
+            const TA* src = pr.A + ao + k0;
+#pragma unroll
+            for (int q = 0; q < VL; q += 4) {
+                const Vec4<TA> t = *reinterpret_cast<const Vec4<TA>*>(src + q);
+#pragma unroll
+                for (int u = 0; u < 4; ++u) a[jj].v[q + u] = (CT)t.v[u];
+            }
+        }
+    };
+
+    // The rows of all tiles of this wavefront go through a private LDS table first (lane group gq fills
+    // tiles gq and gq + 4): inside the tile loop the only vector-memory operations are then the row loads
+    // and the stores, and no small dependent load has to be waited for behind a tile's stores.
+    int2* rows_of = reinterpret_cast<int2*>(smem_raw + (size_t)((Kd + KG - 1) / KG * KG) * SW * sizeof(CT)) + wave * (ROWS_MMAX * 16);
+    for (int jt = gq; jt < m; jt += 4) rows_of[jt * 16 + r] = row_of(row_base + (srow + 4 * jt) * 16 + r);
+    int2 o_cur = rows_of[r];
+    const long ao = a_offset(o_cur);
+    VecN<CT, VL> a[KJ];
+    fetch(ao, a);
+    // the weight block goes to LDS while the first rows are on their way: all loads first, then the writes
+    {
+        const CT* W = pr.W + (size_t)type * pr.w_type_stride + pr.w_off;
+        const int Kp = (Kd + KG - 1) / KG * KG;
+        constexpr int WQ = ROWS_KMAX * (GN / 4) / 512;   // four-element groups per thread at most
+        Vec4<CT> w[WQ];
+        const int groups = Kp * (GN / 4);
+#pragma unroll
+        for (int q = 0; q < WQ; ++q) {
+            const int v = tid + q * 512;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) w[q].v[j] = CT(0);
+            if (v < groups) {
+                if (!pr.transW) {
+                    // W block is [Kd][Nn]: four consecutive columns of one k
+                    const int k = v / (GN / 4), n = (v % (GN / 4)) * 4;
+                    if (k < Kd) w[q] = load4<CT, CT>(W + (size_t)k * Nn, col0 + n, Nn, true);
+                } else {
+                    // W block is [Nn][Kd]: four consecutive k of one column
+                    const int k = (v % (Kp / 4)) * 4, n = v / (Kp / 4);
+                    if (col0 + n < Nn) w[q] = load4<CT, CT>(W + (size_t)(col0 + n) * Kd, k, Kd, true);
+                }
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < WQ; ++q) {
+            const int v = tid + q * 512;
+            if (v < groups) {
+                if (!pr.transW) {
+                    const int k = v / (GN / 4), n = (v % (GN / 4)) * 4;
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) Wl[k * SW + n + j] = w[q].v[j];
+                } else {
+                    const int k = (v % (Kp / 4)) * 4, n = v / (Kp / 4);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) Wl[(k + j) * SW + n] = w[q].v[j];
+                }
+            }
+        }
+    }
+    __syncthreads();
+    if (col0 + t0 * 16 >= Nn) return;                   // this half has no live column
+    const CT* wl = Wl + gq * VL * SW + t0 * 16 + r;
+    for (int j = 0; j < m; ++j) {
+        const int row0 = row_base + (srow + 4 * j) * 16;
+        if (row0 >= nrows_seg) break;
+        // rows of the next tile (past the last one: the last one again, unused)
+        const int2 o_n = rows_of[min(j + 1, m - 1) * 16 + r];
+        VecN<CT, VL> an[KJ];
+        fetch(a_offset(o_n), an);
+
+        typename Mfma<CT>::acc_t acc[NTW];
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) acc[t] = {0, 0, 0, 0};
+#pragma unroll
+        for (int jj = 0; jj < KJ; ++jj) {
+            if (jj * KG < Kd) {
+#pragma unroll
+                for (int q = 0; q < VL; ++q) {
+#pragma unroll
+                    for (int t = 0; t < NTW; ++t) {
+                        const CT bv = wl[(jj * KG + q) * SW + t * 16];
+                        acc[t] = Mfma<CT>::run(a[jj].v[q], bv, acc[t]);
+                    }
+                }
+            }
+        }
+        // The next tile's rows become the current ones before this tile's results are stored: waiting for
+        // them here waits for loads issued a tile ago, after the stores it would wait for the stores too.
+#pragma unroll
+        for (int jj = 0; jj < KJ; ++jj) {
+            a[jj] = an[jj];
+#pragma unroll
+            for (int q = 0; q < VL; ++q) asm volatile("" : "+v"(a[jj].v[q]));
+        }
+        // the offset of output row q is held by lane q
+        const long co = c_offset(o_cur);
+        long crow[4];
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int src = Mfma<CT>::out_row(lane, q);
+            const int lo = __shfl((int)(co & 0xffffffff), src), hi = __shfl((int)(co >> 32), src);
+            crow[q] = ((long)hi << 32) | (unsigned)lo;
+        }
+#pragma unroll
+        for (int t = 0; t < NTW; ++t) {
+            const int nn = col0 + (t0 + t) * 16 + r;
+            if (nn >= Nn) continue;
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+                if (crow[q] < 0) continue;
+                const CT v = acc[t][q];
+                if (pr.accumulate) pr.C[crow[q] + nn] = (TC)((CT)pr.C[crow[q] + nn] + v);
+                else pr.C[crow[q] + nn] = (TC)v;
+            }
+        }
+        o_cur = o_n;
+    }
+}
+
+template <typename TA, typename TC, typename CT, int NTW>
+hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, int max_k, long total_rows,
+                              hipStream_t s)
+{
+    constexpr int GN = 32 * NTW, KG = 4 * rows_vl<CT>();
+    const size_t lds = (size_t)((max_k + KG - 1) / KG * KG) * rows_sw<CT, NTW>() * sizeof(CT) + ROWS_OFFS_BYTES;
+    static bool attr_done = false;   // per instantiation
+    if (!attr_done) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_rows<TA, TC, CT, NTW>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (err != hipSuccess) return err;
+        attr_done = true;
+    }
+    const unsigned gy = (unsigned)((max_n + GN - 1) / GN);
+    // 16-row tiles per SIMD of a block (at most eight): the smallest number with which all blocks that find
+    // rows are resident at once.  Blocks go to the eight dies in turn, whatever they find there, so the
+    // count leaves an eighth of the block slots free for an uneven split.
+    int per_cu = 1;
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemm_rows<TA, TC, CT, NTW>, 512, lds) != hipSuccess || per_cu < 1)
+        per_cu = 1;
+    const long slots = 224L * per_cu;
+    const long slack = p.perm ? std::min<long>((long)p.nprob * p.T, 64) : p.nprob;
+    long m = 1;
+    while (m < ROWS_MMAX && (total_rows + 64 * m - 1) / (64 * m) * gy + slack > slots) ++m;
+    const long rows = (long)p.num_nodes * max_sub;
+    const unsigned gx = (unsigned)((rows + 64 * m - 1) / (64 * m) + (p.perm ? p.T : 0));
+    hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW>), dim3(gx, gy, p.nprob), dim3(512), lds, s, p, (int)m);
+    return hipGetLastError();
+}
+
 template <typename TA, typename TC, typename CT, int NT>
 hipError_t launch_gemm_t(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, hipStream_t s)
 {
@@ -236,6 +457,23 @@ hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p_in, hipStream_t s)
         if (q.A2) vec = vec && mult4(q.Kd2) && mult4(q.a2_node_stride) && mult4(q.w2_type_stride);
     }
     p.vec_ok = vec ? 1 : 0;
+    // row-streaming kernel: weights of one block resident in LDS
+    {
+        bool rows_ok = vec && max_n >= 32;
+        int max_k = 0;
+        long total_rows = 0;
+        for (int z = 0; z < p.nprob; ++z) {
+            const auto& q = p.prob[z];
+            rows_ok = rows_ok && !q.A2 && q.Kd <= ROWS_KMAX && q.Kd % rows_vl<CT>() == 0;
+            max_k = max_k > q.Kd ? max_k : q.Kd;
+            total_rows += (long)p.num_nodes * q.sub;
+        }
+        if (rows_ok) {
+            if (max_n % 96 == 0) return launch_gemm_rows_t<TA, TC, CT, 3>(p, max_sub, max_n, max_k, total_rows, s);
+            if (max_n <= 64) return launch_gemm_rows_t<TA, TC, CT, 2>(p, max_sub, max_n, max_k, total_rows, s);
+            return launch_gemm_rows_t<TA, TC, CT, 4>(p, max_sub, max_n, max_k, total_rows, s);
+        }
+    }
     // tile width: the narrowest of 16, 32, 64, 96, 128 that covers the output, else the least padded of 64, 96, 128
     int nt = 8;
     if (max_n <= 16) nt = 1;

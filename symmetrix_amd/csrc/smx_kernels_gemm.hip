@@ -273,34 +273,41 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
     auto c_offset = [&](int2 o) {
         return (o.y & OUTSIDE) ? -1L : (long)o.x * pr.c_node_stride + pr.c_off + (long)o.y * pr.c_sub_stride;
     };
-    // a run beyond Kd (a multiple of VL) is read from the last run instead: it meets zero rows of Wl
-    auto fetch = [&](long ao, VecN<CT, VL> (&a)[KJ]) {
+    // a run beyond Kx (a multiple of VL) is read from the last run instead: it meets zero rows of the weights
+    auto fetch = [&](const TA* A, long ao, int Kx, VecN<CT, VL> (&dst)[KJ]) {
 #pragma unroll
         for (int jj = 0; jj < KJ; ++jj) {
-            const int k0 = min(jj * KG + gq * VL, Kd - VL);
-            const TA* src = pr.A + ao + k0;
+            const int k0 = min(jj * KG + gq * VL, Kx - VL);
+            const TA* src = A + ao + k0;
 #pragma unroll
             for (int q = 0; q < VL; q += 4) {
                 const Vec4<TA> t = *reinterpret_cast<const Vec4<TA>*>(src + q);
 #pragma unroll
-                for (int u = 0; u < 4; ++u) a[jj].v[q + u] = (CT)t.v[u];
+                for (int u = 0; u < 4; ++u) dst[jj].v[q + u] = (CT)t.v[u];
             }
         }
     };
 
+    // A problem with a second product (sub = 1) walks every tile twice: first A with W, then A2 with W2
+    // into the same accumulators; both weight blocks are resident.
+    const int S = pr.A2 ? 2 : 1;
+    const int Kp1 = (Kd + KG - 1) / KG * KG, Kp2 = pr.A2 ? (pr.Kd2 + KG - 1) / KG * KG : 0;
+    CT* Wl2 = Wl + (size_t)Kp1 * SW;
     // The rows of all tiles of this wavefront go through a private LDS table first (lane group gq fills
     // tiles gq and gq + 4): inside the tile loop the only vector-memory operations are then the row loads
     // and the stores, and no small dependent load has to be waited for behind a tile's stores.
-    int2* rows_of = reinterpret_cast<int2*>(smem_raw + (size_t)((Kd + KG - 1) / KG * KG) * SW * sizeof(CT)) + wave * (ROWS_MMAX * 16);
+    int2* rows_of = reinterpret_cast<int2*>(smem_raw + (size_t)(Kp1 + Kp2) * SW * sizeof(CT)) + wave * (ROWS_MMAX * 16);
     for (int jt = gq; jt < m; jt += 4) rows_of[jt * 16 + r] = row_of(row_base + (srow + 4 * jt) * 16 + r);
     int2 o_cur = rows_of[r];
-    const long ao = a_offset(o_cur);
+    // step u = tile u / S, source u % S
+    auto fetch_step = [&](int2 o, int src, VecN<CT, VL> (&dst)[KJ]) {
+        if (src == 0) fetch(pr.A, a_offset(o), Kd, dst);
+        else fetch(pr.A2, (long)o.x * pr.a2_node_stride, pr.Kd2, dst);
+    };
     VecN<CT, VL> a[KJ];
-    fetch(ao, a);
-    // the weight block goes to LDS while the first rows are on their way: all loads first, then the writes
-    {
-        const CT* W = pr.W + (size_t)type * pr.w_type_stride + pr.w_off;
-        const int Kp = (Kd + KG - 1) / KG * KG;
+    fetch_step(o_cur, 0, a);
+    // the weight blocks go to LDS while the first rows are on their way: all loads first, then the writes
+    auto load_w = [&](CT* dst, const CT* W, int trans, int Kw, int Kp) {
         constexpr int WQ = ROWS_KMAX * (GN / 4) / 512;   // four-element groups per thread at most
         Vec4<CT> w[WQ];
         const int groups = Kp * (GN / 4);
@@ -310,14 +317,14 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
 #pragma unroll
             for (int j = 0; j < 4; ++j) w[q].v[j] = CT(0);
             if (v < groups) {
-                if (!pr.transW) {
-                    // W block is [Kd][Nn]: four consecutive columns of one k
+                if (!trans) {
+                    // W block is [Kw][Nn]: four consecutive columns of one k
                     const int k = v / (GN / 4), n = (v % (GN / 4)) * 4;
-                    if (k < Kd) w[q] = load4<CT, CT>(W + (size_t)k * Nn, col0 + n, Nn, true);
+                    if (k < Kw) w[q] = load4<CT, CT>(W + (size_t)k * Nn, col0 + n, Nn, true);
                 } else {
-                    // W block is [Nn][Kd]: four consecutive k of one column
+                    // W block is [Nn][Kw]: four consecutive k of one column
                     const int k = (v % (Kp / 4)) * 4, n = v / (Kp / 4);
-                    if (col0 + n < Nn) w[q] = load4<CT, CT>(W + (size_t)(col0 + n) * Kd, k, Kd, true);
+                    if (col0 + n < Nn) w[q] = load4<CT, CT>(W + (size_t)(col0 + n) * Kw, k, Kw, true);
                 }
             }
         }
@@ -325,35 +332,43 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
         for (int q = 0; q < WQ; ++q) {
             const int v = tid + q * 512;
             if (v < groups) {
-                if (!pr.transW) {
+                if (!trans) {
                     const int k = v / (GN / 4), n = (v % (GN / 4)) * 4;
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) Wl[k * SW + n + j] = w[q].v[j];
+                    for (int j = 0; j < 4; ++j) dst[k * SW + n + j] = w[q].v[j];
                 } else {
                     const int k = (v % (Kp / 4)) * 4, n = v / (Kp / 4);
 #pragma unroll
-                    for (int j = 0; j < 4; ++j) Wl[(k + j) * SW + n] = w[q].v[j];
+                    for (int j = 0; j < 4; ++j) dst[(k + j) * SW + n] = w[q].v[j];
                 }
             }
         }
-    }
+    };
+    load_w(Wl, pr.W + (size_t)type * pr.w_type_stride + pr.w_off, pr.transW, Kd, Kp1);
+    if (pr.A2) load_w(Wl2, pr.W2 + (size_t)type * pr.w2_type_stride, pr.transW2, pr.Kd2, Kp2);
     __syncthreads();
     if (col0 + t0 * 16 >= Nn) return;                   // this half has no live column
-    const CT* wl = Wl + gq * VL * SW + t0 * 16 + r;
-    for (int j = 0; j < m; ++j) {
-        const int row0 = row_base + (srow + 4 * j) * 16;
-        if (row0 >= nrows_seg) break;
-        // rows of the next tile (past the last one: the last one again, unused)
-        const int2 o_n = rows_of[min(j + 1, m - 1) * 16 + r];
+    const int lane_w = gq * VL * SW + t0 * 16 + r;
+    typename Mfma<CT>::acc_t acc[NTW];
+    const int steps = m * S;
+    for (int u = 0; u < steps; ++u) {
+        const int j = u / S, src = u - j * S;
+        if (row_base + (srow + 4 * j) * 16 >= nrows_seg) break;
+        // rows of the next step (past the last one: the last one again, unused)
+        const int un = min(u + 1, steps - 1), jn = un / S;
+        const int2 o_n = rows_of[jn * 16 + r];
         VecN<CT, VL> an[KJ];
-        fetch(a_offset(o_n), an);
+        fetch_step(o_n, un - jn * S, an);
 
-        typename Mfma<CT>::acc_t acc[NTW];
+        if (src == 0) {
 #pragma unroll
-        for (int t = 0; t < NTW; ++t) acc[t] = {0, 0, 0, 0};
+            for (int t = 0; t < NTW; ++t) acc[t] = {0, 0, 0, 0};
+        }
+        const CT* wl = (src ? Wl2 : Wl) + lane_w;
+        const int Ks = src ? pr.Kd2 : Kd;
 #pragma unroll
         for (int jj = 0; jj < KJ; ++jj) {
-            if (jj * KG < Kd) {
+            if (jj * KG < Ks) {
 #pragma unroll
                 for (int q = 0; q < VL; ++q) {
 #pragma unroll
@@ -364,33 +379,35 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
                 }
             }
         }
-        // The next tile's rows become the current ones before this tile's results are stored: waiting for
-        // them here waits for loads issued a tile ago, after the stores it would wait for the stores too.
+        // The next step's rows become the current ones before this tile's results are stored: waiting for
+        // them here waits for loads issued a step ago, after the stores it would wait for the stores too.
 #pragma unroll
         for (int jj = 0; jj < KJ; ++jj) {
             a[jj] = an[jj];
 #pragma unroll
             for (int q = 0; q < VL; ++q) asm volatile("" : "+v"(a[jj].v[q]));
         }
-        // the offset of output row q is held by lane q
-        const long co = c_offset(o_cur);
-        long crow[4];
-#pragma unroll
-        for (int q = 0; q < 4; ++q) {
-            const int src = Mfma<CT>::out_row(lane, q);
-            const int lo = __shfl((int)(co & 0xffffffff), src), hi = __shfl((int)(co >> 32), src);
-            crow[q] = ((long)hi << 32) | (unsigned)lo;
-        }
-#pragma unroll
-        for (int t = 0; t < NTW; ++t) {
-            const int nn = col0 + (t0 + t) * 16 + r;
-            if (nn >= Nn) continue;
+        if (src == S - 1) {
+            // the offset of output row q is held by lane q
+            const long co = c_offset(o_cur);
+            long crow[4];
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
-                if (crow[q] < 0) continue;
-                const CT v = acc[t][q];
-                if (pr.accumulate) pr.C[crow[q] + nn] = (TC)((CT)pr.C[crow[q] + nn] + v);
-                else pr.C[crow[q] + nn] = (TC)v;
+                const int from = Mfma<CT>::out_row(lane, q);
+                const int lo = __shfl((int)(co & 0xffffffff), from), hi = __shfl((int)(co >> 32), from);
+                crow[q] = ((long)hi << 32) | (unsigned)lo;
+            }
+#pragma unroll
+            for (int t = 0; t < NTW; ++t) {
+                const int nn = col0 + (t0 + t) * 16 + r;
+                if (nn >= Nn) continue;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    if (crow[q] < 0) continue;
+                    const CT v = acc[t][q];
+                    if (pr.accumulate) pr.C[crow[q] + nn] = (TC)((CT)pr.C[crow[q] + nn] + v);
+                    else pr.C[crow[q] + nn] = (TC)v;
+                }
             }
         }
         o_cur = o_n;
@@ -398,11 +415,10 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
 }
 
 template <typename TA, typename TC, typename CT, int NTW>
-hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, int max_k, long total_rows,
+hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, size_t lds, long total_rows,
                               hipStream_t s)
 {
-    constexpr int GN = 32 * NTW, KG = 4 * rows_vl<CT>();
-    const size_t lds = (size_t)((max_k + KG - 1) / KG * KG) * rows_sw<CT, NTW>() * sizeof(CT) + ROWS_OFFS_BYTES;
+    constexpr int GN = 32 * NTW;
     static bool attr_done = false;   // per instantiation
     if (!attr_done) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_rows<TA, TC, CT, NTW>),
@@ -459,19 +475,38 @@ hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p_in, hipStream_t s)
     p.vec_ok = vec ? 1 : 0;
     // row-streaming kernel: weights of one block resident in LDS
     {
+        constexpr int VL = rows_vl<CT>(), KG = 4 * VL;
         bool rows_ok = vec && max_n >= 32;
-        int max_k = 0;
-        long total_rows = 0;
+        long kp_sum = 0, total_rows = 0;   // padded inner sizes of the widest problem (both products)
         for (int z = 0; z < p.nprob; ++z) {
             const auto& q = p.prob[z];
-            rows_ok = rows_ok && !q.A2 && q.Kd <= ROWS_KMAX && q.Kd % rows_vl<CT>() == 0;
-            max_k = max_k > q.Kd ? max_k : q.Kd;
+            rows_ok = rows_ok && q.Kd <= ROWS_KMAX && q.Kd % VL == 0;
+            long kp = (q.Kd + KG - 1) / KG * KG;
+            if (q.A2) {
+                rows_ok = rows_ok && q.Kd2 <= ROWS_KMAX && q.Kd2 % VL == 0;
+                kp += (q.Kd2 + KG - 1) / KG * KG;
+            }
+            kp_sum = kp_sum > kp ? kp_sum : kp;
             total_rows += (long)p.num_nodes * q.sub;
         }
         if (rows_ok) {
-            if (max_n % 96 == 0) return launch_gemm_rows_t<TA, TC, CT, 3>(p, max_sub, max_n, max_k, total_rows, s);
-            if (max_n <= 64) return launch_gemm_rows_t<TA, TC, CT, 2>(p, max_sub, max_n, max_k, total_rows, s);
-            return launch_gemm_rows_t<TA, TC, CT, 4>(p, max_sub, max_n, max_k, total_rows, s);
+            auto lds_for = [&](int ntw) {
+                return (size_t)kp_sum * (32 * ntw + (sizeof(CT) == 4 ? 2 : 0)) * sizeof(CT) + ROWS_OFFS_BYTES;
+            };
+            // preferred width of a column block: narrow for few rows (more compute units share the work),
+            // else the one that tiles the output; narrower when the weight blocks would not fit
+            int ntw = (total_rows <= 128 * 64 && max_n % 32 == 0) ? 1 : max_n % 96 == 0 ? 3 : max_n <= 64 ? 2 : 4;
+            while (ntw > 1 && lds_for(ntw) > 160 * 1024) --ntw;
+            if (ntw == 3 && max_n % 96 != 0) ntw = 2;
+            const size_t lds = lds_for(ntw);
+            if (lds <= 160 * 1024) {
+                switch (ntw) {
+                case 1: return launch_gemm_rows_t<TA, TC, CT, 1>(p, max_sub, max_n, lds, total_rows, s);
+                case 2: return launch_gemm_rows_t<TA, TC, CT, 2>(p, max_sub, max_n, lds, total_rows, s);
+                case 3: return launch_gemm_rows_t<TA, TC, CT, 3>(p, max_sub, max_n, lds, total_rows, s);
+                default: return launch_gemm_rows_t<TA, TC, CT, 4>(p, max_sub, max_n, lds, total_rows, s);
+                }
+            }
         }
     }
     // tile width: the narrowest of 16, 32, 64, 96, 128 that covers the output, else the least padded of 64, 96, 128

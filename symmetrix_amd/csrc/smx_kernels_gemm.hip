@@ -293,23 +293,11 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
     const int S = pr.A2 ? 2 : 1;
     const int Kp1 = (Kd + KG - 1) / KG * KG, Kp2 = pr.A2 ? (pr.Kd2 + KG - 1) / KG * KG : 0;
     CT* Wl2 = Wl + (size_t)Kp1 * SW;
-    // The rows of all tiles of this wavefront go through a private LDS table first (lane group gq fills
-    // tiles gq and gq + 4): inside the tile loop the only vector-memory operations are then the row loads
-    // and the stores, and no small dependent load has to be waited for behind a tile's stores.
-    int2* rows_of = reinterpret_cast<int2*>(smem_raw + (size_t)(Kp1 + Kp2) * SW * sizeof(CT)) + wave * (ROWS_MMAX * 16);
-    for (int jt = gq; jt < m; jt += 4) rows_of[jt * 16 + r] = row_of(row_base + (srow + 4 * jt) * 16 + r);
-    int2 o_cur = rows_of[r];
-    // step u = tile u / S, source u % S
-    auto fetch_step = [&](int2 o, int src, VecN<CT, VL> (&dst)[KJ]) {
-        if (src == 0) fetch(pr.A, a_offset(o), Kd, dst);
-        else fetch(pr.A2, (long)o.x * pr.a2_node_stride, pr.Kd2, dst);
-    };
-    VecN<CT, VL> a[KJ];
-    fetch_step(o_cur, 0, a);
-    // the weight blocks go to LDS while the first rows are on their way: all loads first, then the writes
-    auto load_w = [&](CT* dst, const CT* W, int trans, int Kw, int Kp) {
-        constexpr int WQ = ROWS_KMAX * (GN / 4) / 512;   // four-element groups per thread at most
-        Vec4<CT> w[WQ];
+    // A weight block goes to LDS in two steps: all loads (four-element groups, WQ per thread at most), later
+    // the writes.  The first block's loads are issued before anything else: they are answered from L2 while
+    // the species permutation, on which the first rows' addresses depend, is still on its way.
+    constexpr int WQ = ROWS_KMAX * (GN / 4) / 512;
+    auto w_issue = [&](const CT* W, int trans, int Kw, int Kp, Vec4<CT> (&w)[WQ]) {
         const int groups = Kp * (GN / 4);
 #pragma unroll
         for (int q = 0; q < WQ; ++q) {
@@ -328,6 +316,9 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
                 }
             }
         }
+    };
+    auto w_store = [&](CT* dst, int trans, int Kp, const Vec4<CT> (&w)[WQ]) {
+        const int groups = Kp * (GN / 4);
 #pragma unroll
         for (int q = 0; q < WQ; ++q) {
             const int v = tid + q * 512;
@@ -344,8 +335,27 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
             }
         }
     };
-    load_w(Wl, pr.W + (size_t)type * pr.w_type_stride + pr.w_off, pr.transW, Kd, Kp1);
-    if (pr.A2) load_w(Wl2, pr.W2 + (size_t)type * pr.w2_type_stride, pr.transW2, pr.Kd2, Kp2);
+    Vec4<CT> wreg[WQ];
+    w_issue(pr.W + (size_t)type * pr.w_type_stride + pr.w_off, pr.transW, Kd, Kp1, wreg);
+
+    // The rows of all tiles of this wavefront go through a private LDS table first (lane group gq fills
+    // tiles gq and gq + 4): inside the tile loop the only vector-memory operations are then the row loads
+    // and the stores, and no small dependent load has to be waited for behind a tile's stores.
+    int2* rows_of = reinterpret_cast<int2*>(smem_raw + (size_t)(Kp1 + Kp2) * SW * sizeof(CT)) + wave * (ROWS_MMAX * 16);
+    for (int jt = gq; jt < m; jt += 4) rows_of[jt * 16 + r] = row_of(row_base + (srow + 4 * jt) * 16 + r);
+    int2 o_cur = rows_of[r];
+    // step u = tile u / S, source u % S
+    auto fetch_step = [&](int2 o, int src, VecN<CT, VL> (&dst)[KJ]) {
+        if (src == 0) fetch(pr.A, a_offset(o), Kd, dst);
+        else fetch(pr.A2, (long)o.x * pr.a2_node_stride, pr.Kd2, dst);
+    };
+    VecN<CT, VL> a[KJ];
+    fetch_step(o_cur, 0, a);
+    w_store(Wl, pr.transW, Kp1, wreg);
+    if (pr.A2) {
+        w_issue(pr.W2 + (size_t)type * pr.w2_type_stride, pr.transW2, pr.Kd2, Kp2, wreg);
+        w_store(Wl2, pr.transW2, Kp2, wreg);
+    }
     __syncthreads();
     if (col0 + t0 * 16 >= Nn) return;                   // this half has no live column
     const int lane_w = gq * VL * SW + t0 * 16 + r;

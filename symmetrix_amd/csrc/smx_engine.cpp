@@ -551,17 +551,21 @@ struct Engine : EngineBase {
         return q;
     }
     // A0[i, l-block] = Phi0[i, l-block] . A0_weights[type_i][l]  (reverse: transposed weights)
-    void st_A0_lin(int N, bool reverse)
+    // `from_M0`: the adjoint product takes M0_grad . M0_adj (one polynomial per channel) as its operand
+    // instead of a stored A0_adj
+    void st_A0_lin(int N, bool reverse, bool from_M0 = false)
     {
         const int k = K();
-        const F* src = reverse ? A0_adj.p : Phi0.p;
+        const F* src = reverse ? (from_M0 ? M0_grad.p : A0_adj.p) : Phi0.p;
         if (reverse) Phi0.size_to((size_t)N * 16 * k, stream); else A0.size_to((size_t)N * 16 * k, stream);
         F* dst = reverse ? Phi0.p : A0.p;
         auto g = gemm_base<F, F, F>(N, true);
         g.nprob = 4;
-        for (int l = 0; l < 4; ++l)
+        for (int l = 0; l < 4; ++l) {
             g.prob[l] = gemm_prob<F, F, F>(src, 16L * k, (long)l * l * k, k, dst, 16L * k, (long)l * l * k, k, A0w.p,
                                            4L * k * k, (long)l * k * k, reverse ? 1 : 0, 0, k, k, 2 * l + 1);
+            if (from_M0) { g.prob[l].Ascale = M0_adj.p; g.prob[l].ascale_node_stride = k; }
+        }
         HIPCHK((launch_gemm<F, F, F>(g, stream)));
     }
     // density normalisation of A0 / A1 and its adjoint; no-ops for models without it (mace.cpp:280, 688)
@@ -649,7 +653,7 @@ struct Engine : EngineBase {
         p.out = Phi1.p;
         HIPCHK(launch_agg_fwd<F>(hm.L_max, p, stream));
     }
-    void st_A1(int N, bool reverse)
+    void st_A1(int N, bool reverse, bool from_M1 = false)
     {
         const int k = K(), ne = NE();
         if (reverse) dPhi1.size_to(Phi1.n, stream); else A1.size_to((size_t)N * 16 * k, stream);
@@ -662,8 +666,11 @@ struct Engine : EngineBase {
                 g.prob[l] = gemm_prob<F, F, F>(Phi1.p, (long)ne * k, lme_off * k, (long)nel * k, A1.p, 16L * k,
                                                (long)l * l * k, k, A1w.p, 0, A1w_off[l], 0, 0, nel * k, k, 2 * l + 1);
             else
-                g.prob[l] = gemm_prob<F, F, F>(A1_adj.p, 16L * k, (long)l * l * k, k, dPhi1.p, (long)ne * k, lme_off * k,
-                                               (long)nel * k, A1w.p, 0, A1w_off[l], 1, 0, k, nel * k, 2 * l + 1);
+            {
+                g.prob[l] = gemm_prob<F, F, F>(from_M1 ? M1_grad.p : A1_adj.p, 16L * k, (long)l * l * k, k, dPhi1.p, (long)ne * k,
+                                               lme_off * k, (long)nel * k, A1w.p, 0, A1w_off[l], 1, 0, k, nel * k, 2 * l + 1);
+                if (from_M1) { g.prob[l].Ascale = M1_adj.p; g.prob[l].ascale_node_stride = k; }
+            }
             lme_off += (2 * l + 1) * nel;
         }
         HIPCHK((launch_gemm<F, F, F>(g, stream)));
@@ -706,6 +713,13 @@ struct Engine : EngineBase {
                                        H1.p, H2.p, H2_adj.p, H1_adj.p, node_energies.p, zero_energies ? 1 : 0,
                                        energies_copy, stream));
         energies_copy = nullptr;
+    }
+    // node counts for which compute() left A1_adj / A0_adj unwritten (-1: they are current)
+    int pending_A1_adj = -1, pending_A0_adj = -1;
+    void materialise_adjoints()
+    {
+        if (pending_A1_adj >= 0) { st_reverse_M1(pending_A1_adj); pending_A1_adj = -1; }
+        if (pending_A0_adj >= 0) { st_reverse_M0(pending_A0_adj); pending_A0_adj = -1; }
     }
     void st_reverse_M1(int N)
     {
@@ -919,15 +933,22 @@ struct Engine : EngineBase {
         stage_begin(ST_H2); st_H2(N1); stage_end(ST_H2);
         stage_begin(ST_READOUT); st_readouts(N1, !hm.has_zbl); stage_end(ST_READOUT);
         stage_begin(ST_REVH2); st_reverse_H2(N1, false); stage_end(ST_REVH2);
-        stage_begin(ST_REVM1); st_reverse_M1(N1); stage_end(ST_REVM1);
+        // Without density normalisation nothing between reverse_M and the adjoint linear reads A_adj: the
+        // linear then forms M_grad . M_adj itself while loading its rows (one polynomial per channel) and
+        // A_adj is only written if somebody asks for it (get_array).
+        const bool fuse1 = !hm.A1_scaled && gemm_scaled_operand_ok(K(), K(), sizeof(F));
+        const bool fuse0 = !hm.A0_scaled && NLM() == 1 && gemm_scaled_operand_ok(K(), K(), sizeof(F));
+        stage_begin(ST_REVM1); if (!fuse1) st_reverse_M1(N1); stage_end(ST_REVM1);
+        pending_A1_adj = fuse1 ? N1 : -1;
         st_scale(1, N1, true);
-        stage_begin(ST_REVA1); st_A1(N1, true); stage_end(ST_REVA1);
+        stage_begin(ST_REVA1); st_A1(N1, true, fuse1); stage_end(ST_REVA1);
         st_agg1_bwd(N1, !early_forces, false);
         if (N1 < N) node_lists_for(N);
         stage_begin(ST_REVH1); st_H1(N, true); stage_end(ST_REVH1);
-        stage_begin(ST_REVM0); st_reverse_M0(N); stage_end(ST_REVM0);
+        stage_begin(ST_REVM0); if (!fuse0) st_reverse_M0(N); stage_end(ST_REVM0);
+        pending_A0_adj = fuse0 ? N : -1;
         st_scale(0, N, true);
-        stage_begin(ST_REVA0LIN); st_A0_lin(N, true); stage_end(ST_REVA0LIN);
+        stage_begin(ST_REVA0LIN); st_A0_lin(N, true, fuse0); stage_end(ST_REVA0LIN);
         st_agg0_bwd(N);
 
         if (energies_copy) HIPCHK(hipMemcpyAsync(energies_copy, node_energies.p, (size_t)N1 * sizeof(double), hipMemcpyDeviceToDevice, stream));
@@ -944,6 +965,7 @@ struct Engine : EngineBase {
     {
         const std::string s(name);
         energies_copy = nullptr; forces_copy = nullptr;
+        materialise_adjoints();
         if (N < 0) throw Error(SMX_EINVAL, "negative num_nodes");
         if (nn && E_ >= 0) edges_from_counts_check(N, nn, E_);
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, false);
@@ -1009,6 +1031,7 @@ struct Engine : EngineBase {
     {
         const std::string s(name);
         hipStream_t st = stream;
+        materialise_adjoints();
         const double* src = nullptr;
         size_t len = 0;
         if (s == "Y" || s == "Y_grad") {
@@ -1051,6 +1074,7 @@ struct Engine : EngineBase {
         const std::string s(name);
         hipStream_t st = stream;
         if (n < 0) throw Error(SMX_EINVAL, "negative length");
+        materialise_adjoints();
         Named v = find(s);
         if ((!v.f && !v.d) || s == "H0_weights" || s == "M0_grad" || s == "M1_grad")
             throw Error(SMX_EINVAL, "array '" + s + "' cannot be set");

@@ -196,6 +196,9 @@ struct GemmProb {
     int Kd, Nn, sub;         // inner size, output columns, rows per node
     // optional second product into the same rows (sub must be 1): row of A2 starts at A2 + node*a2_node_stride
     const TA* A2; long a2_node_stride;
+    // optional per-node factor of the first operand: A[row(node,s)][k] * Ascale[node*ascale_node_stride + k]
+    // (row-streaming kernel only; not together with A2)
+    const TA* Ascale; long ascale_node_stride;
     const CT* W2; long w2_type_stride;
     int transW2, Kd2;
 };
@@ -211,6 +214,8 @@ struct GemmParams {
 };
 template <typename TA, typename TC, typename CT>
 hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p, hipStream_t s);
+// whether a product with inner size Kd, Nn output columns and elements of `elem` bytes can take Ascale
+bool gemm_scaled_operand_ok(int Kd, int Nn, size_t elem);
 
 // ---------------------------------------------------------------------------
 // Readout tail (MACE::compute_readouts, mace.cpp:876-903) in one launch: node_energies[i] (+)= E0[type] +

@@ -14,6 +14,7 @@
 #include "smx_kernels.hpp"
 
 #include <algorithm>
+#include <type_traits>
 
 namespace smx {
 
@@ -227,7 +228,7 @@ constexpr int ROWS_KMAX = 128;
 constexpr int ROWS_MMAX = 8;                     // 16-row tiles per wavefront at most
 constexpr size_t ROWS_OFFS_BYTES = 8 * ROWS_MMAX * 16 * sizeof(int2);
 
-template <typename TA, typename TC, typename CT, int NTW>
+template <typename TA, typename TC, typename CT, int NTW, bool SCALED>
 __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> g, const int m)
 {
     constexpr int VL = rows_vl<CT>(), KG = 4 * VL, KJ = ROWS_KMAX / KG;
@@ -351,6 +352,14 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
     };
     VecN<CT, VL> a[KJ];
     fetch_step(o_cur, 0, a);
+    if constexpr (SCALED) {
+        VecN<CT, VL> sc[KJ];
+        fetch(pr.Ascale, (long)o_cur.x * pr.ascale_node_stride, Kd, sc);
+#pragma unroll
+        for (int jj = 0; jj < KJ; ++jj)
+#pragma unroll
+            for (int q = 0; q < VL; ++q) a[jj].v[q] *= sc[jj].v[q];
+    }
     w_store(Wl, pr.transW, Kp1, wreg);
     if (pr.A2) {
         w_issue(pr.W2 + (size_t)type * pr.w2_type_stride, pr.transW2, pr.Kd2, Kp2, wreg);
@@ -367,8 +376,10 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
         // rows of the next step (past the last one: the last one again, unused)
         const int un = min(u + 1, steps - 1), jn = un / S;
         const int2 o_n = rows_of[jn * 16 + r];
-        VecN<CT, VL> an[KJ];
+        VecN<CT, VL> an[KJ], sn[SCALED ? KJ : 1];
         fetch_step(o_n, un - jn * S, an);
+        // the factor rows stay apart until the hand-over: a product here would wait for both loads
+        if constexpr (SCALED) fetch(pr.Ascale, (long)o_n.x * pr.ascale_node_stride, Kd, sn);
 
         if (src == 0) {
 #pragma unroll
@@ -393,9 +404,12 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
         // them here waits for loads issued a step ago, after the stores it would wait for the stores too.
 #pragma unroll
         for (int jj = 0; jj < KJ; ++jj) {
-            a[jj] = an[jj];
 #pragma unroll
-            for (int q = 0; q < VL; ++q) asm volatile("" : "+v"(a[jj].v[q]));
+            for (int q = 0; q < VL; ++q) {
+                if constexpr (SCALED) a[jj].v[q] = an[jj].v[q] * sn[jj].v[q];
+                else a[jj].v[q] = an[jj].v[q];
+                asm volatile("" : "+v"(a[jj].v[q]));
+            }
         }
         if (src == S - 1) {
             // the offset of output row q is held by lane q
@@ -424,14 +438,14 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
     }
 }
 
-template <typename TA, typename TC, typename CT, int NTW>
+template <typename TA, typename TC, typename CT, int NTW, bool SCALED>
 hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, size_t lds, long total_rows,
                               hipStream_t s)
 {
     constexpr int GN = 32 * NTW;
     static bool attr_done = false;   // per instantiation
     if (!attr_done) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_rows<TA, TC, CT, NTW>),
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_rows<TA, TC, CT, NTW, SCALED>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (err != hipSuccess) return err;
         attr_done = true;
@@ -441,7 +455,7 @@ hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int 
     // rows are resident at once.  Blocks go to the eight dies in turn, whatever they find there, so the
     // count leaves an eighth of the block slots free for an uneven split.
     int per_cu = 1;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemm_rows<TA, TC, CT, NTW>, 512, lds) != hipSuccess || per_cu < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemm_rows<TA, TC, CT, NTW, SCALED>, 512, lds) != hipSuccess || per_cu < 1)
         per_cu = 1;
     const long slots = 224L * per_cu;
     const long slack = p.perm ? std::min<long>((long)p.nprob * p.T, 64) : p.nprob;
@@ -449,7 +463,7 @@ hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int 
     while (m < ROWS_MMAX && (total_rows + 64 * m - 1) / (64 * m) * gy + slack > slots) ++m;
     const long rows = (long)p.num_nodes * max_sub;
     const unsigned gx = (unsigned)((rows + 64 * m - 1) / (64 * m) + (p.perm ? p.T : 0));
-    hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW>), dim3(gx, gy, p.nprob), dim3(512), lds, s, p, (int)m);
+    hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW, SCALED>), dim3(gx, gy, p.nprob), dim3(512), lds, s, p, (int)m);
     return hipGetLastError();
 }
 
@@ -483,6 +497,8 @@ hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p_in, hipStream_t s)
         if (q.A2) vec = vec && mult4(q.Kd2) && mult4(q.a2_node_stride) && mult4(q.w2_type_stride);
     }
     p.vec_ok = vec ? 1 : 0;
+    bool scaled = false;
+    for (int z = 0; z < p.nprob; ++z) scaled = scaled || p.prob[z].Ascale != nullptr;
     // row-streaming kernel: weights of one block resident in LDS
     {
         constexpr int VL = rows_vl<CT>(), KG = 4 * VL;
@@ -490,6 +506,7 @@ hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p_in, hipStream_t s)
         long kp_sum = 0, total_rows = 0;   // padded inner sizes of the widest problem (both products)
         for (int z = 0; z < p.nprob; ++z) {
             const auto& q = p.prob[z];
+            if (scaled) rows_ok = rows_ok && q.Ascale && !q.A2 && mult4(q.ascale_node_stride);
             rows_ok = rows_ok && q.Kd <= ROWS_KMAX && q.Kd % VL == 0;
             long kp = (q.Kd + KG - 1) / KG * KG;
             if (q.A2) {
@@ -508,17 +525,30 @@ hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p_in, hipStream_t s)
             int ntw = (total_rows <= 128 * 64 && max_n % 32 == 0) ? 1 : max_n % 96 == 0 ? 3 : max_n <= 64 ? 2 : 4;
             while (ntw > 1 && lds_for(ntw) > 160 * 1024) --ntw;
             if (ntw == 3 && max_n % 96 != 0) ntw = 2;
+            // the factor rows of the next tile take as many registers as the rows themselves: with them the
+            // widest column block does not fit the register file
+            if (scaled && ntw == 4) ntw = 2;
             const size_t lds = lds_for(ntw);
-            if (lds <= 160 * 1024) {
+            if (lds <= 160 * 1024 && !scaled) {
                 switch (ntw) {
-                case 1: return launch_gemm_rows_t<TA, TC, CT, 1>(p, max_sub, max_n, lds, total_rows, s);
-                case 2: return launch_gemm_rows_t<TA, TC, CT, 2>(p, max_sub, max_n, lds, total_rows, s);
-                case 3: return launch_gemm_rows_t<TA, TC, CT, 3>(p, max_sub, max_n, lds, total_rows, s);
-                default: return launch_gemm_rows_t<TA, TC, CT, 4>(p, max_sub, max_n, lds, total_rows, s);
+                case 1: return launch_gemm_rows_t<TA, TC, CT, 1, false>(p, max_sub, max_n, lds, total_rows, s);
+                case 2: return launch_gemm_rows_t<TA, TC, CT, 2, false>(p, max_sub, max_n, lds, total_rows, s);
+                case 3: return launch_gemm_rows_t<TA, TC, CT, 3, false>(p, max_sub, max_n, lds, total_rows, s);
+                default: return launch_gemm_rows_t<TA, TC, CT, 4, false>(p, max_sub, max_n, lds, total_rows, s);
+                }
+            }
+            if constexpr (std::is_same<TA, CT>::value && std::is_same<TC, CT>::value) {
+                if (lds <= 160 * 1024 && scaled) {
+                    switch (ntw) {
+                    case 1: return launch_gemm_rows_t<TA, TC, CT, 1, true>(p, max_sub, max_n, lds, total_rows, s);
+                    case 2: return launch_gemm_rows_t<TA, TC, CT, 2, true>(p, max_sub, max_n, lds, total_rows, s);
+                    default: return launch_gemm_rows_t<TA, TC, CT, 3, true>(p, max_sub, max_n, lds, total_rows, s);
+                    }
                 }
             }
         }
     }
+    if (scaled) return hipErrorInvalidValue;   // callers check gemm_scaled_operand_ok first
     // tile width: the narrowest of 16, 32, 64, 96, 128 that covers the output, else the least padded of 64, 96, 128
     int nt = 8;
     if (max_n <= 16) nt = 1;
@@ -540,6 +570,11 @@ hipError_t launch_gemm(const GemmParams<TA, TC, CT>& p_in, hipStream_t s)
     case 6: return launch_gemm_t<TA, TC, CT, 6>(p, max_sub, max_n, s);
     default: return launch_gemm_t<TA, TC, CT, 8>(p, max_sub, max_n, s);
     }
+}
+bool gemm_scaled_operand_ok(int Kd, int Nn, size_t elem)
+{
+    const int vl = 32 / (int)elem;
+    return Kd <= ROWS_KMAX && Kd % vl == 0 && Nn >= 32 && Nn % 4 == 0;
 }
 template hipError_t launch_gemm<double, double, double>(const GemmParams<double, double, double>&, hipStream_t);
 template hipError_t launch_gemm<float, float, float>(const GemmParams<float, float, float>&, hipStream_t);

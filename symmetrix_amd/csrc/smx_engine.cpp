@@ -211,7 +211,8 @@ struct Engine : EngineBase {
     // them too and clears the pointer, otherwise a copy is enqueued at the end
     double* energies_copy = nullptr;
     double* forces_copy = nullptr;
-    bool counters_zeroed = false;   // the sender counters were cleared by the fused node-list launch
+    bool senders_counted = false;   // the sender histogram was formed by the fused node-list launch
+    long counters_clean = 0;        // leading entries of s_count known to be zero
 
     // ---- state (mace.hpp members)
     DVec<F> Phi0, A0, A0_adj, M0, M0_grad, M0_adj, H1, H1_adj, Phi1, dPhi1, A1, A1_adj, M1, M1_grad, M1_adj, msg;
@@ -443,8 +444,9 @@ struct Engine : EngineBase {
         s_list.size_to((size_t)E1, s);
         scan_tmp.size_to((size_t)rows / 1024 + 2, s);
         HIPCHK(launch_sender_lists(neigh_indices, (int)E1, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p,
-                                   counters_zeroed ? 1 : 0, s));
-        counters_zeroed = false;
+                                   senders_counted ? 2 : 0, s));
+        senders_counted = false;
+        counters_clean = 2L * rows;   // every build leaves its counters and cursors at zero
         sender_rows = rows;
     }
     // Host-path validation of what the reference leaves unchecked (mace.cpp:17-64 trusts
@@ -883,16 +885,18 @@ struct Engine : EngineBase {
         if (N1 < N) E1 = E_local;
         // range checks come before any kernel that uses these integers as indices
         if (on_device && N <= 65536) {
-            // one launch for first_neigh, degree order, species groups and the cleared sender counters
+            // one launch for first_neigh, degree order, species groups and the sender histogram
             hipStream_t s = stream;
             first_neigh.size_to((size_t)N + 1, s); recv_order.size_to((size_t)N, s);
             t_start.size_to((size_t)hm.T + 1, s); t_perm.size_to((size_t)N, s);
+            const int* before = s_count.p;
             s_count.size_to((size_t)2 * N, s); s_start.size_to((size_t)N + 1, s);
             scan_tmp.size_to((size_t)N / 1024 + 2, s);
-            HIPCHK(launch_node_lists(num_neigh, N, first_neigh.p, recv_order.p, node_types, hm.T, t_start.p, t_perm.p,
-                                     s_count.p, 2L * N, s));
+            if (s_count.p != before || counters_clean < 2L * N) HIPCHK(launch_fill<int>(s_count.p, 2L * N, 0, s));
+            HIPCHK(launch_node_lists_count(num_neigh, N, first_neigh.p, recv_order.p, node_types, hm.T, t_start.p, t_perm.p,
+                                           neigh_indices, E1, N, s_count.p, s));
             N_geo = N;
-            counters_zeroed = true;
+            senders_counted = true;
         } else {
             build_first_neigh(N);
             if (!on_device) validate(N, N);

@@ -3,6 +3,8 @@
 #include "smx_kernels.hpp"
 #include "smx_host_model.hpp"
 
+#include <algorithm>
+
 namespace smx {
 
 // ===========================================================================
@@ -90,10 +92,13 @@ __global__ void k_place(const int* key, long n, int rows, const int* start, int*
 // One wavefront per bucket; entries are distinct, so the rank of an entry is the
 // number of smaller ones: bucket staged in LDS, every lane counts for its entries.
 constexpr int SORT_LDS = 1024;
-__global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows, int* list)
+// The bucket's counter and cursor are dead by now: they are cleared here, so that the next list build
+// finds them at zero without a launch of its own.
+__global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows, int* list, int* count, int* cursor)
 {
     __shared__ int buf[SORT_LDS];
     const int j = blockIdx.x;
+    if (threadIdx.x == 0) { count[j] = 0; cursor[j] = 0; }
     const int s0 = start[j], n = start[j + 1] - s0;
     if (n <= 1) return;
     if (n <= SORT_LDS) {
@@ -242,7 +247,37 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists(const int* num_neigh,
     __syncthreads();
     type_groups_body(node_types, N, T, tstart, perm, sh);
 }
+// The same with the sender histogram in the same launch: block 0 forms the node lists, the other blocks
+// count the senders (counters at zero on entry), which does not depend on the node lists.
+__global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order,
+                                                                const int* node_types, int T, int* tstart, int* perm,
+                                                                const int* key, long n, int rows, int* count)
+{
+    extern __shared__ int sh[];
+    if (blockIdx.x == 0) {
+        scan_single_body(num_neigh, first_neigh, N);
+        __syncthreads();   // first_neigh, written by this block, is read back below
+        degree_order_body(N, first_neigh, order);
+        __syncthreads();
+        type_groups_body(node_types, N, T, tstart, perm, sh);
+        return;
+    }
+    for (long i = (long)(blockIdx.x - 1) * SCAN_BLOCK + threadIdx.x; i < n; i += (long)(gridDim.x - 1) * SCAN_BLOCK) {
+        const int j = key[i];
+        if (j >= 0 && j < rows) atomicAdd(&count[j], 1);
+    }
+}
 }  // namespace
+
+hipError_t launch_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
+                                   int* tstart, int* perm, const int* key, long n, int rows, int* count, hipStream_t s)
+{
+    if (N <= 0 || N > 64 * SCAN_BLOCK || T <= 0) return hipErrorInvalidValue;
+    const unsigned nb = 1 + (unsigned)std::min<long>((n + SCAN_BLOCK - 1) / SCAN_BLOCK, 2048);
+    hipLaunchKernelGGL(k_node_lists_count, dim3(nb), dim3(SCAN_BLOCK), 2 * T * sizeof(int), s, num_neigh, N, first_neigh,
+                       order, node_types, T, tstart, perm, key, n, rows, count);
+    return hipGetLastError();
+}
 
 hipError_t launch_node_lists(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
                              int* tstart, int* perm, int* zero_p, long zero_n, hipStream_t s)
@@ -270,20 +305,21 @@ hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, i
                                int* slist, int* block_sums, int counters_are_zero, hipStream_t s)
 {
     if (rows <= 0) return hipSuccess;
+    const bool counted = counters_are_zero == 2;   // the histogram came with the node lists
     if (counters_are_zero) {
-        // k_node_lists has cleared them
+        // cleared by the previous build (or by k_node_lists)
     } else if (cursor == count + rows) {
         hipLaunchKernelGGL(k_fill<int>, dim3(nblk(2L * rows, 256)), dim3(256), 0, s, count, 2L * rows, 0);
     } else {
         hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, count, (long)rows, 0);
         hipLaunchKernelGGL(k_fill<int>, dim3(nblk(rows, 256)), dim3(256), 0, s, cursor, (long)rows, 0);
     }
-    if (E > 0) hipLaunchKernelGGL(k_count, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, count);
+    if (E > 0 && !counted) hipLaunchKernelGGL(k_count, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, count);
     hipError_t err = launch_scan_exclusive(count, sstart, rows, block_sums, s);
     if (err != hipSuccess) return err;
     if (E > 0) {
         hipLaunchKernelGGL(k_place, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, sstart, cursor, slist);
-        hipLaunchKernelGGL(k_sort_buckets, dim3(rows), dim3(64), 0, s, sstart, rows, slist);
+        hipLaunchKernelGGL(k_sort_buckets, dim3(rows), dim3(64), 0, s, sstart, rows, slist, count, cursor);
     }
     return hipGetLastError();
 }

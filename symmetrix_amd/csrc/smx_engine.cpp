@@ -703,6 +703,26 @@ struct Engine : EngineBase {
         g.prob[1] = gemm_prob<double, F, double>(H2_adj.p, k, 0, 0, M1_adj.p, k, 0, 0, H2w_M1.p, 0, 0, 1, 0, k, k, 1);
         HIPCHK((launch_gemm<double, F, double>(g, stream)));
     }
+    // H2, readouts and reverse_H2 of the full pipeline in one launch (they touch one atom's rows only)
+    void st_tail(int N, bool zero_energies)
+    {
+        const int k = K(), nlm = NLM();
+        need(t_perm.p, "species groups");
+        H2.size_to((size_t)N * k, stream); H2_adj.size_to((size_t)N * k, stream);
+        node_energies.resize((size_t)N, stream);
+        H1_adj.size_to(H1.n, stream); M1_adj.size_to(M1.n, stream);
+        const int rows = (int)(H1.n / ((size_t)nlm * k));
+        if (rows < N || M1.n < (size_t)N * k) throw Error(SMX_EINVAL, "readouts called before H1 and M1 exist for these nodes");
+        TailParams<F> p{};
+        p.N = N; p.rows = rows; p.K = k; p.num_LM = nlm; p.T = hm.T;
+        p.perm = t_perm.p; p.tstart = t_start.p;
+        p.E0 = E0.p; p.w1 = ro1.p; p.W1 = ro2_w1.p; p.w2 = ro2_w2.p; p.scale = hm.readout_2_scale;
+        p.H1 = H1.p; p.M1 = M1.p; p.W_H1 = H2w_H1.p; p.W_M1 = H2w_M1.p;
+        p.H2 = H2.p; p.H2_adj = H2_adj.p; p.H1_adj = H1_adj.p; p.M1_adj = M1_adj.p;
+        p.node_energies = node_energies.p; p.zero_energies = zero_energies ? 1 : 0; p.energies_copy = energies_copy;
+        HIPCHK(launch_tail_fused<F>(p, stream));
+        energies_copy = nullptr;
+    }
     void st_readouts(int N, bool zero_energies)
     {
         const int k = K(), nlm = NLM();
@@ -934,9 +954,15 @@ struct Engine : EngineBase {
         stage_begin(ST_A1); st_A1(N1, false); stage_end(ST_A1);
         st_scale(1, N1, false);
         stage_begin(ST_M1); st_poly(N1, true); stage_end(ST_M1);
-        stage_begin(ST_H2); st_H2(N1); stage_end(ST_H2);
-        stage_begin(ST_READOUT); st_readouts(N1, !hm.has_zbl); stage_end(ST_READOUT);
-        stage_begin(ST_REVH2); st_reverse_H2(N1, false); stage_end(ST_REVH2);
+        if (tail_fused_ok(K())) {
+            stage_begin(ST_H2); st_tail(N1, !hm.has_zbl); stage_end(ST_H2);
+            stage_begin(ST_READOUT); stage_end(ST_READOUT);
+            stage_begin(ST_REVH2); stage_end(ST_REVH2);
+        } else {
+            stage_begin(ST_H2); st_H2(N1); stage_end(ST_H2);
+            stage_begin(ST_READOUT); st_readouts(N1, !hm.has_zbl); stage_end(ST_READOUT);
+            stage_begin(ST_REVH2); st_reverse_H2(N1, false); stage_end(ST_REVH2);
+        }
         // Without density normalisation nothing between reverse_M and the adjoint linear reads A_adj: the
         // linear then forms M_grad . M_adj itself while loading its rows (one polynomial per channel) and
         // A_adj is only written if somebody asks for it (get_array).

@@ -232,6 +232,22 @@ hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* n
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,
                                 const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
                                 double* energies_copy, hipStream_t s);
+// H2 (mace.cpp:820-845), the readout tail and reverse_H2 (mace.cpp:847-874) in one launch; K a multiple of 16
+// up to 128 (tail_fused_ok).  Atoms grouped by species (perm, tstart); H1_adj [rows][num_LM][K] is written
+// whole (seed plus the adjoint of H2 in the scalar block, zero elsewhere), M1_adj [N][K] too.
+template <typename F>
+struct TailParams {
+    int N, rows, K, num_LM, T;
+    const int* perm; const int* tstart;
+    const double* E0; const double* w1; const double* W1; const double* w2; double scale;
+    const F* H1; const F* M1;
+    const double* W_H1;      // [T][K][K]
+    const double* W_M1;      // [K][K]
+    double* H2; double* H2_adj; F* H1_adj; F* M1_adj;
+    double* node_energies; int zero_energies; double* energies_copy;
+};
+bool tail_fused_ok(int K);
+template <typename F> hipError_t launch_tail_fused(const TailParams<F>& p, hipStream_t s);
 template <typename T> hipError_t launch_fill(T* p, long n, T v, hipStream_t s);
 template <typename TS, typename TD> hipError_t launch_convert(const TS* src, TD* dst, long n, hipStream_t s);
 

@@ -649,6 +649,193 @@ __global__ __launch_bounds__(256) void k_readout_fused(int N, int rows, int K, i
 }
 }  // namespace
 
+// ---------------------------------------------------------------------------
+// H2, the readout tail above and reverse_H2 in one launch (mace.cpp:820-903).  All three work on one atom's
+// rows only.  A block takes 16 atoms of one species (species groups of the list preparation) through:
+//   H2 = H1[l=0] . W_H1[type] + M1 . W_M1 on the matrix cores (operands from LDS, weights straight from
+//   L2 in the operand layout: a 16-lane group reads 16 consecutive columns of one weight row),
+//   the K -> 16 -> 1 network with its gradient H2_adj, energies, the seed of H1_adj,
+//   H1_adj[l=0] += H2_adj . W_H1[type]^T and M1_adj = H2_adj . W_M1^T (a lane reads 32 consecutive bytes of
+//   its weight row; k is permuted inside groups of 16 on both operands).
+// Sums over k run in one fixed order per output element, independent of the atom's tile mates.
+namespace {
+typedef double f64x4 __attribute__((ext_vector_type(4)));
+constexpr int TAIL_BLOCK = 512;   // eight wavefronts: wavefront w owns column tile w of both products
+template <typename F, int KT>
+__global__ __launch_bounds__(TAIL_BLOCK) void k_tail_fused(const TailParams<F> p)
+{
+    extern __shared__ double tsm[];
+    constexpr int K = 16 * KT, ld = K + 1;   // padded rows: a column read by 16 rows hits 16 banks
+    double* W1s = tsm;                       // [16][ld]
+    double* hg = W1s + 16 * ld;              // [16 atoms][16 hidden]
+    double* XA = hg + 256;                   // [16][ld] H1[l=0] rows
+    double* XB = XA + 16 * ld;               // [16][ld] M1 rows
+    double* XH = XB + 16 * ld;               // [16][ld] H2 rows
+    double* XY = XH + 16 * ld;               // [16][ld] H2_adj rows
+    __shared__ int node_s[16];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int width = p.num_LM * K;
+    // rows beyond the atoms (ghost rows of H1_adj) are cleared by all blocks together
+    {
+        const long ghost = (long)(p.rows - p.N) * width;
+        for (long t = (long)blockIdx.x * TAIL_BLOCK + tid; t < ghost; t += (long)gridDim.x * TAIL_BLOCK)
+            p.H1_adj[(size_t)p.N * width + t] = F(0);
+    }
+    // species segment and tile of this block
+    int type = -1, tile = blockIdx.x, seg0 = 0, seg_n = 0;
+    for (int t = 0; t < p.T; ++t) {
+        const int n_t = p.tstart[t + 1] - p.tstart[t];
+        const int tiles = (n_t + 15) / 16;
+        if (tile < tiles) { type = t; seg0 = p.tstart[t]; seg_n = n_t; break; }
+        tile -= tiles;
+    }
+    if (type < 0) return;
+    const int r = lane & 15, g = lane >> 4;
+    const double* WH = p.W_H1 + (size_t)type * K * K;
+    const bool owner = wave < KT;            // this wavefront owns column tile `wave`
+    // the weights of the first product pair are requested before anything else: they do not depend on the atoms
+    double b1[K / 4], b2[K / 4];
+    if (owner) {
+#pragma unroll
+        for (int q = 0; q < K / 4; ++q) {
+            b1[q] = WH[(size_t)(4 * q + g) * K + wave * 16 + r];
+            b2[q] = p.W_M1[(size_t)(4 * q + g) * K + wave * 16 + r];
+        }
+    }
+    if (tid < 16) node_s[tid] = tile * 16 + tid < seg_n ? p.perm[seg0 + tile * 16 + tid] : -1;
+    __syncthreads();
+    for (int t = tid; t < 16 * K; t += TAIL_BLOCK) {
+        const int rr = t / K, k = t - rr * K;
+        W1s[rr * ld + k] = p.W1[t];
+        const int nd = node_s[rr];
+        XA[rr * ld + k] = nd >= 0 ? (double)p.H1[(size_t)nd * width + k] : 0.0;
+        XB[rr * ld + k] = nd >= 0 ? (double)p.M1[(size_t)nd * K + k] : 0.0;
+    }
+    __syncthreads();
+    // ---- H2 tile
+    f64x4 w1v[KT], w2v[KT];                   // weights of the transposed products, requested early as well
+    if (owner) {
+        f64x4 acc1 = {0, 0, 0, 0}, acc2 = {0, 0, 0, 0};
+#pragma unroll
+        for (int q = 0; q < K / 4; ++q) {
+            acc1 = __builtin_amdgcn_mfma_f64_16x16x4f64(XA[r * ld + 4 * q + g], b1[q], acc1, 0, 0, 0);
+            acc2 = __builtin_amdgcn_mfma_f64_16x16x4f64(XB[r * ld + 4 * q + g], b2[q], acc2, 0, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < KT; ++j) {
+            w1v[j] = *reinterpret_cast<const f64x4*>(WH + (size_t)(wave * 16 + r) * K + 16 * j + 4 * g);
+            w2v[j] = *reinterpret_cast<const f64x4*>(p.W_M1 + (size_t)(wave * 16 + r) * K + 16 * j + 4 * g);
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int row = 4 * q + g, col = wave * 16 + r;
+            const double v = acc1[q] + acc2[q];
+            XH[row * ld + col] = v;
+            const int nd = node_s[row];
+            if (nd >= 0) p.H2[(size_t)nd * K + col] = v;
+        }
+    }
+    __syncthreads();
+    // ---- readout network, energies (thread = atom n, hidden unit h)
+    if (tid < 256) {
+        const int n = tid >> 4, h = tid & 15;
+        const int i = node_s[n];
+        double e = 0.0, gr = 0.0;
+        if (i >= 0) {
+            const double* h2 = XH + n * ld;
+            double sdot = 0.0;
+#pragma unroll 8
+            for (int k = 0; k < K; ++k) sdot += W1s[h * ld + k] * h2[k];
+            // multilayer_perceptron.cpp:107-113: scaled SiLU and its derivative
+            const double sig = 1.0 / (1.0 + exp(-sdot));
+            e = p.w2[h] * (p.scale * sdot * sig);
+            gr = p.w2[h] * (p.scale * sig + p.scale * sdot * sig * (1 - sig));
+            for (int k = h; k < K; k += 16) e += p.w1[k] * XA[n * ld + k];
+        }
+#pragma unroll
+        for (int off = 8; off >= 1; off >>= 1) e += __shfl_xor(e, off, 64);
+        hg[tid] = gr;
+        if (h == 0 && i >= 0) {
+            const double en = (p.zero_energies ? 0.0 : p.node_energies[i]) + p.E0[type] + e;
+            p.node_energies[i] = en;
+            if (p.energies_copy) p.energies_copy[i] = en;
+        }
+    }
+    __syncthreads();
+    // ---- H2_adj tile
+    for (int t = tid; t < 16 * K; t += TAIL_BLOCK) {
+        const int n2 = t / K, k = t - n2 * K;
+        double sum = 0.0;
+#pragma unroll
+        for (int q = 0; q < 16; ++q) sum += hg[n2 * 16 + q] * W1s[q * ld + k];
+        XY[n2 * ld + k] = sum;
+        const int nd = node_s[n2];
+        if (nd >= 0) p.H2_adj[(size_t)nd * K + k] = sum;
+    }
+    __syncthreads();
+    // ---- H1_adj[l=0] = w1 + H2_adj . W_H1^T, M1_adj = H2_adj . W_M1^T
+    if (owner) {
+        f64x4 acc1 = {0, 0, 0, 0}, acc2 = {0, 0, 0, 0};
+        const double* a = XY + r * ld + 4 * g;
+#pragma unroll
+        for (int j = 0; j < KT; ++j) {
+#pragma unroll
+            for (int t = 0; t < 4; ++t) {
+                acc1 = __builtin_amdgcn_mfma_f64_16x16x4f64(a[16 * j + t], w1v[j][t], acc1, 0, 0, 0);
+                acc2 = __builtin_amdgcn_mfma_f64_16x16x4f64(a[16 * j + t], w2v[j][t], acc2, 0, 0, 0);
+            }
+        }
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int nd = node_s[4 * q + g], col = wave * 16 + r;
+            if (nd >= 0) {
+                p.H1_adj[(size_t)nd * width + col] = (F)((double)(F)p.w1[col] + acc1[q]);
+                p.M1_adj[(size_t)nd * K + col] = (F)acc2[q];
+            }
+        }
+    }
+    // the other blocks of H1_adj start at zero
+    for (int t = tid; t < 16 * (width - K); t += TAIL_BLOCK) {
+        const int n2 = t / (width - K), c = K + t - n2 * (width - K);
+        const int nd = node_s[n2];
+        if (nd >= 0) p.H1_adj[(size_t)nd * width + c] = F(0);
+    }
+}
+}  // namespace
+
+template <typename F>
+size_t tail_fused_lds(int K) { return ((size_t)5 * 16 * (K + 1) + 256) * sizeof(double); }
+bool tail_fused_ok(int K) { return K == 32 || K == 48 || K == 64 || K == 96 || K == 128; }
+
+template <typename F, int KT>
+static hipError_t launch_tail_fused_t(const TailParams<F>& p, hipStream_t s)
+{
+    const size_t lds = tail_fused_lds<F>(p.K);
+    if (lds > 64 * 1024) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_tail_fused<F, KT>),
+                                             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+    }
+    const unsigned blocks = (unsigned)((p.N + 15) / 16 + p.T);
+    hipLaunchKernelGGL((k_tail_fused<F, KT>), dim3(blocks), dim3(TAIL_BLOCK), lds, s, p);
+    return hipGetLastError();
+}
+template <typename F>
+hipError_t launch_tail_fused(const TailParams<F>& p, hipStream_t s)
+{
+    if (p.rows < p.N || !tail_fused_ok(p.K) || p.T <= 0) return hipErrorInvalidValue;
+    if (p.rows <= 0) return hipSuccess;
+    switch (p.K / 16) {
+    case 2: return launch_tail_fused_t<F, 2>(p, s);
+    case 3: return launch_tail_fused_t<F, 3>(p, s);
+    case 4: return launch_tail_fused_t<F, 4>(p, s);
+    case 6: return launch_tail_fused_t<F, 6>(p, s);
+    default: return launch_tail_fused_t<F, 8>(p, s);
+    }
+}
+template hipError_t launch_tail_fused<double>(const TailParams<double>&, hipStream_t);
+template hipError_t launch_tail_fused<float>(const TailParams<float>&, hipStream_t);
+
 template <typename F>
 hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,

@@ -786,9 +786,19 @@ struct Engine : EngineBase {
         }
         stage_begin(ST_SRED);
         if (sender_rows != rows) build_sender_lists(rows);
-        HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, 0, E1, stream));
+        if (fuse_reverse_H1 && nlm == 1 && sender_reduce_linear_ok(k) && M0.n == (size_t)rows * k) {
+            // scalar hidden features: reverse_H1 of the summed rows in the same launch
+            M0_adj.size_to(M0.n, stream);
+            HIPCHK(launch_sender_reduce_linear<F>(rows, k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, H1w.p,
+                                                  M0_adj.p, stream));
+            reverse_H1_done = true;
+        } else {
+            HIPCHK(launch_sender_reduce<F>(rows, nlm * k, s_start.p, s_list.p, msg.p, H1_adj.p, zero_H1_adj ? 1 : 0, 0, E1, stream));
+        }
         stage_end(ST_SRED);
     }
+    bool fuse_reverse_H1 = false;   // compute() wants reverse_H1 folded into the sender-side sum
+    bool reverse_H1_done = false;   // ... and the stage did it
     // The same stage for edge lists whose messages do not fit the staging buffer: receivers are taken in
     // chunks, each chunk's messages are added to the sender rows before the next chunk overwrites them.  Every
     // sender still receives its messages in ascending edge order, so the result does not depend on the chunking.
@@ -972,9 +982,11 @@ struct Engine : EngineBase {
         pending_A1_adj = fuse1 ? N1 : -1;
         st_scale(1, N1, true);
         stage_begin(ST_REVA1); st_A1(N1, true, fuse1); stage_end(ST_REVA1);
+        fuse_reverse_H1 = N1 == N; reverse_H1_done = false;
         st_agg1_bwd(N1, !early_forces, false);
+        fuse_reverse_H1 = false;
         if (N1 < N) node_lists_for(N);
-        stage_begin(ST_REVH1); st_H1(N, true); stage_end(ST_REVH1);
+        stage_begin(ST_REVH1); if (!reverse_H1_done) st_H1(N, true); stage_end(ST_REVH1);
         stage_begin(ST_REVM0); if (!fuse0) st_reverse_M0(N); stage_end(ST_REVM0);
         pending_A0_adj = fuse0 ? N : -1;
         st_scale(0, N, true);

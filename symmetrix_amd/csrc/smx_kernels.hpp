@@ -89,6 +89,12 @@ hipError_t launch_fpart_reduce(long edges, long E, int nslices, const double* fp
 template <typename F>
 hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const int* slist, const F* msg, F* H_adj,
                                 int zero_first, long e_lo, long e_hi, hipStream_t s);
+// The same sum for rows of K scalar features, followed by M_adj[rows][K] = H_adj . W^T (W [K][K], row n holding
+// the weights of input channel n: reverse_H1 of an L_max = 0 model) in the same launch; K as sender_reduce_linear_ok
+bool sender_reduce_linear_ok(int K);
+template <typename F>
+hipError_t launch_sender_reduce_linear(int rows, int K, const int* sstart, const int* slist, const F* msg, F* H_adj,
+                                       int zero_first, const F* W, F* M_adj, hipStream_t s);
 
 // ---------------------------------------------------------------------------
 // Neighbour list on the device (smx_kernels_nlist.hip)

@@ -714,6 +714,103 @@ hipError_t launch_sender_reduce(int rows, int width, const int* sstart, const in
     }
     return hipGetLastError();
 }
+// ---------------------------------------------------------------------------
+// The sender-side sum followed by reverse_H1 for scalar hidden features (mace.cpp:402-436 with one block of
+// H1): a block of 16 wavefronts sums the messages of 16 consecutive sender rows (wavefront w takes row w, in
+// ascending edge order as above), keeps the finished rows in LDS as doubles, and forms
+// M0_adj = H1_adj . W^T for them on the matrix cores; wavefront w owns column tile w, its weight operands
+// (32 contiguous bytes per lane, k permuted inside groups of 16 on both operands) are requested before the
+// sums start.
+namespace {
+typedef double f64x4_t __attribute__((ext_vector_type(4)));
+template <typename F, int KT>
+__global__ __launch_bounds__(1024) void k_sender_reduce_linear(int rows, const int* sstart, const int* slist, const F* msg,
+                                                              F* H_adj, int zero_first, const F* W, F* M_adj)
+{
+    constexpr int K = 16 * KT, ld = K + 1, V = 16 / (int)sizeof(F);
+    __shared__ double X[16 * ld];
+    const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int r = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.x * 16;
+    const bool owner = wave < KT;
+    f64x4_t wv[KT];
+    if (owner) {
+#pragma unroll
+        for (int j = 0; j < KT; ++j) {
+            const Vec<F, 4> t = ldv<F, 4>(W + (size_t)(wave * 16 + r) * K + 16 * j + 4 * g);
+#pragma unroll
+            for (int c = 0; c < 4; ++c) wv[j][c] = (double)t.v[c];
+        }
+    }
+    {
+        const int rr = wave, j = row0 + rr;
+        const int q = lane * V;
+        if (q < K) {
+            Vec<F, V> acc;
+#pragma unroll
+            for (int c = 0; c < V; ++c) acc.v[c] = F(0);
+            if (j < rows) {
+                const int s0 = sstart[j], s1 = sstart[j + 1];
+                if (!zero_first) acc = ldv<F, V>(H_adj + (size_t)j * K + q);
+                int t = s0;
+                for (; t + 4 <= s1; t += 4) {
+                    Vec<F, V> m[4];
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) m[i] = ldv<F, V>(msg + (size_t)slist[t + i] * K + q);
+#pragma unroll
+                    for (int i = 0; i < 4; ++i)
+#pragma unroll
+                        for (int c = 0; c < V; ++c) acc.v[c] += m[i].v[c];
+                }
+                for (; t < s1; ++t) {
+                    const Vec<F, V> m = ldv<F, V>(msg + (size_t)slist[t] * K + q);
+#pragma unroll
+                    for (int c = 0; c < V; ++c) acc.v[c] += m.v[c];
+                }
+                *reinterpret_cast<Vec<F, V>*>(H_adj + (size_t)j * K + q) = acc;
+            }
+#pragma unroll
+            for (int c = 0; c < V; ++c) X[rr * ld + q + c] = (double)acc.v[c];
+        }
+    }
+    __syncthreads();
+    if (owner) {
+        f64x4_t acc = {0, 0, 0, 0};
+        const double* a = X + r * ld + 4 * g;
+#pragma unroll
+        for (int j = 0; j < KT; ++j)
+#pragma unroll
+            for (int t = 0; t < 4; ++t) acc = __builtin_amdgcn_mfma_f64_16x16x4f64(a[16 * j + t], wv[j][t], acc, 0, 0, 0);
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+            const int j = row0 + 4 * q + g;
+            if (j < rows) M_adj[(size_t)j * K + wave * 16 + r] = (F)acc[q];
+        }
+    }
+}
+}  // namespace
+
+bool sender_reduce_linear_ok(int K) { return K == 32 || K == 48 || K == 64 || K == 96 || K == 128; }
+
+template <typename F>
+hipError_t launch_sender_reduce_linear(int rows, int K, const int* sstart, const int* slist, const F* msg, F* H_adj,
+                                       int zero_first, const F* W, F* M_adj, hipStream_t s)
+{
+    if (!sender_reduce_linear_ok(K)) return hipErrorInvalidValue;
+    if (rows <= 0) return hipSuccess;
+    const dim3 grid((unsigned)((rows + 15) / 16)), block(1024);
+    switch (K / 16) {
+    case 2: hipLaunchKernelGGL((k_sender_reduce_linear<F, 2>), grid, block, 0, s, rows, sstart, slist, msg, H_adj, zero_first, W, M_adj); break;
+    case 3: hipLaunchKernelGGL((k_sender_reduce_linear<F, 3>), grid, block, 0, s, rows, sstart, slist, msg, H_adj, zero_first, W, M_adj); break;
+    case 4: hipLaunchKernelGGL((k_sender_reduce_linear<F, 4>), grid, block, 0, s, rows, sstart, slist, msg, H_adj, zero_first, W, M_adj); break;
+    case 6: hipLaunchKernelGGL((k_sender_reduce_linear<F, 6>), grid, block, 0, s, rows, sstart, slist, msg, H_adj, zero_first, W, M_adj); break;
+    default: hipLaunchKernelGGL((k_sender_reduce_linear<F, 8>), grid, block, 0, s, rows, sstart, slist, msg, H_adj, zero_first, W, M_adj); break;
+    }
+    return hipGetLastError();
+}
+template hipError_t launch_sender_reduce_linear<double>(int, int, const int*, const int*, const double*, double*, int, const double*, double*, hipStream_t);
+template hipError_t launch_sender_reduce_linear<float>(int, int, const int*, const int*, const float*, float*, int, const float*, float*, hipStream_t);
+
 template hipError_t launch_sender_reduce<double>(int, int, const int*, const int*, const double*, double*, int, long, long, hipStream_t);
 template hipError_t launch_sender_reduce<float>(int, int, const int*, const int*, const float*, float*, int, long, long, hipStream_t);
 

@@ -34,7 +34,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 STAGE_KERNEL = {
     "agg0_fwd": ("k_slice_fwd", "k_slice_fwd"), "agg1_fwd": ("k_slice_fwd", "k_agg_fwd"),
     "agg1_bwd": ("k_slice_bwd", "k_agg_bwd"), "agg0_bwd": ("k_slice_bwd", "k_slice_bwd"),
-    "sender_reduce": ("k_sender_reduce", "k_sender_reduce"),
+    "sender_reduce": ("k_sender_reduce_linear", "k_sender_reduce"),
 }
 
 # HBM bytes per launch from rocprofv3 counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the factors read off a
@@ -42,9 +42,9 @@ STAGE_KERNEL = {
 # profiles/edge_kernels_mp_medium_hbm_traffic.txt
 MEASURED_TRAFFIC = {
     ("off_small", "float64"): {"agg0_fwd": 78.8e6, "agg1_fwd": 106.2e6, "agg1_bwd": 436.0e6, "agg0_bwd": 257.9e6,
-                               "sender_reduce": 93.6e6},
+                               "sender_reduce": 95.7e6},
     ("off_small", "float32"): {"agg0_fwd": 58.8e6, "agg1_fwd": 86.2e6, "agg1_bwd": 247.3e6, "agg0_bwd": 151.8e6,
-                               "sender_reduce": 47.7e6},
+                               "sender_reduce": 48.3e6},
     ("mp_medium", "float32"): {"agg0_fwd": 1733.4e6, "agg1_fwd": 4609.0e6, "agg1_bwd": 16226.3e6, "agg0_bwd": 4490.6e6,
                                "sender_reduce": 8257.2e6},
     ("mp_medium", "float64"): {"agg0_fwd": 2291.3e6, "agg1_fwd": 20204.2e6, "agg1_bwd": 45819.8e6, "agg0_bwd": 7626.9e6,

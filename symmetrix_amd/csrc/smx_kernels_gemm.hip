@@ -235,12 +235,27 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
     constexpr int GN = 32 * NTW, SW = rows_sw<CT, NTW>();
     extern __shared__ __align__(16) unsigned char smem_raw[];
     CT* Wl = reinterpret_cast<CT*>(smem_raw);          // [Kp][SW], rows Kd..Kp-1 zero
-    const GemmProb<TA, TC, CT>& pr = g.prob[blockIdx.z];
-    const int Nn = pr.Nn, Kd = pr.Kd, sub = pr.sub;
-    const int col0 = blockIdx.y * GN;
-    if (col0 >= Nn) return;
     const int chunk_rows = 64 * m;
-    int type = 0, chunk = blockIdx.x, nrows_seg = g.num_nodes * sub, seg_node0 = 0;
+    // Products whose weights do not depend on the species come as a one-dimensional grid of exactly the blocks
+    // that have rows, numbered problem by problem: consecutive blocks go to the dies in turn, so the dies get
+    // equal shares.  (With species segments the host cannot count the blocks: three-dimensional grid, blocks
+    // without rows leave at once.)
+    int z = blockIdx.z, chunk = blockIdx.x, cb = blockIdx.y;
+    if (!g.perm) {
+        int b = blockIdx.x;
+        for (z = 0; z < g.nprob; ++z) {
+            const int chunks = (g.num_nodes * g.prob[z].sub + chunk_rows - 1) / chunk_rows;
+            const int cols = (g.prob[z].Nn + GN - 1) / GN;
+            if (b < chunks * cols) { chunk = b / cols; cb = b - chunk * cols; break; }
+            b -= chunks * cols;
+        }
+        if (z == g.nprob) return;
+    }
+    const GemmProb<TA, TC, CT>& pr = g.prob[z];
+    const int Nn = pr.Nn, Kd = pr.Kd, sub = pr.sub;
+    const int col0 = cb * GN;
+    if (col0 >= Nn) return;
+    int type = 0, nrows_seg = g.num_nodes * sub, seg_node0 = 0;
     if (g.perm) {
         bool found = false;
         for (int t = 0; t < g.T; ++t) {
@@ -457,12 +472,25 @@ hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int 
     int per_cu = 1;
     if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemm_rows<TA, TC, CT, NTW, SCALED>, 512, lds) != hipSuccess || per_cu < 1)
         per_cu = 1;
+    if (!p.perm) {
+        // exact block count: every slot can be used
+        auto blocks_for = [&](long mm) {
+            long b = 0;
+            for (int z = 0; z < p.nprob; ++z)
+                b += ((long)p.num_nodes * p.prob[z].sub + 64 * mm - 1) / (64 * mm) * ((p.prob[z].Nn + GN - 1) / GN);
+            return b;
+        };
+        long m = 1;
+        while (m < ROWS_MMAX && blocks_for(m) > 256L * per_cu) ++m;
+        hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW, SCALED>), dim3((unsigned)blocks_for(m)), dim3(512), lds, s, p, (int)m);
+        return hipGetLastError();
+    }
     const long slots = 224L * per_cu;
-    const long slack = p.perm ? std::min<long>((long)p.nprob * p.T, 64) : p.nprob;
+    const long slack = std::min<long>((long)p.nprob * p.T, 64);
     long m = 1;
     while (m < ROWS_MMAX && (total_rows + 64 * m - 1) / (64 * m) * gy + slack > slots) ++m;
     const long rows = (long)p.num_nodes * max_sub;
-    const unsigned gx = (unsigned)((rows + 64 * m - 1) / (64 * m) + (p.perm ? p.T : 0));
+    const unsigned gx = (unsigned)((rows + 64 * m - 1) / (64 * m) + p.T);
     hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW, SCALED>), dim3(gx, gy, p.nprob), dim3(512), lds, s, p, (int)m);
     return hipGetLastError();
 }

@@ -451,59 +451,60 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
         F f[NB], g[NB];
 #pragma unroll
         for (int b = 0; b < NB; ++b) f[b] = g[b] = F(0);
-        // this group's chunks are contiguous: [c, c_end)
+        // this group's chunks are contiguous and start at c
         int c = 0;
         for (int q = 0; q < 2 * VPG * vg; ++q) c += nch[q];
-        int c_end = c;
-        for (int q = 0; q < 2 * VPG; ++q) c_end += nch[2 * VPG * vg + q];
-        int t = 0, v = vg, done = 0;
-        int n0 = nch[2 * VPG * vg], n1 = nch[2 * VPG * vg + 1];
-        // a finished variable (possibly one without entries) stores its gradient and hands over to the next
-        auto flush = [&]() {
-            while (t < VPG && done == n0 + n1) {
-#pragma unroll
-                for (int b = 0; b < NB; ++b) {
-                    if (klive && nlive[b]) a.M_grad[(((size_t)node[b] * a.NP + pl) * 16 + v) * a.K + k] = g[b];
-                    g[b] = F(0);
-                }
-                ++t; v += POLY_VG; done = 0;
-                if (t < VPG) { n0 = nch[2 * (VPG * vg + t)]; n1 = nch[2 * (VPG * vg + t) + 1]; }
-            }
-        };
         auto weights = [&](const int4& e, F (&w)[4]) {
             const int e4[4] = {e.x, e.y, e.z, e.w};
 #pragma unroll
             for (int q = 0; q < 4; ++q) w[q] = (coef + (size_t)(e4[q] & 0xffff) * a.K)[kk];
         };
-        flush();
-        // indices two chunks ahead and coefficients one chunk ahead of the arithmetic; the list ends with
-        // spare chunks of padding entries, so nothing here depends on where the group's range stops
+        // indices two chunks ahead and coefficients one chunk ahead of the arithmetic, across the variables
+        // of the group; the list ends with spare chunks of padding entries, so nothing here depends on where
+        // the group's range stops
         int4 cur = pk(c), nxt = pk(c + 1);
         F w[4];
         weights(cur, w);
-        for (; c < c_end; ++c) {
-            F wn[4];
-            weights(nxt, wn);
-            const int4 nn = pk(c + 2);
-            const int e4[4] = {cur.x, cur.y, cur.z, cur.w};
+        // The gradients of the group's variables stay in registers until all lists are walked: a store between
+        // the lists would sit in front of the next coefficient loads, whose wait would then wait for it too.
+        F gs[VPG][NB];
 #pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                const int ia = (e4[q] >> 16) & 0xff, ib = (e4[q] >> 24) & 0xff;
-                const PolyVec<F, NB> xa = X[ia][tid], xb = X[ib][tid];
+        for (int t = 0; t < VPG; ++t) {
+            const int v = vg + POLY_VG * t;
+            const int n0 = nch[2 * (VPG * vg + t)], n1 = nch[2 * (VPG * vg + t) + 1];
 #pragma unroll
-                for (int b = 0; b < NB; ++b) g[b] += w[q] * (xa.v[b] * xb.v[b]);
+            for (int b = 0; b < NB; ++b) g[b] = F(0);
+            for (int i = 0; i < n0 + n1; ++i, ++c) {
+                F wn[4];
+                weights(nxt, wn);
+                const int4 nn = pk(c + 2);
+                const int e4[4] = {cur.x, cur.y, cur.z, cur.w};
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const int ia = (e4[q] >> 16) & 0xff, ib = (e4[q] >> 24) & 0xff;
+                    const PolyVec<F, NB> xa = X[ia][tid], xb = X[ib][tid];
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) g[b] += w[q] * (xa.v[b] * xb.v[b]);
+                }
+                cur = nxt; nxt = nn;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) w[q] = wn[q];
+                if (i + 1 == n0) {
+                    // the monomials that start with v are done: their sum times x_v is v's share of P
+                    const PolyVec<F, NB> xv = X[v][tid];
+#pragma unroll
+                    for (int b = 0; b < NB; ++b) f[b] += xv.v[b] * g[b];
+                }
             }
-            cur = nxt; nxt = nn;
 #pragma unroll
-            for (int q = 0; q < 4; ++q) w[q] = wn[q];
-            if (++done == n0) {
-                // the monomials that start with v are done: their sum times x_v is v's share of P
-                const PolyVec<F, NB> xv = X[v][tid];
-#pragma unroll
-                for (int b = 0; b < NB; ++b) f[b] += xv.v[b] * g[b];
-            }
-            flush();
+            for (int b = 0; b < NB; ++b) gs[t][b] = g[b];
         }
+#pragma unroll
+        for (int t = 0; t < VPG; ++t)
+#pragma unroll
+            for (int b = 0; b < NB; ++b)
+                if (klive && nlive[b])
+                    a.M_grad[(((size_t)node[b] * a.NP + pl) * 16 + vg + POLY_VG * t) * a.K + k] = gs[t][b];
         // P = sum of the groups' shares, added in group order
         {
             PolyVec<F, NB> fv;

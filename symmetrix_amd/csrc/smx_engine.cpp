@@ -211,7 +211,8 @@ struct Engine : EngineBase {
     // them too and clears the pointer, otherwise a copy is enqueued at the end
     double* energies_copy = nullptr;
     double* forces_copy = nullptr;
-    bool senders_counted = false;   // the sender histogram was formed by the fused node-list launch
+    bool senders_counted = false;   // the sender histogram (and s_rank) was formed by the fused node-list launch
+    DVec<int> s_rank;               // place of every edge inside its sender's bucket
     long counters_clean = 0;        // leading entries of s_count known to be zero
 
     // ---- state (mace.hpp members)
@@ -444,7 +445,7 @@ struct Engine : EngineBase {
         s_list.size_to((size_t)E1, s);
         scan_tmp.size_to((size_t)rows / 1024 + 2, s);
         HIPCHK(launch_sender_lists(neigh_indices, (int)E1, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p,
-                                   senders_counted ? 2 : 0, s));
+                                   senders_counted ? 2 : 0, senders_counted ? s_rank.p : nullptr, s));
         senders_counted = false;
         counters_clean = 2L * rows;   // every build leaves its counters and cursors at zero
         sender_rows = rows;
@@ -923,8 +924,9 @@ struct Engine : EngineBase {
             s_count.size_to((size_t)2 * N, s); s_start.size_to((size_t)N + 1, s);
             scan_tmp.size_to((size_t)N / 1024 + 2, s);
             if (s_count.p != before || counters_clean < 2L * N) HIPCHK(launch_fill<int>(s_count.p, 2L * N, 0, s));
+            s_rank.size_to((size_t)E1, s);
             HIPCHK(launch_node_lists_count(num_neigh, N, first_neigh.p, recv_order.p, node_types, hm.T, t_start.p, t_perm.p,
-                                           neigh_indices, E1, N, s_count.p, s));
+                                           neigh_indices, E1, N, s_count.p, s_rank.p, s));
             N_geo = N;
             senders_counted = true;
         } else {
@@ -1170,7 +1172,7 @@ struct Engine : EngineBase {
                 rf_recv.upload(hr.data(), hr.size(), s);
                 HIPCHK(hipStreamSynchronize(s));
                 rf_rstart.size_to((size_t)num_atoms + 1, s); rf_rlist.size_to((size_t)E, s);
-                HIPCHK(launch_sender_lists(rf_recv.p, (int)E, num_atoms, rf_count.p, rf_rstart.p, rf_cursor.p, rf_rlist.p, scan_tmp.p, 0, s));
+                HIPCHK(launch_sender_lists(rf_recv.p, (int)E, num_atoms, rf_count.p, rf_rstart.p, rf_cursor.p, rf_rlist.p, scan_tmp.p, 0, nullptr, s));
                 rstart = rf_rstart.p; rlist = rf_rlist.p;
             } else {
                 if (num_atoms < N_geo) throw Error(SMX_EINVAL, "num_atoms is smaller than the number of receivers");
@@ -1183,7 +1185,7 @@ struct Engine : EngineBase {
                 HIPCHK(hipStreamSynchronize(s));
                 rstart = rf_rstart.p;
             }
-            HIPCHK(launch_sender_lists(send, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, 0, s));
+            HIPCHK(launch_sender_lists(send, (int)E, num_atoms, rf_count.p, rf_sstart.p, rf_cursor.p, rf_slist.p, scan_tmp.p, 0, nullptr, s));
             rf_out.size_to((size_t)3 * num_atoms, s);
             HIPCHK(launch_force_scatter(num_atoms, rstart, rlist, rf_sstart.p, rf_slist.p, node_forces.p, rf_out.p, s));
             HIPCHK(hipMemcpyAsync(atom_forces, rf_out.p, (size_t)3 * num_atoms * sizeof(double), hipMemcpyDeviceToHost, s));

@@ -149,18 +149,20 @@ hipError_t launch_scale_bwd(int N, const int* first_neigh, const int* node_types
 hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums, hipStream_t s);  // out[n] = total
 // order[N]: receivers by decreasing degree
 hipError_t launch_degree_order(int N, const int* first_neigh, int* order, hipStream_t s);
-// counters_are_zero: 0 = clear count and cursor first, 1 = they are zero, 2 = zero cursor and the histogram already in count;
+// counters_are_zero: 0 = clear count and cursor first, 1 = they are zero, 2 = the histogram is already in count and
+// rank[E] holds every entry's place inside its bucket (launch_node_lists_count);
 // count and cursor are zero again when the launches have run
 hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
-                               int* slist, int* block_sums, int counters_are_zero, hipStream_t s);
+                               int* slist, int* block_sums, int counters_are_zero, const int* rank, hipStream_t s);
 // first_neigh, degree order, species groups and `zero_n` cleared counters in one single-block launch
 // (N <= 65536; larger systems use the separate launches, where the extra launches do not matter)
 hipError_t launch_node_lists(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
                              int* tstart, int* perm, int* zero_p, long zero_n, hipStream_t s);
-// launch_node_lists plus the sender histogram count[rows] of `key[n]` in the same launch; the counters must
-// be zero on entry (every sender-list build leaves them so)
+// launch_node_lists plus the sender histogram count[rows] of `key[n]` in the same launch, with rank[n] = the place
+// each entry took in its bucket; the counters must be zero on entry (every sender-list build leaves them so)
 hipError_t launch_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
-                                   int* tstart, int* perm, const int* key, long n, int rows, int* count, hipStream_t s);
+                                   int* tstart, int* perm, const int* key, long n, int rows, int* count, int* rank,
+                                   hipStream_t s);
 hipError_t launch_type_groups(const int* node_types, int N, int T, int* tcount, int* tstart, int* cursor,
                               int* perm, int* block_sums, hipStream_t s);
 // flags[0] |= 1 if any index is outside [0, limit)

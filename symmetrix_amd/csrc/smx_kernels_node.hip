@@ -251,7 +251,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists(const int* num_neigh,
 // count the senders (counters at zero on entry), which does not depend on the node lists.
 __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order,
                                                                 const int* node_types, int T, int* tstart, int* perm,
-                                                                const int* key, long n, int rows, int* count)
+                                                                const int* key, long n, int rows, int* count, int* rank)
 {
     extern __shared__ int sh[];
     if (blockIdx.x == 0) {
@@ -264,18 +264,28 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_
     }
     for (long i = (long)(blockIdx.x - 1) * SCAN_BLOCK + threadIdx.x; i < n; i += (long)(gridDim.x - 1) * SCAN_BLOCK) {
         const int j = key[i];
-        if (j >= 0 && j < rows) atomicAdd(&count[j], 1);
+        if (j >= 0 && j < rows) rank[i] = atomicAdd(&count[j], 1);   // the entry's place inside its bucket
+    }
+}
+// placement of entries that know their place inside the bucket: no atomics
+__global__ void k_place_ranked(const int* key, const int* rank, long n, int rows, const int* start, int* list)
+{
+    const long i = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) {
+        const int j = key[i];
+        if (j >= 0 && j < rows) list[start[j] + rank[i]] = (int)i;
     }
 }
 }  // namespace
 
 hipError_t launch_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
-                                   int* tstart, int* perm, const int* key, long n, int rows, int* count, hipStream_t s)
+                                   int* tstart, int* perm, const int* key, long n, int rows, int* count, int* rank,
+                                   hipStream_t s)
 {
     if (N <= 0 || N > 64 * SCAN_BLOCK || T <= 0) return hipErrorInvalidValue;
     const unsigned nb = 1 + (unsigned)std::min<long>((n + SCAN_BLOCK - 1) / SCAN_BLOCK, 2048);
     hipLaunchKernelGGL(k_node_lists_count, dim3(nb), dim3(SCAN_BLOCK), 2 * T * sizeof(int), s, num_neigh, N, first_neigh,
-                       order, node_types, T, tstart, perm, key, n, rows, count);
+                       order, node_types, T, tstart, perm, key, n, rows, count, rank);
     return hipGetLastError();
 }
 
@@ -302,7 +312,7 @@ hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums
 }
 
 hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
-                               int* slist, int* block_sums, int counters_are_zero, hipStream_t s)
+                               int* slist, int* block_sums, int counters_are_zero, const int* rank, hipStream_t s)
 {
     if (rows <= 0) return hipSuccess;
     const bool counted = counters_are_zero == 2;   // the histogram came with the node lists
@@ -318,7 +328,10 @@ hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, i
     hipError_t err = launch_scan_exclusive(count, sstart, rows, block_sums, s);
     if (err != hipSuccess) return err;
     if (E > 0) {
-        hipLaunchKernelGGL(k_place, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, sstart, cursor, slist);
+        if (counted && rank)
+            hipLaunchKernelGGL(k_place_ranked, dim3(nblk(E, 256)), dim3(256), 0, s, gather, rank, (long)E, rows, sstart, slist);
+        else
+            hipLaunchKernelGGL(k_place, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, sstart, cursor, slist);
         hipLaunchKernelGGL(k_sort_buckets, dim3(rows), dim3(64), 0, s, sstart, rows, slist, count, cursor);
     }
     return hipGetLastError();

@@ -150,17 +150,30 @@ int smx_reverse_M1(smx_model* m, int num_nodes, const int* node_types);         
 int smx_compute_H2(smx_model* m, int num_nodes, const int* node_types);                 /* mace.cpp:796-832 */
 int smx_reverse_H2(smx_model* m, int num_nodes, const int* node_types, int zero_H1_adj);/* mace.cpp:834-874 */
 int smx_compute_readouts(smx_model* m, int num_nodes, const int* node_types);           /* mace.cpp:876-903 */
+/* ZBL::compute_ZBL, libsymmetrix/source/zbl.hpp:26-34 / zbl.cpp:96-125, as the pair style calls it on
+ * mace->zbl before the stage sequence (pair_symmetrix/pair_symmetrix_mace.cpp:449-452, 667-670): adds the pair
+ * repulsion of every edge to the model's node_energies[num_nodes] and node_forces[3*num_edges] (the arrays of
+ * smx_get_array / smx_set_array / smx_fill_array; entries beyond their present length start at zero).  The species
+ * table is the model's own atomic_numbers.  A no-op for models with has_zbl false. */
+int smx_compute_ZBL(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh, const int* neigh_types,
+                    const double* r, const double* xyz, long num_edges);
 
 /* Read/write access to the named intermediates, the def_readwrite members of
  * the pybind class (symmetrix/source/cpp/mace.cpp:14-34): "node_energies",
  * "node_forces", "A0", "A0_adj", "M0", "M0_adj", "H1", "H1_adj", "Phi1",
- * "Phi1_adj", "A1", "A1_adj", "M1", "M1_adj", "H2", "H2_adj", plus "Y",
- * "Y_grad", "R0", "R1" (read-only, evaluated on demand from the remembered
- * geometry), "M0_grad", "M1_grad" and "H0_weights" (read-only).
+ * "Phi1_adj", "A1", "A1_adj", "M1", "M1_adj", "H2", "H2_adj", "H0_weights"
+ * (num_elements * num_channels values), plus "Y", "Y_grad", "R0", "R1"
+ * (read-only: evaluated on demand from the remembered geometry and never
+ * stored, so assigning R0 / R1 is refused with SMX_EUNSUPPORTED where the
+ * pybind class allows it), "M0_grad" and "M1_grad" (read-only).
  * smx_get_array copies min(cap, size) doubles to `out` and stores the full
  * size in *n; out may be NULL to query the size. */
 int smx_get_array(smx_model* m, const char* name, double* out, long cap, long* n);
 int smx_set_array(smx_model* m, const char* name, const double* in, long n);
+/* A settable array sized to n entries that all hold `value`, without a transfer from the host: what
+ * `v.resize(n); std::fill(v.begin(), v.end(), value)` does to a member of the reference class
+ * (pair_symmetrix_mace.cpp:444-447). */
+int smx_fill_array(smx_model* m, const char* name, long n, double value);
 
 /* Upper bound in bytes (default 32 GiB) for the buffer that stages the per-edge adjoint messages of reverse_Phi1
  * (mace.cpp:579-604) in models with l <= 1 hidden features.  Longer edge lists are processed in receiver chunks that

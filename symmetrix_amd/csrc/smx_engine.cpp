@@ -135,6 +135,7 @@ struct EngineBase {
                        long E, int flag_a, int flag_b) = 0;
     virtual void get_array(const char* name, double* out, long cap, long* n) = 0;
     virtual void set_array(const char* name, const double* in, long n) = 0;
+    virtual void fill_array(const char* name, long n, double value) = 0;
     virtual void reduce_forces(int num_atoms, const int* sender_atom, const int* receiver_atom,
                                double* atom_forces, double* virial, bool sender_on_device) = 0;
 
@@ -1011,9 +1012,21 @@ struct Engine : EngineBase {
         energies_copy = nullptr; forces_copy = nullptr;
         materialise_adjoints();
         if (N < 0) throw Error(SMX_EINVAL, "negative num_nodes");
-        if (nn && E_ >= 0) edges_from_counts_check(N, nn, E_);
+        // A stage may cover the leading nodes of a longer edge list (the pair style runs layer 1 on its local
+        // nodes with the arrays of local + ghost nodes, pair_symmetrix_mace.cpp:681-693): the edge arrays keep
+        // their full length, the stage's own edges are the first sum(num_neigh[0..N)).
+        long own_edges = -1;
+        if (nn) {
+            own_edges = 0;
+            for (int i = 0; i < N; ++i) {
+                if (nn[i] < 0) throw Error(SMX_EINVAL, "negative num_neigh entry");
+                own_edges += nn[i];
+            }
+            const long have = E_ >= 0 ? E_ : E;
+            if (own_edges > have) throw Error(SMX_EINVAL, "sum(num_neigh) exceeds the number of edges");
+        }
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, false);
-        if (nn) build_first_neigh(N);
+        if (nn) { build_first_neigh(N); E1 = own_edges; }
         validate_stage_inputs(N, nt != nullptr, ni != nullptr, nty != nullptr, rr != nullptr);
         if (s == "Y" || s == "R0" || s == "R1") return;  // geometry remembered; evaluated inside the fused kernels
         if (s == "A0") { build_type_groups(N); st_agg0_fwd(N); st_A0_lin(N, false); }
@@ -1042,6 +1055,17 @@ struct Engine : EngineBase {
         else if (s == "H2") { build_type_groups(N); st_H2(N); }
         else if (s == "reverse_H2") { build_type_groups(N); st_reverse_H2(N, fa != 0); }
         else if (s == "readouts") st_readouts(N, false);
+        else if (s == "ZBL") {
+            // zbl.cpp:96-125 adds to the caller's node_energies / node_forces: here to the engine's arrays, which
+            // grow like std::vector::resize (new entries zero) when the edge list changed
+            if (hm.has_zbl) {
+                need(xyz, "xyz"); need(r, "r"); need(first_neigh.p, "num_neigh"); need(node_types, "node_types");
+                need(neigh_types, "neigh_types");
+                node_energies.resize((size_t)N, stream);
+                node_forces.resize((size_t)3 * E, stream);
+                st_zbl(N);
+            }
+        }
         else throw Error(SMX_EINVAL, "unknown stage " + s);
     }
 
@@ -1120,8 +1144,13 @@ struct Engine : EngineBase {
         if (n < 0) throw Error(SMX_EINVAL, "negative length");
         materialise_adjoints();
         Named v = find(s);
-        if ((!v.f && !v.d) || s == "H0_weights" || s == "M0_grad" || s == "M1_grad")
+        if (s == "R0" || s == "R1")
+            throw Error(SMX_EUNSUPPORTED, "unsupported: '" + s + "' is evaluated from r inside the edge kernels and never "
+                        "stored; call compute_" + s + " with the edge lengths instead of assigning it");
+        if ((!v.f && !v.d) || s == "M0_grad" || s == "M1_grad")
             throw Error(SMX_EINVAL, "array '" + s + "' cannot be set");
+        if (s == "H0_weights" && (size_t)n != (size_t)hm.T * hm.K)
+            throw Error(SMX_EINVAL, "H0_weights holds num_elements * num_channels values");
         if (v.d) { v.d->upload(in, (size_t)n, st); }
         else if (std::is_same<F, double>::value) { reinterpret_cast<DVec<double>*>(v.f)->upload(in, (size_t)n, st); }
         else {
@@ -1130,6 +1159,19 @@ struct Engine : EngineBase {
             HIPCHK((launch_convert<double, F>(scratch_d.p, v.f->p, n, st)));
         }
         HIPCHK(hipStreamSynchronize(st));
+    }
+
+    // size a named array to n entries, all equal to `value`, without a host copy
+    void fill_array(const char* name, long n, double value) override
+    {
+        const std::string s(name);
+        if (n < 0) throw Error(SMX_EINVAL, "negative length");
+        materialise_adjoints();
+        Named v = find(s);
+        if ((!v.f && !v.d) || s == "H0_weights" || s == "M0_grad" || s == "M1_grad")
+            throw Error(SMX_EINVAL, "array '" + s + "' cannot be set");
+        if (v.d) { v.d->size_to((size_t)n, stream); HIPCHK(launch_fill<double>(v.d->p, n, value, stream)); }
+        else { v.f->size_to((size_t)n, stream); HIPCHK(launch_fill<F>(v.f->p, n, (F)value, stream)); }
     }
 
     // ------------------------------------------------------------------
@@ -1167,8 +1209,10 @@ struct Engine : EngineBase {
                 size_t e = 0;
                 for (int i = 0; i < N_geo; ++i) {
                     if (receiver_atom[i] < 0 || receiver_atom[i] >= num_atoms) throw Error(SMX_EINVAL, "receiver_atom out of range");
+                    if (hn[i] < 0 || e + (size_t)hn[i] > (size_t)E) throw Error(SMX_EINVAL, "num_neigh does not match the number of edges");
                     for (int j = 0; j < hn[i]; ++j) hr[e++] = receiver_atom[i];
                 }
+                if (e != (size_t)E) throw Error(SMX_EINVAL, "num_neigh of the last call does not cover every edge");
                 rf_recv.upload(hr.data(), hr.size(), s);
                 HIPCHK(hipStreamSynchronize(s));
                 rf_rstart.size_to((size_t)num_atoms + 1, s); rf_rlist.size_to((size_t)E, s);
@@ -1605,6 +1649,12 @@ int smx_compute_readouts(smx_model* m, int num_nodes, const int* node_types)
     SMX_STAGE(smx_compute_readouts, "readouts", node_types, nullptr, nullptr, nullptr, nullptr, nullptr, -1, 0, 0);
 }
 
+int smx_compute_ZBL(smx_model* m, int num_nodes, const int* node_types, const int* num_neigh, const int* neigh_types,
+                    const double* r, const double* xyz, long num_edges)
+{
+    SMX_STAGE(smx_compute_ZBL, "ZBL", node_types, num_neigh, nullptr, neigh_types, xyz, r, num_edges, 0, 0);
+}
+
 int smx_get_array(smx_model* m, const char* name, double* out, long cap, long* n)
 {
     return guarded([&] {
@@ -1617,6 +1667,16 @@ int smx_set_array(smx_model* m, const char* name, const double* in, long n)
     return guarded([&] {
         if (!name || (!in && n > 0)) throw smx::Error(SMX_EINVAL, "null argument");
         E(m).set_array(name, in, n);
+    });
+}
+
+int smx_fill_array(smx_model* m, const char* name, long n, double value)
+{
+    return guarded([&] {
+        if (!name) throw smx::Error(SMX_EINVAL, "null name");
+        auto& e = E(m);
+        e.fill_array(name, n, value);
+        HIPCHK(hipStreamSynchronize(e.stream));
     });
 }
 

@@ -165,6 +165,25 @@ class MACE:
         return (F, V) if virial else F
 
     # --- stages --------------------------------------------------------------
+    @property
+    def zbl(self):
+        """The `zbl` member of the reference class (libsymmetrix/source/mace.hpp:39): `mace.zbl.compute_ZBL(...)`."""
+        return _ZBL(self)
+
+    def compute_ZBL(self, num_nodes, node_types, num_neigh, neigh_types, r, xyz):
+        """Pair repulsion added to this model's node_energies / node_forces (zbl.cpp:96-125), the call the pair
+        style makes before the stage sequence (pair_symmetrix_mace.cpp:449-452).  No-op without ZBL."""
+        nt, nn, nty = _i(node_types), _i(num_neigh), _i(neigh_types)
+        x, rr = _d(xyz).reshape(-1), _d(r)
+        if len(x) != 3 * len(rr) or len(nty) != len(rr):
+            raise ValueError("edge arrays differ in length")
+        _lib.check(self._L.smx_compute_ZBL(self._h, int(num_nodes), _pi(nt), _pi(nn), _pi(nty), _pd(rr), _pd(x),
+                                           C.c_long(len(rr))))
+
+    def fill(self, name, n, value=0.0):
+        """`name` sized to n entries equal to value, on the device (no host copy)."""
+        _lib.check(self._L.smx_fill_array(self._h, name.encode(), C.c_long(int(n)), C.c_double(float(value))))
+
     def compute_Y(self, xyz):
         x = _d(xyz).reshape(-1)
         _lib.check(self._L.smx_compute_Y(self._h, _pd(x), C.c_long(len(x))))
@@ -255,3 +274,27 @@ class MACE:
     def compute_readouts(self, num_nodes, node_types):
         nt = _i(node_types)
         _lib.check(self._L.smx_compute_readouts(self._h, int(num_nodes), _pi(nt)))
+
+
+class _ZBL:
+    """`compute_ZBL` with the argument list of libsymmetrix/source/zbl.hpp:26-34.  The pair repulsion is added on the
+    device to the owning model's node_energies / node_forces; the two output arguments are written as well when they
+    are numpy arrays."""
+
+    def __init__(self, owner):
+        self._o = owner
+
+    def compute_ZBL(self, num_nodes, node_types, num_neigh, neigh_types, atomic_numbers, r, xyz, node_energies=None,
+                    node_forces=None):
+        o = self._o
+        if list(atomic_numbers) != list(o.atomic_numbers):
+            raise ValueError("compute_ZBL: atomic_numbers must be the model's own species table")
+        if node_energies is not None:
+            o.node_energies = node_energies
+        if node_forces is not None:
+            o.node_forces = node_forces
+        o.compute_ZBL(num_nodes, node_types, num_neigh, neigh_types, r, xyz)
+        if isinstance(node_energies, np.ndarray):
+            node_energies[...] = o.node_energies[:node_energies.size].reshape(node_energies.shape)
+        if isinstance(node_forces, np.ndarray):
+            node_forces[...] = o.node_forces[:node_forces.size].reshape(node_forces.shape)

@@ -20,29 +20,66 @@ from __future__ import annotations
 import numpy as np
 
 
-def neighbor_list(positions, cell, r_cut, pbc=(True, True, True)):
-    """Full neighbour list of an orthorhombic or triclinic periodic cell.
+def wrap_positions(positions, cell, pbc=(True, True, True), offsets=None):
+    """Positions folded into the cell along the periodic axes, and the integer lattice offsets taken off:
+    returns (wrapped [N,3], offsets int [N,3]) with positions = wrapped + offsets . cell.
 
-    Returns dict with i, j (int32), S (int32 [E,3] cell shifts), xyz ([E,3] =
-    x_j + S.cell - x_i), r ([E]), first_neigh ([N+1]) in canonical order.
-    """
-    pos = np.ascontiguousarray(positions, dtype=np.float64)
+    The builders below enumerate ceil(r_cut / height) image shells, which finds every pair only when all atoms
+    lie within one cell span; molecular dynamics does not keep them there (the reference's caller hands
+    unwrapped positions straight to neighbor_list('ijdD'), symmetrix_calc.py:77).  Atoms already inside the
+    cell come back bit for bit (offset 0).  `offsets` ([N,3] integers) are taken off instead of the floor of
+    the fractional coordinates: the frame of an earlier call, in which atoms that moved since may lie a
+    little outside the cell."""
+    pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
     cell = np.asarray(cell, dtype=np.float64)
     if cell.shape == (3,):
         cell = np.diag(cell)
-    N = len(pos)
+    if len(pos) == 0:
+        return pos, np.zeros((0, 3), dtype=np.int64)
+    pbc = np.asarray(pbc, dtype=bool)
+    frac = pos @ np.linalg.inv(cell)
+    if not np.all(np.isfinite(frac)):
+        raise ValueError("positions are not finite")
+    if offsets is not None:
+        off = np.asarray(offsets, dtype=np.int64).reshape(-1, 3)
+        if off.shape != pos.shape:
+            raise ValueError("offsets must hold three integers per atom")
+    else:
+        off = np.where(pbc[None, :], np.floor(frac), 0.0).astype(np.int64)
+    if not off.any():
+        return pos, off
+    return pos - off.astype(np.float64) @ cell, off
+
+
+def neighbor_list(positions, cell, r_cut, pbc=(True, True, True), offsets=None):
+    """Full neighbour list of an orthorhombic or triclinic periodic cell.
+
+    Returns dict with i, j (int32), S (int32 [E,3] cell shifts), xyz ([E,3] =
+    x_j + S.cell - x_i), r ([E]), first_neigh ([N+1]) in canonical order.  Atoms may lie outside the cell:
+    they are folded in first and the lattice offsets go into S, so that S still refers to the positions given.
+    With `offsets` the list is formed in that frame instead (see wrap_positions).
+    """
+    pos_in = np.ascontiguousarray(positions, dtype=np.float64)
+    cell = np.asarray(cell, dtype=np.float64)
+    if cell.shape == (3,):
+        cell = np.diag(cell)
+    N = len(pos_in)
     if N == 0:
         return dict(i=np.zeros(0, np.int32), j=np.zeros(0, np.int32), S=np.zeros((0, 3), np.int32),
                     xyz=np.zeros((0, 3)), r=np.zeros(0), first_neigh=np.zeros(1, np.int64))
     pbc = np.asarray(pbc, dtype=bool)
+    pos, wrap = wrap_positions(pos_in, cell, pbc, offsets)
     # number of image shells needed along each lattice vector
     vol = abs(np.linalg.det(cell))
     heights = np.array([vol / np.linalg.norm(np.cross(cell[(a + 1) % 3], cell[(a + 2) % 3])) for a in range(3)])
-    nshell = np.where(pbc, np.ceil(r_cut / heights).astype(int), 0)
     inv = np.linalg.inv(cell)
     frac = pos @ inv
     lo_f = frac.min(axis=0) if N else np.zeros(3)
     hi_f = frac.max(axis=0) if N else np.zeros(3)
+    # a pair (i, j + S) within r_cut has |f_j + S - f_i| <= r_cut / height along every axis: |S| <= r_cut / height +
+    # (spread of the fractional coordinates), which is below ceil(r_cut / height) + 1 for atoms inside the cell
+    nshell = np.maximum(np.ceil(r_cut / heights), np.floor(r_cut / heights + (hi_f - lo_f))).astype(int)
+    nshell = np.where(pbc, nshell, 0)
     margin = r_cut / heights
     img_j, img_S, img_pos = [], [], []
     for sx in range(-nshell[0], nshell[0] + 1):
@@ -114,6 +151,8 @@ def neighbor_list(positions, cell, r_cut, pbc=(True, True, True)):
     first = np.zeros(N + 1, dtype=np.int64)
     np.add.at(first, ei + 1, 1)
     first = np.cumsum(first)
+    # x_j + S.cell - x_i for the positions as given: the shift found for the folded atoms, corrected by their offsets
+    eS = eS + wrap[ei] - wrap[ej]
     return dict(i=ei.astype(np.int32), j=ej.astype(np.int32), S=eS.astype(np.int32),
                 xyz=np.ascontiguousarray(d), r=r, first_neigh=first)
 
@@ -128,6 +167,8 @@ def brute_force_neighbor_list(positions, cell, r_cut, pbc=(True, True, True)):
     vol = abs(np.linalg.det(cell))
     heights = np.array([vol / np.linalg.norm(np.cross(cell[(a + 1) % 3], cell[(a + 2) % 3])) for a in range(3)])
     nshell = np.where(np.asarray(pbc, bool), np.ceil(r_cut / heights).astype(int), 0)
+    # edge vectors are defined on the folded positions (as in neighbor_list); shifts refer to the positions given
+    pos, wrap = wrap_positions(pos, cell, pbc)
     rows = []
     for i in range(N):
         for j in range(N):
@@ -140,7 +181,8 @@ def brute_force_neighbor_list(positions, cell, r_cut, pbc=(True, True, True)):
                         d = pj - pos[i]
                         r2 = d[0] * d[0] + d[1] * d[1] + d[2] * d[2]
                         if r2 < r_cut * r_cut:
-                            rows.append((i, j, sx, sy, sz, d[0], d[1], d[2], np.sqrt(r2)))
+                            S = np.array([sx, sy, sz]) + wrap[i] - wrap[j]
+                            rows.append((i, j, S[0], S[1], S[2], d[0], d[1], d[2], np.sqrt(r2)))
     rows.sort(key=lambda t: t[:5])
     a = np.array(rows, dtype=np.float64).reshape(-1, 9)
     return dict(i=a[:, 0].astype(np.int32), j=a[:, 1].astype(np.int32), S=a[:, 2:5].astype(np.int32),
@@ -240,6 +282,13 @@ class DeviceNeighborList:
         self.num_atoms = 0
         self.num_edges = 0
         self.ptr = {}
+        self._wrap = None      # lattice offsets taken off the positions of the last build_host
+        self._cell = None
+
+    @property
+    def offsets(self):
+        """Integer lattice offsets [N,3] that build_host took off the positions (None after build())."""
+        return self._wrap
 
     def __del__(self):
         try:
@@ -262,8 +311,12 @@ class DeviceNeighborList:
         return self.num_edges
 
     def build(self, num_atoms, positions_ptr, types_ptr, cell, r_cut, pbc=(True, True, True), skin=0.0, stream=0):
-        """New search: pairs within r_cut + skin are remembered, edges are the pairs within r_cut."""
+        """New search: pairs within r_cut + skin are remembered, edges are the pairs within r_cut.
+
+        The device positions are used as they are and must lie inside the cell along periodic axes (fold them with
+        wrap_positions first, or use build_host): the shift table covers one cell span."""
         C = self._C
+        self._wrap = None
         r_list = float(r_cut) + float(skin)
         ints, vecs = image_shifts(cell, r_list, pbc)
         E = C.c_long(0)
@@ -278,7 +331,11 @@ class DeviceNeighborList:
         """build() from numpy positions [N][3] and species indices [N]; device copies are kept in the list object
         (addresses in .ptr["positions"], .ptr["node_types"])."""
         C = self._C
-        pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
+        # folded into the cell: the image shifts below cover one cell span (an update keeps these offsets, so
+        # that the remembered pairs stay the same pairs)
+        pos, self._wrap = wrap_positions(positions, cell, pbc)
+        cellm = np.asarray(cell, dtype=np.float64)
+        self._cell = np.diag(cellm) if cellm.shape == (3,) else cellm
         ty = np.ascontiguousarray(types, dtype=np.int32)
         if len(ty) != len(pos):
             raise ValueError("positions and types differ in length")
@@ -298,6 +355,8 @@ class DeviceNeighborList:
         pos = np.ascontiguousarray(positions, dtype=np.float64).reshape(-1, 3)
         if len(pos) != self.num_atoms:
             raise ValueError("the number of atoms differs from the last build")
+        if self._wrap is not None and self._wrap.any():
+            pos = pos - self._wrap.astype(np.float64) @ self._cell
         E = C.c_long(0)
         self._lib.check(self._L.smx_nlist_update_host(C.c_void_p(self._h), pos.ctypes.data_as(C.POINTER(C.c_double)),
                                                       C.c_double(r_cut), C.byref(E)))
@@ -320,5 +379,8 @@ class DeviceNeighborList:
         self._lib.check(self._L.smx_nlist_copy_to_host(C.c_void_p(self._h), p(nn, C.c_int), p(ni, C.c_int), p(nty, C.c_int),
                                                        p(S, C.c_int), p(xyz, C.c_double), p(r, C.c_double)))
         first = np.concatenate([[0], np.cumsum(nn)]).astype(np.int64)
-        return dict(i=np.repeat(np.arange(N, dtype=np.int32), nn), j=ni, S=S, xyz=xyz, r=r, first_neigh=first,
+        i = np.repeat(np.arange(N, dtype=np.int32), nn)
+        if self._wrap is not None and self._wrap.any():
+            S = (S + self._wrap[i] - self._wrap[ni]).astype(np.int32)
+        return dict(i=i, j=ni, S=S, xyz=xyz, r=r, first_neigh=first,
                     num_neigh=nn, neigh_types=nty)

@@ -398,7 +398,8 @@ def test_device_neighbor_list_update_equals_fresh_build():
         dpos = torch.from_numpy(pos).cuda()
         print(f"update step {step}", flush=True)
         E = dnl.update(dpos.data_ptr(), dty.data_ptr(), rc)
-        got, ref = dnl.to_host(), neighbors.neighbor_list(pos, cell, rc)
+        # the list keeps the frame of its build: atoms that drifted out of the cell are not folded back in
+        got, ref = dnl.to_host(), neighbors.neighbor_list(pos, cell, rc, offsets=np.zeros((len(pos), 3), dtype=int))
         assert E == len(ref["r"])
         for k in ("i", "j", "S", "xyz", "r", "first_neigh"):
             assert np.array_equal(got[k], ref[k].reshape(got[k].shape)), k
@@ -409,8 +410,16 @@ def test_device_neighbor_list_update_equals_fresh_build():
     hnl.build_host(pos, types, cell, rc, skin=skin)
     pos2 = pos + rng.uniform(-0.1, 0.1, size=pos.shape)
     E = hnl.update_host(pos2, rc)
-    got, ref = hnl.to_host(), neighbors.neighbor_list(pos2, cell, rc)
+    got, ref = hnl.to_host(), neighbors.neighbor_list(pos2, cell, rc, offsets=hnl.offsets)
+    assert hnl.offsets.any()                   # some atoms had left the cell before this build
     assert E == len(ref["r"]) and np.array_equal(got["j"], ref["j"]) and np.array_equal(got["r"], ref["r"])
+    assert np.array_equal(got["S"], ref["S"]) and np.array_equal(got["xyz"], ref["xyz"])
+    far = pos2 + rng.integers(-2, 3, size=pos2.shape) @ cell      # whole lattice vectors away: same edges
+    E2 = hnl.build_host(far, types, cell, rc)
+    got2, ref2 = hnl.to_host(), neighbors.neighbor_list(far, cell, rc)
+    assert E2 == len(ref2["r"]) == len(neighbors.neighbor_list(pos2, cell, rc)["r"])
+    for k in ("i", "j", "S", "xyz", "r"):
+        assert np.array_equal(got2[k], ref2[k].reshape(got2[k].shape)), k
     assert np.array_equal(got["neigh_types"], types[ref["j"]])
 
 
@@ -470,7 +479,7 @@ def test_pair_style_modes_agree(gpu, tmp_models, L_max, dtype):
     through layer 0 (no_mpi_message_passing, one call), and ghost rows of H1 filled by a forward copy with the
     adjoint summed back (mpi_message_passing, stage calls as pair_symmetrix_mace.cpp:372-550 issues them)."""
     from symmetrix_amd import neighbors
-    model = H.tiny_model(K=16, L_max=L_max, n_pts=48, seed=12, zbl=(dtype == "float32"), density=(L_max == 1))
+    model = H.tiny_model(K=16, L_max=L_max, n_pts=48, seed=12, zbl=(dtype == "float32" or L_max == 1), density=(L_max == 1))
     path = H.write_model(model, tmp_models / f"modes{L_max}{dtype}.json")
     pos, cell, sp = H.small_system(36, seed=21)
     nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
@@ -496,9 +505,9 @@ def test_pair_style_modes_agree(gpu, tmp_models, L_max, dtype):
     nt, nn = ga["node_types"][:Nl], ga["num_neigh"][:Nl]
     ni, nty, x, r = ga["neigh_indices"][:El], ga["neigh_types"][:El], ga["xyz"][:3 * El], ga["r"][:El]
     eng2 = gpu(path, dtype)
-    eng2.node_energies = np.zeros(Nl); eng2.node_forces = np.zeros(3 * El)
-    if model["has_zbl"]:
-        return      # the stage calls hold no separate ZBL step; the two whole-pipeline modes above cover it
+    eng2.fill("node_energies", Nl); eng2.fill("node_forces", 3 * El)
+    if eng2.has_zbl:
+        eng2.zbl.compute_ZBL(Nl, nt, nn, nty, eng2.atomic_numbers, r, x)         # pair_symmetrix_mace.cpp:449-452
     eng2.compute_Y(x)
     eng2.compute_R0(Nl, nt, nn, nty, r); eng2.compute_A0(Nl, nt, nn, nty); eng2.compute_A0_scaled(Nl, nt, nn, nty, r)
     eng2.compute_M0(Nl, nt); eng2.compute_H1(Nl)

@@ -145,9 +145,44 @@ def test_capi_error_paths_without_gpu(tmp_path):
 
 
 def test_cpp_class_header_compiles():
-    """include/symmetrix_amd/mace.hpp is a drop-in for libsymmetrix's mace.hpp for a C++20 caller."""
+    """include/symmetrix_amd/mace.hpp is a drop-in for libsymmetrix's mace.hpp for a C++20 caller: the statement
+    forms the reference pair style applies to its evaluator compile unchanged (tests/cpp/reference_caller_syntax.cpp),
+    and so does the LAMMPS-free half of this repository's pair style."""
     import subprocess
-    src = '#include "mace.hpp"\n#include <memory>\nint f(){ std::unique_ptr<MACE> m; return m ? m->num_channels : 0; }\n'
-    r = subprocess.run(["g++", "-std=c++20", "-fsyntax-only", "-I", os.path.join(ROOT, "include", "symmetrix_amd"),
-                        "-x", "c++", "-"], input=src.encode(), capture_output=True)
-    assert r.returncode == 0, r.stderr.decode()
+    inc = ["-I", os.path.join(ROOT, "include", "symmetrix_amd"), "-I", os.path.join(ROOT, "include")]
+    for src in (os.path.join(ROOT, "tests", "cpp", "reference_caller_syntax.cpp"),
+                os.path.join(ROOT, "pair_symmetrix_amd", "mace_evaluation.cpp")):
+        r = subprocess.run(["g++", "-std=c++20", "-Wall", "-Wextra", "-fsyntax-only", *inc, src], capture_output=True)
+        assert r.returncode == 0, r.stderr.decode()
+
+
+@pytest.mark.parametrize("triclinic", [False, True])
+def test_neighbor_list_of_atoms_outside_the_cell(triclinic):
+    """Atoms translated by whole lattice vectors (as molecular dynamics leaves them: nothing wraps positions
+    between steps, and the reference's calculator passes them on unwrapped, symmetrix_calc.py:77) keep the same
+    neighbours: same (i, j) sets, the shifts differ by the translations, xyz and r agree to rounding.  The two
+    atoms of a 10 A cell at x = 1.0 and x = 21.5 are 0.5 A apart."""
+    cell = np.array([[10.0, 0, 0], [0, 10.0, 0], [0, 0, 10.0]])
+    nl = neighbors.neighbor_list(np.array([[1.0, 5, 5], [21.5, 5, 5]]), cell, 3.0)
+    assert len(nl["i"]) == 2 and np.allclose(nl["r"], 0.5)
+    assert nl["S"].tolist() == [[-2, 0, 0], [2, 0, 0]] and np.allclose(nl["xyz"][0], [0.5, 0, 0])
+    rng = np.random.default_rng(5)
+    cell = np.array([[7.0, 0, 0], [1.5, 6.5, 0], [-0.8, 0.9, 7.5]]) if triclinic else np.diag([7.0, 6.5, 7.5])
+    N = 25
+    pos = rng.uniform(0, 1, size=(N, 3)) @ cell
+    moves = rng.integers(-3, 4, size=(N, 3))
+    moved = pos + moves @ cell
+    a = neighbors.neighbor_list(pos, cell, 4.0)
+    b = neighbors.neighbor_list(moved, cell, 4.0)
+    c = neighbors.brute_force_neighbor_list(moved, cell, 4.0)
+    assert len(a["i"]) > 0
+    for other in (b, c):
+        assert np.array_equal(a["i"], other["i"]) and np.array_equal(a["j"], other["j"])
+        assert np.array_equal(a["S"] + moves[a["i"]] - moves[a["j"]], other["S"])
+        assert np.allclose(a["xyz"], other["xyz"], rtol=0, atol=1e-12) and np.allclose(a["r"], other["r"], rtol=0, atol=1e-12)
+    # open axis: no folding along it
+    d = neighbors.neighbor_list(moved, cell, 4.0, pbc=(True, True, False))
+    e = neighbors.brute_force_neighbor_list(moved, cell, 4.0, pbc=(True, True, False))
+    assert np.array_equal(d["i"], e["i"]) and np.array_equal(d["j"], e["j"]) and np.array_equal(d["S"], e["S"])
+    w, off = neighbors.wrap_positions(moved, cell)
+    assert np.allclose(w + off @ cell, moved, atol=1e-12) and np.all((w @ np.linalg.inv(cell) > -1e-9) & (w @ np.linalg.inv(cell) < 1 + 1e-9))

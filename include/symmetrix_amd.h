@@ -205,6 +205,20 @@ int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const
 int smx_reduce_forces_device(smx_model* m, int num_atoms, const int* d_sender_atom, double* atom_forces,
                              double* virial);
 
+/* The reduction of smx_reduce_forces_device for callers that cannot allocate device memory: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  Same
+ * inputs (the forces of the model's last evaluation, d_sender_atom[num_edges] on the device, receiver i = atom i),
+ * outputs in device memory (d_atom_forces[3*num_atoms], d_virial[6]; either may be NULL), work enqueued on `stream`
+ * without synchronising.  The per-atom sender lists and the partial virial sums live in a fixed array of about
+ * 20 MiB that every GPU holds from the first model load to the end of the process, so sizes beyond
+ * SMX_NOALLOC_MAX_ATOMS atoms or SMX_NOALLOC_MAX_EDGES edges are refused with SMX_EINVAL, and calls that overlap on
+ * one GPU race (all of them share that GPU's array).  A sender index outside [0, num_atoms) cannot be reported
+ * without a synchronisation: the outputs are NaN then.  Calls no hipMalloc / hipFree and no allocating routine. */
+#define SMX_NOALLOC_MAX_ATOMS 262144
+#define SMX_NOALLOC_MAX_EDGES 4194304
+int smx_reduce_forces_device_noalloc(smx_model* m, int num_atoms, const int* d_sender_atom, double* d_atom_forces,
+                                     double* d_virial, void* stream);
+
 /* Full neighbour list built on the device, counterpart of the edge construction of
  * pair_symmetrix_mace.cpp:246-315 (ghost images, r^2 < r_cut^2) and of the ASE caller's
  * neighbor_list('ijdD') (symmetrix_calc.py:77-83), in the canonical order of this library: receivers

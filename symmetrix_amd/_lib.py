@@ -29,7 +29,7 @@ EXPORTS = [
     "smx_reverse_M1", "smx_compute_H2", "smx_reverse_H2", "smx_compute_readouts", "smx_get_array",
     "smx_set_array", "smx_set_profiling", "smx_stage_names", "smx_get_stage_times", "smx_synchronize",
     "smx_reduce_forces", "smx_set_staging_limit", "smx_nlist_create", "smx_nlist_free", "smx_nlist_build", "smx_nlist_update", "smx_nlist_build_host", "smx_nlist_update_host", "smx_nlist_inputs", "smx_reduce_forces_device", "smx_nlist_arrays",
-    "smx_nlist_copy_to_host", "smx_compute_ZBL", "smx_fill_array",
+    "smx_nlist_copy_to_host", "smx_compute_ZBL", "smx_fill_array", "smx_reduce_forces_device_noalloc",
 ]
 
 

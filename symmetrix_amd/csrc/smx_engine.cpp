@@ -29,6 +29,7 @@
 
 #include "../../include/symmetrix_amd.h"
 #include "smx_host_model.hpp"
+#include "smx_internal.hpp"
 #include "smx_json.hpp"
 #include "smx_kernels.hpp"
 #include "smx_paths.hpp"
@@ -136,6 +137,7 @@ struct EngineBase {
     virtual void get_array(const char* name, double* out, long cap, long* n) = 0;
     virtual void set_array(const char* name, const double* in, long n) = 0;
     virtual void fill_array(const char* name, long n, double value) = 0;
+    virtual void forces_view(ForcesView* v) = 0;
     virtual void reduce_forces(int num_atoms, const int* sender_atom, const int* receiver_atom,
                                double* atom_forces, double* virial, bool sender_on_device) = 0;
 
@@ -1161,6 +1163,11 @@ struct Engine : EngineBase {
         HIPCHK(hipStreamSynchronize(st));
     }
 
+    void forces_view(ForcesView* v) override
+    {
+        v->node_forces = node_forces.p; v->forces_len = (long)node_forces.n; v->xyz = xyz; v->first_neigh = first_neigh.p;
+        v->num_edges = E; v->num_receivers = N_geo;
+    }
     // size a named array to n entries, all equal to `value`, without a host copy
     void fill_array(const char* name, long n, double value) override
     {
@@ -1251,12 +1258,23 @@ struct Engine : EngineBase {
     }
 };
 
+void set_last_error(const std::string& msg) { g_last_error = msg; }
+
 }  // namespace smx
 
 // ===========================================================================
 struct smx_model {
     std::unique_ptr<smx::EngineBase> eng;
 };
+
+namespace smx {
+int engine_forces_view(smx_model* m, ForcesView* out, std::string* err)
+{
+    if (!m || !m->eng) { if (err) *err = "null model"; return SMX_EINVAL; }
+    m->eng->forces_view(out);
+    return SMX_OK;
+}
+}  // namespace smx
 
 namespace {
 
@@ -1413,6 +1431,12 @@ int smx_model_load(const char* json_path, int flags, smx_model** out)
         *out = nullptr;
         smx::HostModel hm = smx::load_host_model(json_path);
         require_device();
+        {
+            // the scratch array of the entry point that does not allocate: its address on this device, once
+            std::string err;
+            const int rc = smx::noalloc_setup_current_device(&err);
+            if (rc != SMX_OK) throw smx::Error(rc, err);
+        }
         std::unique_ptr<smx_model> m(new smx_model());
         if (flags == SMX_FP64) m->eng.reset(new smx::Engine<double>(std::move(hm), flags));
         else m->eng.reset(new smx::Engine<float>(std::move(hm), flags));

@@ -1,0 +1,176 @@
+"""The benchmark configurations that the other GPU tests do not run as such: the 192-atom H/C/O case at full size
+against the oracle, the 25 002-atom water-like box through the pair style's ghost-node layout, and the capacity
+run's molecular-dynamics loop (positions moved on the device, neighbour list searched or filtered on the device,
+evaluation on device-resident arrays) at a size that takes seconds."""
+import numpy as np
+import pytest
+
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+TOL = {"float64": dict(E=1e-10, F=1e-8), "float32": dict(E=1e-5, F=1e-4)}
+
+
+@pytest.fixture(scope="module")
+def gpu():
+    import torch
+    assert torch.cuda.is_available(), "these tests need the GPU box"
+    from symmetrix_amd.mace import MACE
+    return MACE
+
+
+def _model_file(tmp_models, name, **override):
+    import os
+    from symmetrix_amd import modelgen
+    cfg = dict(modelgen.CONFIGS[name]); cfg.update(override)
+    tag = "_".join(f"{k}{v}" for k, v in sorted(override.items()))
+    path = str(tmp_models / f"cfg_{name}_{tag}.json")
+    if not os.path.exists(path):
+        modelgen.write_model(path, **cfg)
+    return path, cfg
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("pair", [False, True], ids=["one_table", "pair_tables"])
+def test_tiny_configuration_at_full_size_against_the_oracle(gpu, tmp_models, pair, dtype):
+    """192 atoms H/C/O at 0.10 atoms/A^3, K = 32, r_cut 5.0 A, 256 spline points: the configuration the reference
+    CPU path runs.  With one radial table (plain MACE) the channel-slice kernels serve both layers, with six pair
+    tables the general ones do."""
+    from oracle.oracle import OracleMACE
+    from symmetrix_amd import neighbors, systems
+    path, cfg = _model_file(tmp_models, "tiny", pair_dependent_radial=pair)
+    pos, cell, sp = systems.config_system("tiny")
+    assert len(pos) == 192
+    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"]); ea = neighbors.edge_arrays(nl, sp)
+    print(f"tiny: {len(pos)} atoms, {len(ea['r'])} edges, pair tables {pair}, {dtype}", flush=True)
+    orc = OracleMACE(path)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng = gpu(path, dtype)
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    Eo = orc.node_energies.sum()
+    assert abs(eng.node_energies.sum() - Eo) <= TOL[dtype]["E"] * abs(Eo)
+    assert np.abs(eng.node_forces - orc.node_forces).max() <= TOL[dtype]["F"]
+    F = eng.reduce_forces(len(pos), nl["j"])
+    assert np.abs(F - H.atom_forces(nl, orc.node_forces, len(pos))).max() <= TOL[dtype]["F"] * 10
+
+
+def test_water_box_with_ghost_nodes_at_full_size(gpu, tmp_models):
+    """25 002 atoms, K = 128, hidden features up to l = 1, r_cut 5.0 A, through the full neighbour list with ghost
+    atoms as extra nodes (the pair style's no_mpi_message_passing layout on one rank): node energies bit-equal to
+    the owner-indexed layout, atom forces equal to rounding, Newton's third law; the same model on a 1 % box against
+    the oracle in both layouts."""
+    from oracle.oracle import OracleMACE
+    from symmetrix_amd import neighbors, systems
+    path, cfg = _model_file(tmp_models, "off_medium", pair_dependent_radial=False)
+    pos, cell, sp = systems.config_system("off_medium")
+    N = len(pos)
+    assert N == 25002
+    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"]); ea = neighbors.edge_arrays(nl, sp)
+    ga = neighbors.ghost_edge_arrays(nl, sp)
+    Nl, Ng = ga["num_local_nodes"], ga["num_ghost_nodes"]
+    print(f"water box: {N} atoms, {len(ea['r'])} edges; ghost layout {Ng} ghost nodes, {len(ga['r'])} edges", flush=True)
+    assert Nl == N and Ng > 5000
+    eng = gpu(path, "float64")
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    e_own = eng.node_energies.copy()
+    F_own = eng.reduce_forces(N, nl["j"])
+    assert np.abs(F_own.sum(0)).max() < 1e-8
+    eng.compute_ghosted(Nl, Ng, ga["node_types"], ga["num_neigh"], ga["neigh_indices"], ga["neigh_types"], ga["xyz"], ga["r"])
+    e_gh = eng.node_energies.copy()
+    F_gh = eng.reduce_forces(N, ga["sender_atom"], ga["receiver_atom"])
+    assert np.array_equal(e_gh, e_own)
+    assert np.abs(F_gh - F_own).max() <= 1e-9 * max(1.0, np.abs(F_own).max())
+    e32 = gpu(path, "float32")
+    e32.compute_ghosted(Nl, Ng, ga["node_types"], ga["num_neigh"], ga["neigh_indices"], ga["neigh_types"], ga["xyz"], ga["r"])
+    assert abs(e32.node_energies.sum() - e_own.sum()) <= 1e-5 * abs(e_own.sum())
+    # hydrogens are placed without regard to other molecules, so some pairs are nearly on top of each other and their
+    # forces reach hundreds of eV/A: the float32 bound of 1e-4 eV/A is taken relative to that scale here
+    f_scale = max(1.0, np.abs(F_own).max())
+    print(f"largest force component {f_scale:.1f} eV/A", flush=True)
+    assert np.abs(e32.reduce_forces(N, ga["sender_atom"], ga["receiver_atom"]) - F_own).max() <= 1e-4 * f_scale
+    # 1 % of the box (same recipe and density) against the oracle
+    pos, cell, sp = systems.config_system("off_medium", scale=0.01)
+    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"]); ea = neighbors.edge_arrays(nl, sp)
+    ga = neighbors.ghost_edge_arrays(nl, sp)
+    n = len(pos)
+    print(f"1 % box: {n} atoms, {len(ea['r'])} edges, {ga['num_ghost_nodes']} ghost nodes", flush=True)
+    orc = OracleMACE(path)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    F_ref = H.atom_forces(nl, orc.node_forces, n)
+    for dtype, engine in (("float64", eng), ("float32", e32)):
+        engine.compute_ghosted(n, ga["num_ghost_nodes"], ga["node_types"], ga["num_neigh"], ga["neigh_indices"],
+                               ga["neigh_types"], ga["xyz"], ga["r"])
+        Eo = orc.node_energies.sum()
+        assert abs(engine.node_energies.sum() - Eo) <= TOL[dtype]["E"] * abs(Eo), dtype
+        F = engine.reduce_forces(n, ga["sender_atom"], ga["receiver_atom"])
+        fs = max(1.0, np.abs(orc.node_forces).max()) if dtype == "float32" else 1.0
+        assert np.abs(F - F_ref).max() <= TOL[dtype]["F"] * 10 * fs, dtype
+        engine.compute_node_energies_forces(*H.call_args(ea))
+        assert np.abs(engine.node_forces - orc.node_forces).max() <= TOL[dtype]["F"] * fs, dtype
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+def test_capacity_loop_at_reduced_size(gpu, tmp_models, dtype):
+    """The capacity run's loop on 49 920 atoms (4 x 4 x 4 copies of a 780-atom water box): before the first move
+    all 64 copies of an atom get the same energy and force; then every step moves the atoms on the device by
+    N(0, 0.01^2) A, searches the list anew every fifth step and filters the remembered pairs otherwise, and
+    evaluates on the device-resident arrays.  After the last step the result is compared with an evaluation of a
+    list built on the host from the final positions."""
+    import torch
+    from symmetrix_amd import neighbors, systems
+    path, cfg = _model_file(tmp_models, "off_medium", pair_dependent_radial=False)
+    dev = torch.device("cuda:0")
+    reps, n_mol = 4, 260
+    bpos, bcell, bsp = systems.water_box(n_mol, seed=0)
+    nb = len(bpos)
+    offs = np.array([[a, b, c] for a in range(reps) for b in range(reps) for c in range(reps)], dtype=np.float64) * bcell
+    pos = (offs[:, None, :] + bpos[None, :, :]).reshape(-1, 3)
+    species = np.tile(bsp, reps ** 3).astype(np.int32)
+    cell = bcell * reps
+    N = len(pos)
+    r_cut, skin = cfg["r_cut"], 0.6
+    dpos = torch.from_numpy(np.ascontiguousarray(pos)).to(dev)
+    dty = torch.from_numpy(species).to(dev)
+    eng = gpu(path, dtype)
+    dnl = neighbors.DeviceNeighborList()
+    stream = torch.cuda.current_stream().cuda_stream
+    out_E = torch.zeros(N, dtype=torch.float64, device=dev)
+
+    def evaluate(E):
+        p = dnl.ptr
+        out_F = torch.zeros(3 * E, dtype=torch.float64, device=dev)
+        eng.compute_device(N, dty.data_ptr(), p["num_neigh"], p["neigh_indices"], p["neigh_types"], p["xyz"], p["r"], E,
+                           out_E.data_ptr(), out_F.data_ptr(), stream)
+        F = eng.reduce_forces_device(N, p["neigh_indices"])
+        return out_E.cpu().numpy().copy(), F
+
+    E = dnl.build(N, dpos.data_ptr(), dty.data_ptr(), cell, r_cut, skin=skin)
+    print(f"capacity loop: {N} atoms, {E} edges, {dtype}", flush=True)
+    en, F = evaluate(E)
+    e_rep, f_rep = en.reshape(reps ** 3, nb), F.reshape(reps ** 3, nb, 3)
+    e_scale, f_scale = np.abs(e_rep[0]).max(), np.abs(f_rep[0]).max()
+    etol, ftol = (1e-11, 1e-9) if dtype == "float64" else (2e-5, 2e-4)
+    assert np.abs(e_rep - e_rep[0]).max() <= etol * e_scale
+    assert np.abs(f_rep - f_rep[0]).max() <= ftol * max(1.0, f_scale)
+    gen = torch.Generator(device=dev); gen.manual_seed(0)
+    for it in range(12):
+        dpos.add_(torch.randn(dpos.shape, dtype=torch.float64, device=dev, generator=gen), alpha=0.01)
+        if it % 5 == 0:
+            E = dnl.build(N, dpos.data_ptr(), dty.data_ptr(), cell, r_cut, skin=skin)
+        else:
+            E = dnl.update(dpos.data_ptr(), dty.data_ptr(), r_cut)
+        en, F = evaluate(E)
+        assert np.isfinite(en).all() and np.isfinite(F).all()
+        if it % 4 == 0:
+            print(f"  step {it}: {E} edges, E = {en.sum():.6f}", flush=True)
+    # the final state from a list built on the host (atoms that left the cell are folded in there)
+    final = dpos.cpu().numpy()
+    nl = neighbors.neighbor_list(final, cell, r_cut); ea = neighbors.edge_arrays(nl, species)
+    assert len(ea["r"]) == E
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    e_host = eng.node_energies
+    F_host = eng.reduce_forces(N, nl["j"])
+    tol = TOL[dtype]
+    fs = max(1.0, np.abs(F).max()) if dtype == "float32" else 1.0
+    assert abs(e_host.sum() - en.sum()) <= tol["E"] * abs(en.sum())
+    assert np.abs(F_host - F).max() <= tol["F"] * 10 * fs

@@ -138,6 +138,7 @@ struct EngineBase {
     virtual void set_array(const char* name, const double* in, long n) = 0;
     virtual void fill_array(const char* name, long n, double value) = 0;
     virtual void forces_view(ForcesView* v) = 0;
+    virtual void check_device_status() = 0;
     virtual void reduce_forces(int num_atoms, const int* sender_atom, const int* receiver_atom,
                                double* atom_forces, double* virial, bool sender_on_device) = 0;
 
@@ -322,8 +323,42 @@ struct Engine : EngineBase {
         pp_packed.upload(vpk.data(), vpk.size(), s); pp_chunks.upload(vch.data(), vch.size(), s);
         pp_coef.upload(vco.data(), vco.size(), s);
         pp_nent.upload(vne.data(), vne.size(), s);
-        flags.resize(4, s);
+        flags.resize(8, s);
         HIPCHK(hipStreamSynchronize(s));
+    }
+
+    // ---- input checks of device-resident evaluations.  flags[0]: host-array calls (read back at once);
+    // flags[1]: sticky status of device-resident calls, read by the next synchronising call; flags[2], flags[3]:
+    // status word of the running / the next device-resident evaluation, taken in turn (an evaluation clears the
+    // other word for its successor; a captured graph keeps the word it was captured with, so after a failed
+    // evaluation one replay of an older graph may be skipped as well: the sticky word reports either).
+    long device_calls = 0;
+    int* guard_status = nullptr;   // status word of the running evaluation (nullptr: host-array call, checked already)
+    InputGuard input_guard(int N)
+    {
+        InputGuard g;
+        if (!guard_status) return g;
+        g.status = guard_status;
+        g.next_status = flags.p + 2 + (guard_status == flags.p + 2 ? 1 : 0);
+        g.sticky = flags.p + 1;
+        g.first_neigh = first_neigh.p; g.n_first = N + 1;
+        g.tstart = t_start.p; g.n_tstart = hm.T + 1;
+        return g;
+    }
+    void check_device_status() override
+    {
+        if (!device_calls) return;
+        int f = 0;
+        HIPCHK(hipMemcpyAsync(&f, flags.p + 1, sizeof(int), hipMemcpyDeviceToHost, stream));
+        HIPCHK(hipStreamSynchronize(stream));
+        if (!f) return;
+        HIPCHK(launch_fill<int>(flags.p + 1, 1, 0, stream));
+        if (f & 1)
+            throw Error(SMX_EINVAL, "a device-resident evaluation was skipped: node_types / neigh_types / neigh_indices hold an "
+                                    "index outside the model or the node range, or num_neigh does not add up to the number "
+                                    "of edges (its node energies are NaN)");
+        throw Error(SMX_ERANGE, "a device-resident evaluation was skipped: an edge length lies outside (0, r_cut) "
+                                "(its node energies are NaN)");
     }
 
     // Regroup a radial table per channel slice, or return 0 when the slice path does not apply.
@@ -448,7 +483,7 @@ struct Engine : EngineBase {
         s_list.size_to((size_t)E1, s);
         scan_tmp.size_to((size_t)rows / 1024 + 2, s);
         HIPCHK(launch_sender_lists(neigh_indices, (int)E1, rows, s_count.p, s_start.p, s_count.p + rows, s_list.p, scan_tmp.p,
-                                   senders_counted ? 2 : 0, senders_counted ? s_rank.p : nullptr, s));
+                                   senders_counted ? 2 : 0, senders_counted ? s_rank.p : nullptr, s, input_guard(N_geo)));
         senders_counted = false;
         counters_clean = 2L * rows;   // every build leaves its counters and cursors at zero
         sender_rows = rows;
@@ -724,6 +759,7 @@ struct Engine : EngineBase {
         p.H1 = H1.p; p.M1 = M1.p; p.W_H1 = H2w_H1.p; p.W_M1 = H2w_M1.p;
         p.H2 = H2.p; p.H2_adj = H2_adj.p; p.H1_adj = H1_adj.p; p.M1_adj = M1_adj.p;
         p.node_energies = node_energies.p; p.zero_energies = zero_energies ? 1 : 0; p.energies_copy = energies_copy;
+        p.guard = guard_status;
         HIPCHK(launch_tail_fused<F>(p, stream));
         energies_copy = nullptr;
     }
@@ -737,7 +773,7 @@ struct Engine : EngineBase {
         if (rows < N || H2.n < (size_t)N * k) throw Error(SMX_EINVAL, "readouts called before H1 and H2 exist for these nodes");
         HIPCHK(launch_readout_fused<F>(N, rows, k, nlm, node_types, E0.p, ro1.p, ro2_w1.p, ro2_w2.p, hm.readout_2_scale,
                                        H1.p, H2.p, H2_adj.p, H1_adj.p, node_energies.p, zero_energies ? 1 : 0,
-                                       energies_copy, stream));
+                                       energies_copy, guard_status, stream));
         energies_copy = nullptr;
     }
     // node counts for which compute() left A1_adj / A0_adj unwritten (-1: they are current)
@@ -897,7 +933,22 @@ struct Engine : EngineBase {
                  const double* rr, long E_, bool on_device, double* d_energies, double* d_forces, int N_local,
                  long E_local) override
     {
+        try {
+            compute_impl(N, nt, nn, ni, nty, x, rr, E_, on_device, d_energies, d_forces, N_local, E_local);
+        } catch (...) {
+            // whatever was half built is not trusted by the next call
+            senders_counted = false; counters_clean = 0; sender_rows = -1; guard_status = nullptr;
+            energies_copy = nullptr; forces_copy = nullptr;
+            throw;
+        }
+        guard_status = nullptr;
+    }
+    void compute_impl(int N, const int* nt, const int* nn, const int* ni, const int* nty, const double* x,
+                      const double* rr, long E_, bool on_device, double* d_energies, double* d_forces, int N_local,
+                      long E_local)
+    {
         if (N < 0 || E_ < 0) throw Error(SMX_EINVAL, "negative num_nodes or num_edges");
+        if (E_ > 2147483647L) throw Error(SMX_EINVAL, "more than 2^31 - 1 edges: edge offsets are 32-bit");
         // ghost nodes (the last N - N1 nodes and their edges) go through layer 0 only: their H1 rows feed the
         // local receivers, their adjoint comes back through H1_adj (pair_symmetrix_mace.cpp:662-698)
         const int N1 = N_local < 0 ? N : N_local;
@@ -917,7 +968,14 @@ struct Engine : EngineBase {
         stage_begin(ST_PREP);
         set_geometry_ptrs(N, nt, nn, ni, nty, x, rr, E_, on_device);
         if (N1 < N) E1 = E_local;
-        // range checks come before any kernel that uses these integers as indices
+        // range checks come before any kernel that uses these integers as indices: host arrays are checked with a
+        // read-back below; device arrays inside the list preparation, whose last launch empties the lists when a
+        // check failed (input_guard)
+        guard_status = nullptr;
+        if (on_device) {
+            guard_status = flags.p + 2 + (int)(device_calls & 1);
+            ++device_calls;
+        }
         if (on_device && N <= 65536) {
             // one launch for first_neigh, degree order, species groups and the sender histogram
             hipStream_t s = stream;
@@ -928,13 +986,23 @@ struct Engine : EngineBase {
             scan_tmp.size_to((size_t)N / 1024 + 2, s);
             if (s_count.p != before || counters_clean < 2L * N) HIPCHK(launch_fill<int>(s_count.p, 2L * N, 0, s));
             s_rank.size_to((size_t)E1, s);
+            InputChecks chk;
+            chk.status = guard_status; chk.neigh_types = neigh_types; chk.r = r; chk.r_cut = hm.r_cut; chk.num_edges = E;
+            chk.num_local_nodes = N1;
             HIPCHK(launch_node_lists_count(num_neigh, N, first_neigh.p, recv_order.p, node_types, hm.T, t_start.p, t_perm.p,
-                                           neigh_indices, E1, N, s_count.p, s_rank.p, s));
+                                           neigh_indices, E1, N, s_count.p, s_rank.p, chk, s));
             N_geo = N;
             senders_counted = true;
         } else {
             build_first_neigh(N);
             if (!on_device) validate(N, N);
+            else {
+                HIPCHK(launch_check_counts(num_neigh, N, first_neigh.p, N1, E, E1, guard_status, stream));
+                HIPCHK(launch_check_range(node_types, N, hm.T, guard_status, stream));
+                HIPCHK(launch_check_range(neigh_types, E, hm.T, guard_status, stream));
+                HIPCHK(launch_check_range(neigh_indices, E1, N, guard_status, stream));
+                HIPCHK(launch_check_r(r, E, hm.r_cut, guard_status, stream));
+            }
             build_type_groups(N);
         }
         sender_rows = -1;
@@ -1683,6 +1751,7 @@ int smx_get_array(smx_model* m, const char* name, double* out, long cap, long* n
 {
     return guarded([&] {
         if (!name) throw smx::Error(SMX_EINVAL, "null name");
+        E(m).check_device_status();
         E(m).get_array(name, out, cap, n);
     });
 }
@@ -1734,7 +1803,11 @@ int smx_get_stage_times(smx_model* m, float* ms, int cap, int* n)
 }
 int smx_synchronize(smx_model* m)
 {
-    return guarded([&] { HIPCHK(hipStreamSynchronize(E(m).stream)); });
+    return guarded([&] {
+        auto& e = E(m);
+        HIPCHK(hipStreamSynchronize(e.stream));
+        e.check_device_status();
+    });
 }
 int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const int* receiver_atom,
                       double* atom_forces, double* virial)

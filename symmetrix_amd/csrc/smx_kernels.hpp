@@ -152,8 +152,33 @@ hipError_t launch_degree_order(int N, const int* first_neigh, int* order, hipStr
 // counters_are_zero: 0 = clear count and cursor first, 1 = they are zero, 2 = the histogram is already in count and
 // rank[E] holds every entry's place inside its bucket (launch_node_lists_count);
 // count and cursor are zero again when the launches have run
+// Guard of a device-resident evaluation, carried by the last launch of the sender-list build: when this
+// evaluation's status word is raised, first_neigh[n_first] and tstart[n_tstart] are zeroed (no edges, no species
+// groups: the kernels that follow then touch no unchecked index), the status is ORed into the sticky word the host
+// reads later, and the status word of the next evaluation is cleared.  status == nullptr: no guard.
+struct InputGuard {
+    const int* status = nullptr;
+    int* next_status = nullptr;
+    int* sticky = nullptr;
+    int* first_neigh = nullptr; int n_first = 0;
+    int* tstart = nullptr; int n_tstart = 0;
+};
+// What launch_node_lists_count checks besides the sender rows when status is not null: species of nodes and edges,
+// edge lengths inside (0, r_cut), no negative count, counts adding up to num_edges (all nodes) and to the key
+// count (the first num_local_nodes nodes).  Bits: 1 = index or count, 2 = edge length.
+struct InputChecks {
+    int* status = nullptr;
+    const int* neigh_types = nullptr;
+    const double* r = nullptr;
+    double r_cut = 0.0;
+    long num_edges = 0;
+    int num_local_nodes = 0;
+};
 hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
-                               int* slist, int* block_sums, int counters_are_zero, const int* rank, hipStream_t s);
+                               int* slist, int* block_sums, int counters_are_zero, const int* rank, hipStream_t s,
+                               const InputGuard& guard = InputGuard());
+hipError_t launch_check_counts(const int* num_neigh, int N, const int* first_neigh, int num_local_nodes, long num_edges,
+                               long num_local_edges, int* status, hipStream_t s);
 // first_neigh, degree order, species groups and `zero_n` cleared counters in one single-block launch
 // (N <= 65536; larger systems use the separate launches, where the extra launches do not matter)
 hipError_t launch_node_lists(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
@@ -162,7 +187,7 @@ hipError_t launch_node_lists(const int* num_neigh, int N, int* first_neigh, int*
 // each entry took in its bucket; the counters must be zero on entry (every sender-list build leaves them so)
 hipError_t launch_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
                                    int* tstart, int* perm, const int* key, long n, int rows, int* count, int* rank,
-                                   hipStream_t s);
+                                   const InputChecks& chk, hipStream_t s);
 hipError_t launch_type_groups(const int* node_types, int N, int T, int* tcount, int* tstart, int* cursor,
                               int* perm, int* block_sums, hipStream_t s);
 // flags[0] |= 1 if any index is outside [0, limit)
@@ -239,7 +264,7 @@ template <typename F>
 hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,
                                 const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
-                                double* energies_copy, hipStream_t s);
+                                double* energies_copy, const int* guard, hipStream_t s);
 // H2 (mace.cpp:820-845), the readout tail and reverse_H2 (mace.cpp:847-874) in one launch; K a multiple of 16
 // up to 128 (tail_fused_ok).  Atoms grouped by species (perm, tstart); H1_adj [rows][num_LM][K] is written
 // whole (seed plus the adjoint of H2 in the scalar block, zero elsewhere), M1_adj [N][K] too.
@@ -253,6 +278,7 @@ struct TailParams {
     const double* W_M1;      // [K][K]
     double* H2; double* H2_adj; F* H1_adj; F* M1_adj;
     double* node_energies; int zero_energies; double* energies_copy;
+    const int* guard;        // status word of a device-resident evaluation (or null): raised -> energies are NaN
 };
 bool tail_fused_ok(int K);
 template <typename F> hipError_t launch_tail_fused(const TailParams<F>& p, hipStream_t s);

@@ -94,10 +94,24 @@ __global__ void k_place(const int* key, long n, int rows, const int* start, int*
 constexpr int SORT_LDS = 1024;
 // The bucket's counter and cursor are dead by now: they are cleared here, so that the next list build
 // finds them at zero without a launch of its own.
-__global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows, int* list, int* count, int* cursor)
+// With a guard (device-resident callers, whose arrays no host code has looked at): when the checks of this
+// evaluation raised its status word, the CSR offsets and the species groups are set to "no edges, no nodes", so
+// that no later kernel of the evaluation uses an unchecked integer as an address; the status goes into the sticky
+// word the host reads at its next synchronising call, and the word of the next evaluation is cleared.
+__global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows, int* list, int* count, int* cursor,
+                                                     InputGuard g)
 {
     __shared__ int buf[SORT_LDS];
     const int j = blockIdx.x;
+    if (g.status) {
+        const int st = *g.status;
+        if (st) {
+            for (int i = j * 64 + threadIdx.x; i < g.n_first; i += gridDim.x * 64) g.first_neigh[i] = 0;
+            for (int i = j * 64 + threadIdx.x; i < g.n_tstart; i += gridDim.x * 64) g.tstart[i] = 0;
+            if (j == 0 && threadIdx.x == 0) atomicOr(g.sticky, st);
+        }
+        if (j == 0 && threadIdx.x == 0) *g.next_status = 0;
+    }
     if (threadIdx.x == 0) { count[j] = 0; cursor[j] = 0; }
     const int s0 = start[j], n = start[j + 1] - s0;
     if (n <= 1) return;
@@ -161,7 +175,7 @@ __device__ void degree_order_body(int N, const int* first_neigh, int* order)
     start[tid] = 0; cur[tid] = 0;
     __syncthreads();
     for (int i = tid; i < N; i += 1024) {
-        const int d = min(first_neigh[i + 1] - first_neigh[i], 1023);
+        const int d = min(max(first_neigh[i + 1] - first_neigh[i], 0), 1023);   // a negative count must not index below the table
         atomicAdd(&start[1023 - d], 1);
     }
     __syncthreads();
@@ -181,7 +195,7 @@ __device__ void degree_order_body(int N, const int* first_neigh, int* order)
     start[tid] = base + incl - c;
     __syncthreads();
     for (int i = tid; i < N; i += 1024) {
-        const int b = 1023 - min(first_neigh[i + 1] - first_neigh[i], 1023);
+        const int b = 1023 - min(max(first_neigh[i + 1] - first_neigh[i], 0), 1023);
         order[start[b] + atomicAdd(&cur[b], 1)] = i;
     }
 }
@@ -249,14 +263,23 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists(const int* num_neigh,
 }
 // The same with the sender histogram in the same launch: block 0 forms the node lists, the other blocks
 // count the senders (counters at zero on entry), which does not depend on the node lists.
+// With `chk.status` set the launch also checks everything the later kernels use as an address or a table argument
+// (species, sender rows, edge lengths, counts that add up to the edge totals) and raises bits in the status word.
 __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order,
                                                                 const int* node_types, int T, int* tstart, int* perm,
-                                                                const int* key, long n, int rows, int* count, int* rank)
+                                                                const int* key, long n, int rows, int* count, int* rank,
+                                                                InputChecks chk)
 {
     extern __shared__ int sh[];
     if (blockIdx.x == 0) {
         scan_single_body(num_neigh, first_neigh, N);
         __syncthreads();   // first_neigh, written by this block, is read back below
+        if (chk.status) {
+            int bad = 0;
+            for (int i = threadIdx.x; i < N; i += SCAN_BLOCK) bad |= (num_neigh[i] < 0) | (node_types[i] < 0) | (node_types[i] >= T);
+            if (threadIdx.x == 0) bad |= (first_neigh[N] != (int)chk.num_edges) | (first_neigh[chk.num_local_nodes] != (int)n);
+            if (bad) atomicOr(chk.status, 1);
+        }
         degree_order_body(N, first_neigh, order);
         __syncthreads();
         type_groups_body(node_types, N, T, tstart, perm, sh);
@@ -265,7 +288,29 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_
     for (long i = (long)(blockIdx.x - 1) * SCAN_BLOCK + threadIdx.x; i < n; i += (long)(gridDim.x - 1) * SCAN_BLOCK) {
         const int j = key[i];
         if (j >= 0 && j < rows) rank[i] = atomicAdd(&count[j], 1);   // the entry's place inside its bucket
+        else if (chk.status) atomicOr(chk.status, 1);
     }
+    if (chk.status) {
+        // species and length of every edge (layer 0 covers the edges of ghost receivers as well)
+        int bad = 0;
+        for (long i = (long)(blockIdx.x - 1) * SCAN_BLOCK + threadIdx.x; i < chk.num_edges; i += (long)(gridDim.x - 1) * SCAN_BLOCK) {
+            const int t = chk.neigh_types[i];
+            const double rr = chk.r[i];
+            bad |= (t < 0 || t >= T) ? 1 : 0;
+            bad |= (rr > 0.0 && rr < chk.r_cut) ? 0 : 2;
+        }
+        if (bad) atomicOr(chk.status, bad);
+    }
+}
+// the same checks as separate work for lists too long for the single-block scan
+__global__ void k_check_counts(const int* num_neigh, int N, const int* first_neigh, int num_local_nodes, long num_edges,
+                               long num_local_edges, int* status)
+{
+    int bad = 0;
+    for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < N; i += (long)gridDim.x * blockDim.x) bad |= num_neigh[i] < 0;
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+        bad |= (first_neigh[N] != (int)num_edges) | (first_neigh[num_local_nodes] != (int)num_local_edges);
+    if (bad) atomicOr(status, 1);
 }
 // placement of entries that know their place inside the bucket: no atomics
 __global__ void k_place_ranked(const int* key, const int* rank, long n, int rows, const int* start, int* list)
@@ -280,12 +325,21 @@ __global__ void k_place_ranked(const int* key, const int* rank, long n, int rows
 
 hipError_t launch_node_lists_count(const int* num_neigh, int N, int* first_neigh, int* order, const int* node_types, int T,
                                    int* tstart, int* perm, const int* key, long n, int rows, int* count, int* rank,
-                                   hipStream_t s)
+                                   const InputChecks& chk, hipStream_t s)
 {
     if (N <= 0 || N > 64 * SCAN_BLOCK || T <= 0) return hipErrorInvalidValue;
-    const unsigned nb = 1 + (unsigned)std::min<long>((n + SCAN_BLOCK - 1) / SCAN_BLOCK, 2048);
+    const long work = chk.status ? std::max(n, chk.num_edges) : n;
+    const unsigned nb = 1 + (unsigned)std::max<long>(1, std::min<long>((work + SCAN_BLOCK - 1) / SCAN_BLOCK, 2048));
     hipLaunchKernelGGL(k_node_lists_count, dim3(nb), dim3(SCAN_BLOCK), 2 * T * sizeof(int), s, num_neigh, N, first_neigh,
-                       order, node_types, T, tstart, perm, key, n, rows, count, rank);
+                       order, node_types, T, tstart, perm, key, n, rows, count, rank, chk);
+    return hipGetLastError();
+}
+hipError_t launch_check_counts(const int* num_neigh, int N, const int* first_neigh, int num_local_nodes, long num_edges,
+                               long num_local_edges, int* status, hipStream_t s)
+{
+    if (N > 0)
+        hipLaunchKernelGGL(k_check_counts, dim3(std::min<unsigned>(nblk(N, 256), 1024u)), dim3(256), 0, s, num_neigh, N,
+                           first_neigh, num_local_nodes, num_edges, num_local_edges, status);
     return hipGetLastError();
 }
 
@@ -312,7 +366,8 @@ hipError_t launch_scan_exclusive(const int* in, int* out, int n, int* block_sums
 }
 
 hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, int* sstart, int* cursor,
-                               int* slist, int* block_sums, int counters_are_zero, const int* rank, hipStream_t s)
+                               int* slist, int* block_sums, int counters_are_zero, const int* rank, hipStream_t s,
+                               const InputGuard& guard)
 {
     if (rows <= 0) return hipSuccess;
     const bool counted = counters_are_zero == 2;   // the histogram came with the node lists
@@ -332,8 +387,10 @@ hipError_t launch_sender_lists(const int* gather, int E, int rows, int* count, i
             hipLaunchKernelGGL(k_place_ranked, dim3(nblk(E, 256)), dim3(256), 0, s, gather, rank, (long)E, rows, sstart, slist);
         else
             hipLaunchKernelGGL(k_place, dim3(nblk(E, 256)), dim3(256), 0, s, gather, (long)E, rows, sstart, cursor, slist);
-        hipLaunchKernelGGL(k_sort_buckets, dim3(rows), dim3(64), 0, s, sstart, rows, slist, count, cursor);
     }
+    // the guard's bookkeeping rides on this launch, so it also runs for an edge list that claims to be empty
+    if (E > 0 || guard.status)
+        hipLaunchKernelGGL(k_sort_buckets, dim3(rows), dim3(64), 0, s, sstart, rows, slist, count, cursor, guard);
     return hipGetLastError();
 }
 
@@ -607,9 +664,18 @@ __global__ __launch_bounds__(256) void k_readout_fused(int N, int rows, int K, i
                                                        const double* E0, const double* w1, const double* W1,
                                                        const double* w2, double scale, const F* H1, const double* H2,
                                                        double* H2_adj, F* H1_adj, double* node_energies,
-                                                       int zero_energies, double* energies_copy)
+                                                       int zero_energies, double* energies_copy, const int* guard)
 {
     extern __shared__ double rsm[];
+    if (guard && *guard) {
+        // unchecked species indices: no table lookup, the energies say so
+        const int i = blockIdx.x * 16 + (threadIdx.x >> 4);
+        if ((threadIdx.x & 15) == 0 && i < N) {
+            node_energies[i] = __builtin_nan("");
+            if (energies_copy) energies_copy[i] = __builtin_nan("");
+        }
+        return;
+    }
     const int ldw = K + 1;                 // rows of W1 start two banks apart
     double* W = rsm;                       // [16][K + 1]
     double* hg = W + 16 * ldw;             // [16 nodes][16]
@@ -689,6 +755,15 @@ __global__ __launch_bounds__(TAIL_BLOCK) void k_tail_fused(const TailParams<F> p
     __shared__ int node_s[16];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int width = p.num_LM * K;
+    if (p.guard && *p.guard) {
+        // the inputs of this evaluation failed their checks and the species groups are empty: the energies say so
+        const int i = blockIdx.x * 16 + tid;
+        if (tid < 16 && i < p.N) {
+            p.node_energies[i] = __builtin_nan("");
+            if (p.energies_copy) p.energies_copy[i] = __builtin_nan("");
+        }
+        return;
+    }
     // rows beyond the atoms (ghost rows of H1_adj) are cleared by all blocks together
     {
         const long ghost = (long)(p.rows - p.N) * width;
@@ -854,7 +929,7 @@ template <typename F>
 hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,
                                 const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
-                                double* energies_copy, hipStream_t s)
+                                double* energies_copy, const int* guard, hipStream_t s)
 {
     if (rows < N) return hipErrorInvalidValue;
     if (rows <= 0) return hipSuccess;
@@ -867,11 +942,11 @@ hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* n
     }
     hipLaunchKernelGGL(k_readout_fused<F>, dim3((rows + 15) / 16), dim3(256), lds, s, N, rows, K, num_LM, node_types,
                        atomic_energies, w1, W1, w2, scale, H1, H2, H2_adj, H1_adj, node_energies, zero_energies,
-                       energies_copy);
+                       energies_copy, guard);
     return hipGetLastError();
 }
-template hipError_t launch_readout_fused<double>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const double*, const double*, double*, double*, double*, int, double*, hipStream_t);
-template hipError_t launch_readout_fused<float>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const float*, const double*, double*, float*, double*, int, double*, hipStream_t);
+template hipError_t launch_readout_fused<double>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const double*, const double*, double*, double*, double*, int, double*, const int*, hipStream_t);
+template hipError_t launch_readout_fused<float>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const float*, const double*, double*, float*, double*, int, double*, const int*, hipStream_t);
 
 
 // ===========================================================================

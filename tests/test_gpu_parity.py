@@ -608,3 +608,52 @@ def test_a_step_captured_in_a_hip_graph_replays_bitwise(gpu, tmp_models, L_max):
         g.replay()
         torch.cuda.synchronize()
         assert torch.equal(oE, refE) and torch.equal(oF, refF)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("L_max,big", [(0, False), (1, False), (0, True)])
+def test_device_resident_call_checks_its_inputs_on_the_device(gpu, tmp_models, L_max, big):
+    """Arrays handed over as device addresses are checked inside the list preparation; when a check fails, the
+    evaluation runs on emptied lists (no unchecked integer is used as an address), the node energies come back as
+    NaN and the next synchronising call raises.  Every kernel exits normally; the call after is unaffected.
+    `big`: more than 65 536 atoms, where the preparation is made of separate launches."""
+    import torch
+    from symmetrix_amd import neighbors, systems
+    model = H.tiny_model(K=16 if big else 32, L_max=L_max, n_pts=48, seed=40 + L_max, r_cut=3.0 if big else 4.0)
+    path = H.write_model(model, tmp_models / f"guard{L_max}{int(big)}.json")
+    if big:
+        pos, cell, sp = systems.fcc_alloy((26, 26, 25), n_species=3, seed=1)     # 67 600 atoms
+    else:
+        pos, cell, sp = H.small_system(40, seed=5)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    N, E = len(sp), len(ea["r"])
+    dev = torch.device("cuda:0")
+    t = lambda a, dt: torch.from_numpy(np.ascontiguousarray(a)).to(dev, dtype=dt)
+    names = ["node_types", "num_neigh", "neigh_indices", "neigh_types", "xyz", "r"]
+    good = {k: t(ea[k], torch.float64 if k in ("xyz", "r") else torch.int32) for k in names}
+    oE = torch.zeros(N, dtype=torch.float64, device=dev); oF = torch.zeros(3 * E, dtype=torch.float64, device=dev)
+    eng = gpu(path, "float64")
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def run(d):
+        eng.compute_device(N, *[d[k].data_ptr() for k in names], E, oE.data_ptr(), oF.data_ptr(), stream)
+        torch.cuda.synchronize()
+
+    run(good)
+    eng.synchronize()
+    e_ref, f_ref = oE.clone(), oF.clone()
+    assert torch.isfinite(e_ref).all()
+    bad_cases = {"sender row": ("neigh_indices", 5, N + 3), "edge species": ("neigh_types", 0, 3),
+                 "node species": ("node_types", 1, -1), "counts": ("num_neigh", 0, int(ea["num_neigh"][0]) + 1),
+                 "edge length": ("r", 3, 2.0 * model["r_cut"])}
+    for what, (key, pos_, value) in bad_cases.items():
+        d = dict(good); d[key] = good[key].clone(); d[key][pos_] = value
+        print(f"bad {what} (L_max {L_max}, {N} atoms)", flush=True)
+        run(d)
+        assert torch.isnan(oE).all(), what
+        with pytest.raises(ValueError):
+            eng.synchronize()
+        eng.synchronize()                       # reported once
+        run(good)
+        eng.synchronize()
+        assert torch.equal(oE, e_ref) and torch.equal(oF, f_ref), what

@@ -167,6 +167,10 @@ struct Engine : EngineBase {
     // channel-slice tables (see smx_kernels_slice.hip); CH = 0 disables the path for that layer
     DVec<F> tabS0, tabS1;
     int slice_CH0 = 0, slice_CH1 = 0, slice_W = 0, slice_U0 = 0, slice_U1 = 0, num_cus = 0;
+    // the same slices with the row padding of the adjoint kernel that gives every edge a lane of its own
+    // (empty when the forward table already has that row length, or when the kernel does not apply)
+    DVec<F> tabE0, tabE1;
+    bool edge_lanes = false;
     double cdiag1[16] = {};
     DVec<double> fpart;
     DVec<double> H2w_H1, H2w_M1, ro1, ro2_w1, ro2_w2, E0;
@@ -362,7 +366,7 @@ struct Engine : EngineBase {
     }
 
     // Regroup a radial table per channel slice, or return 0 when the slice path does not apply.
-    int build_slice_table(const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst, hipStream_t s)
+    int build_slice_table(const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst, DVec<F>& edst, hipStream_t s)
     {
         const int R = hm.spl_nodes - 1, Kc = hm.K, U = (int)tables.size();
         if (nspl != 4 * Kc || U > 4) return 0;
@@ -396,13 +400,25 @@ struct Engine : EngineBase {
             dst.upload(buf.data(), buf.size(), s);
             HIPCHK(hipStreamSynchronize(s));
             slice_W = W;
+            // adjoint kernel with one lane per edge: CH channels are 32 bytes, table slice and the staged adjoint
+            // rows of twelve wavefronts fit the LDS
+            edge_lanes = CH * sizeof(F) == 32 && slice_edge_lds_bytes<F>(hm.spl_nodes) <= lds_cap &&
+                         !std::getenv("SMX_SLICE_BWD_ROWS");
+            if (edge_lanes && slice_edge_row_elements<F>() != W) {
+                const int We = slice_edge_row_elements<F>();
+                std::vector<F> eb((size_t)S * U * R * We, F(0));
+                for (size_t rowi = 0; rowi < (size_t)S * U * R; ++rowi)
+                    std::copy(buf.begin() + rowi * W, buf.begin() + rowi * W + 16 * CH, eb.begin() + rowi * We);
+                edst.upload(eb.data(), eb.size(), s);
+                HIPCHK(hipStreamSynchronize(s));
+            }
             return CH;
         }
         return 0;
     }
     void build_slices(hipStream_t s)
     {
-        slice_CH0 = build_slice_table(hm.tables0, hm.nspl0, tabS0, s);
+        slice_CH0 = build_slice_table(hm.tables0, hm.nspl0, tabS0, tabE0, s);
         slice_U0 = (int)hm.tables0.size();
         if (hm.L_max == 0) {
             // layer 1 qualifies when every output slot lm is fed by harmonic lm alone
@@ -415,18 +431,23 @@ struct Engine : EngineBase {
                 }
             }
             if (diag) {
-                slice_CH1 = build_slice_table(hm.tables1, hm.nspl1, tabS1, s);
+                slice_CH1 = build_slice_table(hm.tables1, hm.nspl1, tabS1, tabE1, s);
                 slice_U1 = (int)hm.tables1.size();
             }
         }
     }
-    SliceParams<F> slice_params(int layer, int N)
+    SliceParams<F> slice_params(int layer, int N, bool adjoint = false)
     {
         SliceParams<F> p{};
         p.a = agg_params(layer, N);
         p.tabS = layer == 0 ? tabS0.p : tabS1.p;
         p.U = layer == 0 ? slice_U0 : slice_U1;
         p.W = slice_W;
+        if (adjoint && edge_lanes) {
+            p.edge_lanes = 1;
+            DVec<F>& te = layer == 0 ? tabE0 : tabE1;
+            if (te.p) { p.tabS = te.p; p.W = slice_edge_row_elements<F>(); }
+        }
         p.CH = layer == 0 ? slice_CH0 : slice_CH1;
         for (int q = 0; q < 16; ++q) p.cdiag[q] = layer == 0 ? 1.0 : cdiag1[q];
         p.E = E;
@@ -810,7 +831,7 @@ struct Engine : EngineBase {
         msg.size_to((size_t)E1 * nlm * k, stream);
         stage_begin(ST_AGG1B);
         if (slice_CH1) {
-            auto sp = slice_params(1, N);
+            auto sp = slice_params(1, N, true);
             const int S = (k + sp.CH - 1) / sp.CH;
             fpart.size_to((size_t)S * 3 * E, stream);
             sp.a.d_out = dPhi1.p; sp.a.msg = msg.p; sp.fpart = fpart.p;
@@ -893,7 +914,7 @@ struct Engine : EngineBase {
         need(xyz, "xyz"); need(r, "r");
         node_forces.resize((size_t)3 * E, stream);
         if (slice_CH0) {
-            auto sp = slice_params(0, N);
+            auto sp = slice_params(0, N, true);
             const int S = (K() + sp.CH - 1) / sp.CH;
             fpart.size_to((size_t)S * 3 * E, stream);
             sp.a.d_out = Phi0.p; sp.a.msg = nullptr; sp.fpart = fpart.p;

@@ -74,7 +74,11 @@ struct SliceParams {
     long E;
     int num_cus;
     const int* order;     // [num_nodes] receivers by decreasing degree: entry 4t+q is row q of task t
+    int edge_lanes;       // bwd: one lane per edge (tabS rows padded to slice_edge_row_elements, CH * sizeof(F) = 32)
 };
+// row length (elements) and LDS bytes of the adjoint kernel with one lane per edge
+template <typename F> int slice_edge_row_elements();
+template <typename F> size_t slice_edge_lds_bytes(int spl_nodes);
 // padded row length W (elements) of the per-slice table for CH channels, 0 if the kernels cannot take that CH
 template <typename F> int slice_row_elements(int CH);
 template <typename F> hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s);

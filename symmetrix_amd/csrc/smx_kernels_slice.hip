@@ -311,6 +311,165 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     }
 }
 
+// ---------------------------------------------------------------------------
+// Adjoint kernel, one lane per edge.  A 16-lane row serves one receiver and takes 16 of its edges at a time;
+// every lane holds all CH channels of the slice for its edge (CH * sizeof(F) = 32 bytes: one sender-row load, two
+// 16-byte LDS reads per coefficient).  The direction, the harmonics and their gradient are formed once per
+// (edge, slice) instead of once per (edge, channel): for every harmonic the lane first sums over its channels,
+//     P = sum_c d[lm][c] h[c] R_l[c],   Q = sum_c d[lm][c] h[c] R'_l[c],
+// and only then multiplies with Y_lm and its gradient.  No lane talks to another one.  The receiver's adjoint
+// rows d[16][CH] (times the coupling constant) are staged per wavefront in the LDS left free by the table slice
+// and read back as broadcasts, one harmonic at a time.  tabS rows here are [4 coefficients][4 paths][CH] padded to
+// W elements with W * sizeof(F) = 16 (mod 32), so that the rows of 16 edges spread over the banks.
+template <typename F, int CH, int BT>
+__global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
+{
+    static_assert(CH * sizeof(F) == 32, "a lane moves its channels as two 16-byte words");
+    extern __shared__ __align__(16) unsigned char smem[];
+    using V = Vec<F, CH>;
+    const F* lds = reinterpret_cast<const F*>(smem);
+    const AggParams<F>& a = p.a;
+    const int slice = blockIdx.x, K = a.K;
+    const int W = p.W, R = a.spl_nodes - 1;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row = lane >> 4, sub = lane & 15;
+    const int kc = slice * CH;
+    const bool whole = kc + CH <= K;                        // all channels of the slice exist
+    F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + (size_t)(wave * 4 + row) * 16 * CH;
+    const int wave_tasks = (a.num_nodes + 3) / 4;
+    const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
+    double* fpart = p.fpart + (size_t)slice * p.E * 3;
+    const F cd_sub = (F)p.cdiag[sub];
+
+    for (int u = 0; u < p.U; ++u) {
+        __syncthreads();
+        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
+        __syncthreads();
+        for (int task = wave_id; task < wave_tasks; task += wave_stride) {
+            const int slot = task * 4 + row;
+            const bool live = slot < a.num_nodes;
+            const int i = live ? p.order[slot] : 0;
+            int e0 = 0, e1 = 0, ti = 0;
+            if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
+            // lane `sub` of the row brings harmonic `sub` of the receiver's adjoint row
+            {
+                V v;
+#pragma unroll
+                for (int c = 0; c < CH; ++c) v.v[c] = F(0);
+                if (live) {
+                    const F* src = a.d_out + ((size_t)i * 16 + sub) * K + kc;
+                    if (whole) v = *reinterpret_cast<const V*>(src);
+                    else {
+#pragma unroll
+                        for (int c = 0; c < CH; ++c) if (kc + c < K) v.v[c] = src[c];
+                    }
+                }
+#pragma unroll
+                for (int c = 0; c < CH; ++c) v.v[c] *= cd_sub;
+                wave_lds_sync();                                   // the previous task's reads are done
+                *reinterpret_cast<V*>(dstage + sub * CH) = v;
+                wave_lds_sync();
+            }
+            const int iters = (e1 - e0 + 15) >> 4;
+            EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0, 0};
+            if (e0 + sub < e1) nx = load_edge(a, e0 + sub);
+            for (int it = 0; it < iters; ++it) {
+                const int e = e0 + it * 16 + sub;
+                bool on = e < e1;
+                const EdgeGeo cu = nx;
+                nx = load_edge(a, min(e + 16, e1 - 1));   // unconditional: a conditional load costs a register copy per value
+                if (on && p.U > 1 && a.pair_table[pair_index(a.T, ti, cu.tj)] != u) on = false;
+                if (!on) continue;
+                // sender row first: its latency hides behind the radial part
+                V h;
+                {
+                    const F* src = a.Hsrc + (size_t)cu.g * K + kc;
+                    if (whole) h = *reinterpret_cast<const V*>(src);
+                    else {
+#pragma unroll
+                        for (int c = 0; c < CH; ++c) h.v[c] = src[min(c, K - 1 - kc)];
+                    }
+                }
+                const double dx = cu.dx, dy = cu.dy, dz = cu.dz, r = cu.r;
+                const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
+                const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
+                const int n = spline_interval(r, a.spl_inv_h, R - 1);
+                const F x = (F)(r - a.spl_h * n);
+                const F* rowp = lds + (size_t)n * W;
+                F Rv[4][CH], Rd[4][CH];
+#pragma unroll
+                for (int l = 0; l < 4; ++l) {
+                    const V c0 = *reinterpret_cast<const V*>(rowp + (0 * 4 + l) * CH);
+                    const V c1 = *reinterpret_cast<const V*>(rowp + (1 * 4 + l) * CH);
+                    const V c2 = *reinterpret_cast<const V*>(rowp + (2 * 4 + l) * CH);
+                    const V c3 = *reinterpret_cast<const V*>(rowp + (3 * 4 + l) * CH);
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) {
+                        Rv[l][c] = c0.v[c] + x * (c1.v[c] + x * (c2.v[c] + x * c3.v[c]));
+                        Rd[l][c] = c1.v[c] + x * (F(2) * c2.v[c] + F(3) * x * c3.v[c]);
+                    }
+                }
+                F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
+                F mg[CH];
+#pragma unroll
+                for (int c = 0; c < CH; ++c) mg[c] = F(0);
+                double vx = ux, vy = uy, vz = uz;
+                // one order l at a time (the fence keeps the harmonics of the next order from being formed early)
+                static_for<0, 4>([&](auto lc) {
+                    constexpr int l = decltype(lc)::value;
+                    F ul[CH];
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) ul[c] = F(0);
+                    F py = F(0);
+                    static_for<0, 2 * l + 1>([&](auto mc) {
+                        constexpr int lm = l * l + decltype(mc)::value;
+                        double y, g0, g1, g2;
+                        ylm_g<lm>(vx, vy, vz, y, g0, g1, g2);
+                        const V dd = *reinterpret_cast<const V*>(dstage + lm * CH);
+                        const F yf = (F)y;
+                        F P = F(0), Q = F(0);
+#pragma unroll
+                        for (int c = 0; c < CH; ++c) {
+                            const F dh = dd.v[c] * h.v[c];
+                            P += dh * Rv[l][c];
+                            Q += dh * Rd[l][c];
+                            ul[c] += dd.v[c] * yf;
+                        }
+                        srad += Q * yf;
+                        wx += P * (F)g0; wy += P * (F)g1; wz += P * (F)g2;
+                        py += P * yf;
+                    });
+                    lterm += py * F(l);
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) mg[c] += Rv[l][c] * ul[c];
+                    order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) pin_value(mg[c]);
+                });
+                if (a.msg) {
+                    F* dstm = a.msg + (size_t)e * K + kc;
+                    if (whole) {
+                        V m;
+#pragma unroll
+                        for (int c = 0; c < CH; ++c) m.v[c] = mg[c];
+                        *reinterpret_cast<V*>(dstm) = m;
+                    } else {
+#pragma unroll
+                        for (int c = 0; c < CH; ++c) if (kc + c < K) dstm[c] = mg[c];
+                    }
+                }
+                // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
+                // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
+                const double sr = (double)srad, lt = (double)lterm;
+                const double ir = rcp_pos(r);
+                fpart[3 * (size_t)e] = -(dx * ir * sr + ((double)wy - uy * lt) * inv);       // original x is permuted axis 1
+                fpart[3 * (size_t)e + 1] = -(dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
+                fpart[3 * (size_t)e + 2] = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
+            }
+        }
+    }
+}
+
 __global__ void k_fpart_reduce(long n3, long stride3, int nslices, const double* fpart, double* forces, int accumulate,
                                double* copy)
 {
@@ -370,9 +529,42 @@ hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s)
     }
 }
 template <typename F>
+static hipError_t launch_slice_bwd_edge(const SliceParams<F>& p, hipStream_t s)
+{
+    constexpr int CH = 32 / (int)sizeof(F), BT = 768;
+    const int S = (p.a.K + CH - 1) / CH;
+    const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F) + (size_t)(BT / 64) * 4 * 16 * CH * sizeof(F);
+    int RG = p.num_cus / S;
+    if (RG < 1) RG = 1;
+    const long tasks_per_slice = ((long)p.a.num_nodes + 3) / 4;
+    if ((long)RG * (BT / 64) > tasks_per_slice) RG = (int)((tasks_per_slice + BT / 64 - 1) / (BT / 64));
+    auto kern = k_slice_bwd_edge<F, CH, BT>;
+    if (lds > 64 * 1024) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+    }
+    hipLaunchKernelGGL(kern, dim3(S, RG), dim3(BT), lds, s, p);
+    return hipGetLastError();
+}
+template <typename F> int slice_edge_row_elements()
+{
+    // [4][4][CH] with CH * sizeof(F) = 32: 512 bytes, plus 16 so that consecutive rows start four banks apart
+    return (512 + 16) / (int)sizeof(F);
+}
+template int slice_edge_row_elements<double>();
+template int slice_edge_row_elements<float>();
+template <typename F> size_t slice_edge_lds_bytes(int spl_nodes)
+{
+    return (size_t)(spl_nodes - 1) * slice_edge_row_elements<F>() * sizeof(F) + (size_t)12 * 4 * 16 * 32;
+}
+template size_t slice_edge_lds_bytes<double>(int);
+template size_t slice_edge_lds_bytes<float>(int);
+
+template <typename F>
 hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s)
 {
     if (p.a.num_nodes <= 0) return hipSuccess;
+    if (p.edge_lanes) return launch_slice_bwd_edge<F>(p, s);
     switch (p.CH) {
     case 2: return launch_slice_t<F, 2, true>(p, s);
     case 4: return launch_slice_t<F, 4, true>(p, s);

@@ -402,8 +402,7 @@ struct Engine : EngineBase {
             slice_W = W;
             // adjoint kernel with one lane per edge: CH channels are 32 bytes, table slice and the staged adjoint
             // rows of twelve wavefronts fit the LDS
-            edge_lanes = CH * sizeof(F) == 32 && slice_edge_lds_bytes<F>(hm.spl_nodes) <= lds_cap &&
-                         !std::getenv("SMX_SLICE_BWD_ROWS");
+            edge_lanes = CH * sizeof(F) == 32 && slice_edge_lds_bytes<F>(hm.spl_nodes) <= lds_cap;
             if (edge_lanes && slice_edge_row_elements<F>() != W) {
                 const int We = slice_edge_row_elements<F>();
                 std::vector<F> eb((size_t)S * U * R * We, F(0));

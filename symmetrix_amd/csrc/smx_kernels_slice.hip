@@ -30,6 +30,16 @@ __device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, si
     for (size_t q = threadIdx.x; q < n; q += blockDim.x) d[q] = s[q];
 }
 
+// The tasks of a block (groups of receivers, largest first) are handed to its wavefronts as they become free: an
+// integer counter in LDS, so that the wavefronts of a block finish together whatever the degrees.  Which wavefront
+// takes a task has no influence on any result (a task's sums are its own).
+__device__ __forceinline__ int next_block_task(int* counter)
+{
+    int j = 0;
+    if ((threadIdx.x & 63) == 0) j = atomicAdd(counter, 1);
+    return __builtin_amdgcn_readfirstlane(j);
+}
+
 struct EdgeGeo {
     double dx, dy, dz, r;
     int g, tj;
@@ -99,13 +109,15 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
 #pragma unroll
     for (int i = 0; i < 4; ++i) poff[i] = ((i + rot) & 3) * CH;
     const int wave_tasks = (a.num_nodes + 3) / 4;
-    const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
+    __shared__ int task_counter;
 
     for (int u = 0; u < p.U; ++u) {
         __syncthreads();
+        if (threadIdx.x == 0) task_counter = 0;
         copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
         __syncthreads();
-        for (int task = wave_id; task < wave_tasks; task += wave_stride) {
+        for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
+             task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
             const int slot = task * 4 + (lane >> 4);
             const bool live = slot < a.num_nodes;
             const int i = live ? p.order[slot] : 0;
@@ -195,14 +207,16 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
 #pragma unroll
     for (int i = 0; i < 4; ++i) poff[i] = ((i + rot) & 3) * CH;
     const int wave_tasks = (a.num_nodes + 3) / 4;
-    const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
+    __shared__ int task_counter;
     double* fpart = p.fpart + (size_t)slice * p.E * 3;
 
     for (int u = 0; u < p.U; ++u) {
         __syncthreads();
+        if (threadIdx.x == 0) task_counter = 0;
         copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
         __syncthreads();
-        for (int task = wave_id; task < wave_tasks; task += wave_stride) {
+        for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
+             task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
             const int slot = task * 4 + (lane >> 4);
             const bool live = slot < a.num_nodes;
             const int i = live ? p.order[slot] : 0;
@@ -321,7 +335,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
 // rows d[16][CH] (times the coupling constant) are staged per wavefront in the LDS left free by the table slice
 // and read back as broadcasts, one harmonic at a time.  tabS rows here are [4 coefficients][4 paths][CH] padded to
 // W elements with W * sizeof(F) = 16 (mod 32), so that the rows of 16 edges spread over the banks.
-template <typename F, int CH, int BT>
+template <typename F, int CH, int BT, int RL>
 __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
 {
     static_assert(CH * sizeof(F) == 32, "a lane moves its channels as two 16-byte words");
@@ -332,52 +346,56 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     const int slice = blockIdx.x, K = a.K;
     const int W = p.W, R = a.spl_nodes - 1;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int row = lane >> 4, sub = lane & 15;
+    constexpr int ROWS = 64 / RL;                            // receivers a wavefront works on at a time
+    const int row = lane / RL, sub = lane % RL;
     const int kc = slice * CH;
     const bool whole = kc + CH <= K;                        // all channels of the slice exist
-    F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + (size_t)(wave * 4 + row) * 16 * CH;
-    const int wave_tasks = (a.num_nodes + 3) / 4;
-    const int wave_id = blockIdx.y * (BT / 64) + wave, wave_stride = gridDim.y * (BT / 64);
+    F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + (size_t)(wave * ROWS + row) * 16 * CH;
+    const int wave_tasks = (a.num_nodes + ROWS - 1) / ROWS;
+    __shared__ int task_counter;
     double* fpart = p.fpart + (size_t)slice * p.E * 3;
-    const F cd_sub = (F)p.cdiag[sub];
 
     for (int u = 0; u < p.U; ++u) {
         __syncthreads();
+        if (threadIdx.x == 0) task_counter = 0;
         copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
         __syncthreads();
-        for (int task = wave_id; task < wave_tasks; task += wave_stride) {
-            const int slot = task * 4 + row;
+        for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
+             task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
+            const int slot = task * ROWS + row;
             const bool live = slot < a.num_nodes;
             const int i = live ? p.order[slot] : 0;
             int e0 = 0, e1 = 0, ti = 0;
             if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
-            // lane `sub` of the row brings harmonic `sub` of the receiver's adjoint row
-            {
+            // the lanes of the row bring the receiver's adjoint rows, one harmonic each per round
+            wave_lds_sync();                                       // the previous task's reads are done
+#pragma unroll
+            for (int lm = sub; lm < 16; lm += RL) {
                 V v;
 #pragma unroll
                 for (int c = 0; c < CH; ++c) v.v[c] = F(0);
                 if (live) {
-                    const F* src = a.d_out + ((size_t)i * 16 + sub) * K + kc;
+                    const F* src = a.d_out + ((size_t)i * 16 + lm) * K + kc;
                     if (whole) v = *reinterpret_cast<const V*>(src);
                     else {
 #pragma unroll
                         for (int c = 0; c < CH; ++c) if (kc + c < K) v.v[c] = src[c];
                     }
                 }
+                const F cd = (F)p.cdiag[lm];
 #pragma unroll
-                for (int c = 0; c < CH; ++c) v.v[c] *= cd_sub;
-                wave_lds_sync();                                   // the previous task's reads are done
-                *reinterpret_cast<V*>(dstage + sub * CH) = v;
-                wave_lds_sync();
+                for (int c = 0; c < CH; ++c) v.v[c] *= cd;
+                *reinterpret_cast<V*>(dstage + lm * CH) = v;
             }
-            const int iters = (e1 - e0 + 15) >> 4;
+            wave_lds_sync();
+            const int iters = (e1 - e0 + RL - 1) / RL;
             EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0, 0};
             if (e0 + sub < e1) nx = load_edge(a, e0 + sub);
             for (int it = 0; it < iters; ++it) {
-                const int e = e0 + it * 16 + sub;
+                const int e = e0 + it * RL + sub;
                 bool on = e < e1;
                 const EdgeGeo cu = nx;
-                nx = load_edge(a, min(e + 16, e1 - 1));   // unconditional: a conditional load costs a register copy per value
+                nx = load_edge(a, min(e + RL, e1 - 1));   // unconditional: a conditional load costs a register copy per value
                 if (on && p.U > 1 && a.pair_table[pair_index(a.T, ti, cu.tj)] != u) on = false;
                 if (!on) continue;
                 // sender row first: its latency hides behind the radial part
@@ -528,23 +546,32 @@ hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s)
     default: return hipErrorInvalidValue;
     }
 }
-template <typename F>
-static hipError_t launch_slice_bwd_edge(const SliceParams<F>& p, hipStream_t s)
+template <typename F, int BT, int RL>
+static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t s)
 {
-    constexpr int CH = 32 / (int)sizeof(F), BT = 768;
+    constexpr int CH = 32 / (int)sizeof(F), ROWS = 64 / RL;
     const int S = (p.a.K + CH - 1) / CH;
-    const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F) + (size_t)(BT / 64) * 4 * 16 * CH * sizeof(F);
+    const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F) + (size_t)(BT / 64) * ROWS * 16 * CH * sizeof(F);
     int RG = p.num_cus / S;
     if (RG < 1) RG = 1;
-    const long tasks_per_slice = ((long)p.a.num_nodes + 3) / 4;
+    const long tasks_per_slice = ((long)p.a.num_nodes + ROWS - 1) / ROWS;
     if ((long)RG * (BT / 64) > tasks_per_slice) RG = (int)((tasks_per_slice + BT / 64 - 1) / (BT / 64));
-    auto kern = k_slice_bwd_edge<F, CH, BT>;
+    auto kern = k_slice_bwd_edge<F, CH, BT, RL>;
     if (lds > 64 * 1024) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
     }
     hipLaunchKernelGGL(kern, dim3(S, RG), dim3(BT), lds, s, p);
     return hipGetLastError();
+}
+// Twelve wavefronts per block and sixteen lanes per receiver measured best (eight lanes per receiver fill the
+// lanes better, 95 % against 80 % at 38 neighbours, but the staged adjoint rows of twice as many receivers leave
+// room for six wavefronts only: 163 / 138 us against 154 / 114 us for the two adjoint stages of the 3 000-atom
+// benchmark in double precision; eight wavefronts with sixteen lanes run like twelve).
+template <typename F>
+static hipError_t launch_slice_bwd_edge(const SliceParams<F>& p, hipStream_t s)
+{
+    return launch_slice_bwd_edge_cfg<F, 768, 16>(p, s);
 }
 template <typename F> int slice_edge_row_elements()
 {

@@ -12,7 +12,10 @@ Prints ONE JSON line.  Besides the driver's fields it carries
   cpu_baseline  the CPU oracle (serial fp64 restatement of the reference path)
                 timed on this host on the same workload
   stages_ms     HIP-event time of every stage of the pipeline
-  fp32_features the same workload in the fp32-feature mode
+  other_precision   the same workload in the other precision mode
+  second_config     (default run) the metric's second configuration: 50 000-atom alloy, K = 128, l <= 1 hidden
+                    features, float32 features, with its own roofline
+  pair_dependent_tables   (default run) the headline workload with one radial table per species pair
 """
 from __future__ import annotations
 
@@ -30,26 +33,42 @@ sys.path.insert(0, HERE)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 
-# kernel behind each edge stage for models with scalar hidden features (L_max = 0) / with l <= 1 features
-STAGE_KERNEL = {
-    "agg0_fwd": ("k_slice_fwd", "k_slice_fwd"), "agg1_fwd": ("k_slice_fwd", "k_agg_fwd"),
-    "agg1_bwd": ("k_slice_bwd", "k_agg_bwd"), "agg0_bwd": ("k_slice_bwd", "k_slice_bwd"),
-    "sender_reduce": ("k_sender_reduce_linear", "k_sender_reduce"),
-}
+# kernel behind each edge stage: channel-slice kernels (scalar hidden features and at most four distinct radial
+# tables) / general kernels
+SLICE_KERNEL = {"agg0_fwd": "k_slice_fwd", "agg1_fwd": "k_slice_fwd", "agg1_bwd": "k_slice_bwd_edge",
+                "agg0_bwd": "k_slice_bwd_edge", "sender_reduce": "k_sender_reduce_linear"}
+GENERAL_KERNEL = {"agg0_fwd": "k_agg_fwd", "agg1_fwd": "k_agg_fwd", "agg1_bwd": "k_agg_bwd", "agg0_bwd": "k_agg_bwd",
+                  "sender_reduce": "k_sender_reduce"}
+EDGE_STAGES = ["agg0_fwd", "agg1_fwd", "agg1_bwd", "sender_reduce", "agg0_bwd"]
 
-# HBM bytes per launch from rocprofv3 counters (FETCH_SIZE x 2.000 + WRITE_SIZE x 1.000 KiB, the factors read off a
-# 1 GiB copy in the same runs), full-size workloads only: profiles/edge_kernels_off_small_hbm_traffic.txt and
-# profiles/edge_kernels_mp_medium_hbm_traffic.txt
-MEASURED_TRAFFIC = {
-    ("off_small", "float64"): {"agg0_fwd": 78.8e6, "agg1_fwd": 106.2e6, "agg1_bwd": 436.0e6, "agg0_bwd": 257.9e6,
-                               "sender_reduce": 95.7e6},
-    ("off_small", "float32"): {"agg0_fwd": 58.8e6, "agg1_fwd": 86.2e6, "agg1_bwd": 247.3e6, "agg0_bwd": 151.8e6,
-                               "sender_reduce": 48.3e6},
-    ("mp_medium", "float32"): {"agg0_fwd": 1733.4e6, "agg1_fwd": 4609.0e6, "agg1_bwd": 16226.3e6, "agg0_bwd": 4490.6e6,
-                               "sender_reduce": 8257.2e6},
-    ("mp_medium", "float64"): {"agg0_fwd": 2291.3e6, "agg1_fwd": 20204.2e6, "agg1_bwd": 45819.8e6, "agg0_bwd": 7626.9e6,
-                               "sender_reduce": 16442.6e6},
-}
+
+def stage_kernel(stage, L_max, distinct_tables):
+    """Name of the kernel that runs an edge stage for this kind of model."""
+    sliced = distinct_tables <= 4
+    if stage.startswith("agg0"):
+        return (SLICE_KERNEL if sliced else GENERAL_KERNEL)[stage]
+    if stage == "sender_reduce":
+        return SLICE_KERNEL[stage] if L_max == 0 else GENERAL_KERNEL[stage]
+    return (SLICE_KERNEL if (sliced and L_max == 0) else GENERAL_KERNEL)[stage]
+
+
+def measured_traffic(workload, dtype, stage, kernel):
+    """HBM bytes per launch of `kernel` in `stage`, from the rocprofv3 counter summary kept under profiles/
+    (FETCH_SIZE and WRITE_SIZE runs scaled by a copy of known size; the file says how it was made).  None when
+    the file holds no line for this kernel, stage and precision, e.g. after a kernel was renamed."""
+    path = os.path.join(HERE, "profiles", f"edge_kernels_{workload}_hbm_traffic.txt")
+    if not os.path.exists(path):
+        return None
+    tag = "<double" if dtype == "float64" else "<float"
+    for line in open(path):
+        cols = line.split()
+        if len(cols) >= 6 and line.startswith(kernel + tag) and stage in cols:
+            k = cols.index(stage)
+            try:
+                return float(cols[k + 3]) * 1e6      # columns after the stage: fetch MB, write MB, traffic MB
+            except (ValueError, IndexError):
+                return None
+    return None
 
 
 def algorithmic_bytes(stage, N, E, K, s, n_LM, n_e):
@@ -217,6 +236,12 @@ def main():
     ap.add_argument("--ghosts", action="store_true",
                     help="periodic images as explicit ghost nodes that go through layer 0 only (the pair style's "
                          "no_mpi_message_passing layout on one rank) instead of senders mapped to their owners")
+    ap.add_argument("--pair-tables", action="store_true",
+                    help="a radial table of its own for every species pair (more than four distinct tables take the "
+                         "general edge kernels)")
+    ap.add_argument("--no-second", action="store_true",
+                    help="default workload only: skip the second configuration of the metric (mp_medium, float32 features) "
+                         "and the pair-dependent-table variant that ride along")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-atoms", type=int, default=0, help="atoms in the CPU sample (0 = whole workload)")
     ap.add_argument("--model-dir", default=tempfile.gettempdir())
@@ -240,95 +265,133 @@ def main():
     if args.workload == "water_capacity":
         return run_capacity(args)
 
-    # ---- model file (seeded, random-init) and synthetic system
-    cfg = dict(modelgen.CONFIGS[args.workload])
-    # plain MACE has a species-independent radial network: every pair table of the file is equal
-    cfg["pair_dependent_radial"] = False
-    model_path = os.path.join(args.model_dir, f"smx_bench_{args.workload}.json")
-    if not os.path.exists(model_path):
-        modelgen.write_model(model_path, **cfg)
-    pos, cell, species = systems.config_system(args.workload, seed=0, scale=args.scale)
-    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"])
-    ea = neighbors.edge_arrays(nl, species)
-    N, E = int(ea["num_nodes"]), int(len(ea["r"]))
-    N_ghost, E_local = 0, E
-    if args.ghosts:
-        ea = neighbors.ghost_edge_arrays(nl, species)
-        N, N_ghost = int(ea["num_local_nodes"]), int(ea["num_ghost_nodes"])
-        E_local, E = int(ea["num_neigh"][:N].sum()), int(len(ea["r"]))
-        args.no_cpu = True     # the CPU leg times the plain layout
+    def measure(workload, dtype, steps, warmup, pair_tables=False, ghosts=False, scale=1.0, both=True, host_leg=True):
+        """One workload in one precision (and, with `both`, in the other): model file, synthetic system, timing."""
+        cfg = dict(modelgen.CONFIGS[workload])
+        # plain MACE has a species-independent radial network: every pair table of the file is equal;
+        # pair_tables gives every species pair its own table (as a distance transform does)
+        cfg["pair_dependent_radial"] = bool(pair_tables)
+        model_path = os.path.join(args.model_dir, f"smx_bench_{workload}{'_pairs' if pair_tables else ''}.json")
+        if not os.path.exists(model_path):
+            modelgen.write_model(model_path, **cfg)
+        pos, cell, species = systems.config_system(workload, seed=0, scale=scale)
+        nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"])
+        ea = neighbors.edge_arrays(nl, species)
+        N, E = int(ea["num_nodes"]), int(len(ea["r"]))
+        N_ghost, E_local = 0, E
+        if ghosts:
+            ea = neighbors.ghost_edge_arrays(nl, species)
+            N, N_ghost = int(ea["num_local_nodes"]), int(ea["num_ghost_nodes"])
+            E_local, E = int(ea["num_neigh"][:N].sum()), int(len(ea["r"]))
 
-    def to_dev(a, dt):
-        return torch.from_numpy(np.ascontiguousarray(a)).to(dev, dtype=dt)
+        def to_dev(a, dt):
+            return torch.from_numpy(np.ascontiguousarray(a)).to(dev, dtype=dt)
 
-    d = dict(
-        node_types=to_dev(ea["node_types"], torch.int32), num_neigh=to_dev(ea["num_neigh"], torch.int32),
-        neigh_indices=to_dev(ea["neigh_indices"], torch.int32), neigh_types=to_dev(ea["neigh_types"], torch.int32),
-        xyz=to_dev(ea["xyz"], torch.float64), r=to_dev(ea["r"], torch.float64),
-    )
-    out_E = torch.zeros(N, dtype=torch.float64, device=dev)
-    out_F = torch.zeros(3 * E, dtype=torch.float64, device=dev)
+        d = dict(
+            node_types=to_dev(ea["node_types"], torch.int32), num_neigh=to_dev(ea["num_neigh"], torch.int32),
+            neigh_indices=to_dev(ea["neigh_indices"], torch.int32), neigh_types=to_dev(ea["neigh_types"], torch.int32),
+            xyz=to_dev(ea["xyz"], torch.float64), r=to_dev(ea["r"], torch.float64),
+        )
+        out_E = torch.zeros(N, dtype=torch.float64, device=dev)
+        out_F = torch.zeros(3 * E, dtype=torch.float64, device=dev)
 
-    def run_mode(dtype, steps, warmup):
-        eng = MACE(model_path, dtype)
-        stream = torch.cuda.current_stream().cuda_stream
+        def run_mode(dtype, steps, warmup):
+            eng = MACE(model_path, dtype)
+            stream = torch.cuda.current_stream().cuda_stream
 
-        def step_ghosted():
-            eng.compute_ghosted_device(N, N_ghost, d["node_types"].data_ptr(), d["num_neigh"].data_ptr(),
-                                       d["neigh_indices"].data_ptr(), d["neigh_types"].data_ptr(), d["xyz"].data_ptr(),
-                                       d["r"].data_ptr(), E, E_local, out_E.data_ptr(), out_F.data_ptr(), stream)
+            def step():
+                if ghosts:
+                    eng.compute_ghosted_device(N, N_ghost, d["node_types"].data_ptr(), d["num_neigh"].data_ptr(),
+                                               d["neigh_indices"].data_ptr(), d["neigh_types"].data_ptr(), d["xyz"].data_ptr(),
+                                               d["r"].data_ptr(), E, E_local, out_E.data_ptr(), out_F.data_ptr(), stream)
+                else:
+                    eng.compute_device(N, d["node_types"].data_ptr(), d["num_neigh"].data_ptr(), d["neigh_indices"].data_ptr(),
+                                       d["neigh_types"].data_ptr(), d["xyz"].data_ptr(), d["r"].data_ptr(), E,
+                                       out_E.data_ptr(), out_F.data_ptr(), stream)
 
-        def step():
-            if args.ghosts:
-                return step_ghosted()
-            eng.compute_device(N, d["node_types"].data_ptr(), d["num_neigh"].data_ptr(), d["neigh_indices"].data_ptr(),
-                               d["neigh_types"].data_ptr(), d["xyz"].data_ptr(), d["r"].data_ptr(), E,
-                               out_E.data_ptr(), out_F.data_ptr(), stream)
+            for _ in range(warmup):
+                step()
+            torch.cuda.synchronize()
+            # timed region: exactly `steps` evaluations as asynchronous enqueues between two synchronisations
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+            torch.cuda.synchronize()
+            dt_async = time.perf_counter() - t0
+            # the same number of steps with per-stage HIP events on the stream the kernels run on (the events are per
+            # model and reused every step, so they are read back after every step)
+            eng.set_profiling(True)
+            acc = {}
+            t0 = time.perf_counter()
+            for _ in range(steps):
+                step()
+                for k, v in eng.stage_times().items():
+                    acc[k] = acc.get(k, 0.0) + v
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            eng.set_profiling(False)
+            res = dict(ms_sync=1e3 * dt / steps, ms=1e3 * dt_async / steps, stages={k: v / steps for k, v in acc.items()},
+                       tables=eng._int("num_radial_tables_0"))
+            if host_leg:
+                # the same evaluation through the host-array entry point (upload, range checks, download included)
+                hsteps = max(3, min(10, steps // 4))
 
-        for _ in range(warmup):
-            step()
-        torch.cuda.synchronize()
-        # timed region: exactly `steps` evaluations; per-stage HIP events ride along on the same stream
-        eng.set_profiling(True)
-        acc = {}
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            step()
-            # stage events are per model and reused every step: read them back before the next step
-            for k, v in eng.stage_times().items():
-                acc[k] = acc.get(k, 0.0) + v
-        torch.cuda.synchronize()
-        dt = time.perf_counter() - t0
-        eng.set_profiling(False)
-        # the same number of steps without event read-back (pure asynchronous enqueue)
-        torch.cuda.synchronize()
-        t0 = time.perf_counter()
-        for _ in range(steps):
-            step()
-        torch.cuda.synchronize()
-        dt_async = time.perf_counter() - t0
-        # the same evaluation through the host-array entry point (upload, range checks, download included)
-        hsteps = max(3, min(10, steps // 4))
+                def host_step():
+                    if ghosts:
+                        eng.compute_ghosted(N, N_ghost, ea["node_types"], ea["num_neigh"], ea["neigh_indices"],
+                                            ea["neigh_types"], ea["xyz"], ea["r"])
+                    else:
+                        eng.compute_node_energies_forces(N, ea["node_types"], ea["num_neigh"], ea["neigh_indices"],
+                                                         ea["neigh_types"], ea["xyz"], ea["r"])
+                host_step()
+                t0 = time.perf_counter()
+                for _ in range(hsteps):
+                    host_step()
+                    _ = eng.node_energies, eng.node_forces
+                res["ms_host"] = 1e3 * (time.perf_counter() - t0) / hsteps
+                step()
+                torch.cuda.synchronize()
+            res["energy"] = float(out_E.sum().item())
+            res["forces"] = out_F.cpu().numpy().copy()
+            del eng
+            return res
 
-        def host_step():
-            if args.ghosts:
-                eng.compute_ghosted(N, N_ghost, ea["node_types"], ea["num_neigh"], ea["neigh_indices"], ea["neigh_types"],
-                                    ea["xyz"], ea["r"])
-            else:
-                eng.compute_node_energies_forces(N, ea["node_types"], ea["num_neigh"], ea["neigh_indices"],
-                                                 ea["neigh_types"], ea["xyz"], ea["r"])
-        host_step()
-        t0 = time.perf_counter()
-        for _ in range(hsteps):
-            host_step()
-            _ = eng.node_energies, eng.node_forces
-        dt_host = (time.perf_counter() - t0) / hsteps
-        stages = {k: v / steps for k, v in acc.items()}
-        energy = float(out_E.sum().item())
-        fmax = float(out_F.abs().max().item()) if E else 0.0
-        del eng
-        return dict(ms_sync=1e3 * dt / steps, ms=1e3 * dt_async / steps, ms_host=1e3 * dt_host, stages=stages, energy=energy, fmax=fmax,
-                    forces=out_F.cpu().numpy().copy())
+        res = run_mode(dtype, steps, warmup)
+        K, L_max = cfg["num_channels"], cfg["L_max"]
+        n_LM = (L_max + 1) ** 2
+        n_e = 16 if L_max == 0 else 40
+        s_bytes = 8 if dtype == "float64" else 4
+
+        def stage_bytes(k):   # layer-0 stages run over all nodes and edges, layer-1 stages over the local ones
+            if k.startswith("agg0"):
+                return algorithmic_bytes(k, N + N_ghost, E, K, s_bytes, n_LM, n_e)
+            return algorithmic_bytes(k, N, E_local, K, s_bytes, n_LM, n_e)
+
+        dom = max(EDGE_STAGES, key=lambda k: res["stages"].get(k, 0.0))
+        dom_bytes = stage_bytes(dom)
+        dom_s = res["stages"][dom] * 1e-3
+        achieved = dom_bytes / dom_s / 1e9 if dom_s > 0 else 0.0
+        total_bytes = sum(stage_bytes(k) for k in EDGE_STAGES) + (32 * E + 24 * N)
+        kernel = stage_kernel(dom, L_max, res["tables"])
+        out = dict(
+            cfg=cfg, model_path=model_path, ea=ea, N=N, E=E, N_ghost=N_ghost, E_local=E_local, res=res,
+            value=N / (res["ms"] * 1e-3),
+            workload=f"{workload}: {N} atoms, {E} edges, K={K}, L_max={L_max}, r_cut={cfg['r_cut']}, random-init symmetrix "
+                     f"JSON model (seed 0), " + ("one radial table per species pair" if pair_tables else
+                                                 "species-independent radial tables"),
+            roofline={
+                "bound": "hbm", "kernel": kernel, "stage": dom, "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
+                "frac": achieved / (HBM_PEAK / 1e9),
+                "traffic": measured_traffic(workload, dtype, dom, kernel) if scale == 1.0 and not ghosts and not pair_tables else None,
+                "algorithmic_bytes_per_launch": dom_bytes, "kernel_ms": res["stages"][dom],
+                "whole_step_algorithmic_bytes": total_bytes,
+                "whole_step_frac": (total_bytes / HBM_PEAK) / (res["ms"] * 1e-3),
+            },
+        )
+        if both:
+            other = "float32" if dtype == "float64" else "float64"
+            out["other"] = (other, run_mode(other, max(5, steps // 2), warmup))
+        return out
 
     if args.calibrate_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device=dev)   # 1 GiB read + 1 GiB written
@@ -337,31 +400,15 @@ def main():
         torch.cuda.synchronize()
         del src, dst
 
-    res = run_mode(args.dtype, args.steps, args.warmup)
-    other = "float32" if args.dtype == "float64" else "float64"
-    res_other = run_mode(other, max(5, args.steps // 2), args.warmup)
-
-    K = cfg["num_channels"]
-    L_max = cfg["L_max"]
-    n_LM = (L_max + 1) ** 2
-    n_e = 16 if L_max == 0 else 40
-    s_bytes = 8 if args.dtype == "float64" else 4
-    edge_stages = ["agg0_fwd", "agg1_fwd", "agg1_bwd", "sender_reduce", "agg0_bwd"]
-    dom = max(edge_stages, key=lambda k: res["stages"].get(k, 0.0))
-    def stage_bytes(k):   # layer-0 stages run over all nodes and edges, layer-1 stages over the local ones
-        if k.startswith("agg0"):
-            return algorithmic_bytes(k, N + N_ghost, E, K, s_bytes, n_LM, n_e)
-        return algorithmic_bytes(k, N, E_local, K, s_bytes, n_LM, n_e)
-
-    dom_bytes = stage_bytes(dom)
-    dom_s = res["stages"][dom] * 1e-3
-    achieved = dom_bytes / dom_s / 1e9 if dom_s > 0 else 0.0
-    total_bytes = sum(stage_bytes(k) for k in edge_stages) + (32 * E + 24 * N)
-
-    value = N / (res["ms"] * 1e-3)
+    if args.ghosts:
+        args.no_cpu = True     # the CPU leg times the plain layout
+    m = measure(args.workload, args.dtype, args.steps, args.warmup, pair_tables=args.pair_tables, ghosts=args.ghosts,
+                scale=args.scale)
+    res, cfg, N, E = m["res"], m["cfg"], m["N"], m["E"]
+    other, res_other = m["other"]
     line = {
         "metric": "atom-steps/s per MI355X (energy+forces)",
-        "value": value,
+        "value": m["value"],
         "unit": "atom-steps/s",
         "n_gpus": 1,
         "steps": args.steps,
@@ -373,20 +420,10 @@ def main():
         "dtype": "f64" if args.dtype == "float64" else "f32-features/f64-accumulation",
         "data": "synthetic",
         "config": {
-            "workload": f"{args.workload}: {N} atoms, {E} edges, K={K}, L_max={L_max}, r_cut={cfg['r_cut']}, "
-                        f"random-init symmetrix JSON model (seed 0), species-independent radial tables",
-            "atoms": N, "edges": E, "channels": K, "L_max": L_max, "scale": args.scale,
-            "ghost_nodes": N_ghost, "edges_of_local_receivers": E_local,
+            "workload": m["workload"], "atoms": N, "edges": E, "channels": cfg["num_channels"], "L_max": cfg["L_max"],
+            "scale": args.scale, "ghost_nodes": m["N_ghost"], "edges_of_local_receivers": m["E_local"],
         },
-        "roofline": {
-            "bound": "hbm", "kernel": STAGE_KERNEL[dom][0 if L_max == 0 else 1], "stage": dom,
-            "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
-            "frac": achieved / (HBM_PEAK / 1e9),
-            "traffic": MEASURED_TRAFFIC.get((args.workload, args.dtype), {}).get(dom) if args.scale == 1.0 and not args.ghosts else None,
-            "algorithmic_bytes_per_launch": dom_bytes,
-            "whole_step_algorithmic_bytes": total_bytes,
-            "whole_step_frac": (total_bytes / HBM_PEAK) / (res["ms"] * 1e-3),
-        },
+        "roofline": m["roofline"],
         "stages_ms": res["stages"],
         "ms_per_step_with_event_readback": res["ms_sync"],
         "host_arrays": {"ms_per_step": res["ms_host"], "value": N / (res["ms_host"] * 1e-3),
@@ -395,15 +432,34 @@ def main():
         "other_precision": {"dtype": other, "ms_per_step": res_other["ms"], "value": N / (res_other["ms"] * 1e-3),
                             "energy": res_other["energy"], "stages_ms": res_other["stages"]},
     }
+    default_run = args.workload == "off_small" and args.scale == 1.0 and not args.ghosts and not args.pair_tables
+    if default_run and not args.no_second:
+        # the metric is quoted on two configurations: the second one (50 000-atom alloy, K = 128, hidden features up
+        # to l = 1, float32 features) rides along with its own figures; fewer steps, no CPU leg
+        s2 = max(5, args.steps // 5)
+        m2 = measure("mp_medium", "float32", s2, 2, both=False, host_leg=False)
+        line["second_config"] = {
+            "workload": m2["workload"], "dtype": "f32-features/f64-accumulation", "steps": s2, "warmup": 2,
+            "ms_per_step": m2["res"]["ms"], "value": m2["value"], "unit": "atom-steps/s", "roofline": m2["roofline"],
+            "stages_ms": m2["res"]["stages"], "energy": m2["res"]["energy"],
+        }
+        # the headline workload with one radial table per species pair (ten tables for four species): more than four
+        # distinct tables take the general edge kernels instead of the channel-slice ones
+        m3 = measure("off_small", args.dtype, max(5, args.steps // 2), args.warmup, pair_tables=True, both=False, host_leg=False)
+        line["pair_dependent_tables"] = {
+            "workload": m3["workload"], "dtype": line["dtype"], "ms_per_step": m3["res"]["ms"], "value": m3["value"],
+            "unit": "atom-steps/s", "roofline": m3["roofline"], "stages_ms": m3["res"]["stages"],
+        }
 
     # ---- CPU baseline: the oracle (serial fp64 port of the reference path) on this host
     if not args.no_cpu:
         from oracle.oracle import OracleMACE
-        orc = OracleMACE(model_path)
+        ea = m["ea"]
+        orc = OracleMACE(m["model_path"])
         if args.cpu_atoms and args.cpu_atoms < N:
-            p2, c2, s2 = systems.config_system(args.workload, seed=0, scale=args.scale * args.cpu_atoms / N)
+            p2, c2, s2_ = systems.config_system(args.workload, seed=0, scale=args.scale * args.cpu_atoms / N)
             nl2 = neighbors.neighbor_list(p2, c2, cfg["r_cut"])
-            ea2 = neighbors.edge_arrays(nl2, s2)
+            ea2 = neighbors.edge_arrays(nl2, s2_)
             sample = f"{ea2['num_nodes']} atoms / {len(ea2['r'])} edges sub-box of the workload (same density, same model), 1 evaluation"
         else:
             ea2 = ea
@@ -420,7 +476,7 @@ def main():
         cpu_value = ea2["num_nodes"] / dt
         line["cpu_baseline"] = {"value": cpu_value, "unit": "atom-steps/s", "cores": 1, "kind": "port",
                                 "sample": sample, "seconds": dt, "host_cores": os.cpu_count(),
-                                "gpu_over_cpu_1core": value / cpu_value}
+                                "gpu_over_cpu_1core": m["value"] / cpu_value}
         if ea2 is ea:
             Ecpu = float(orc.node_energies.sum())
             line["cpu_baseline"]["energy_rel_diff_vs_gpu"] = abs(Ecpu - res["energy"]) / abs(Ecpu)

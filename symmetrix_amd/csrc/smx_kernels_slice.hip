@@ -350,7 +350,10 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     const int row = lane / RL, sub = lane % RL;
     const int kc = slice * CH;
     const bool whole = kc + CH <= K;                        // all channels of the slice exist
-    F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + (size_t)(wave * ROWS + row) * 16 * CH;
+    // staged adjoint rows of this lane's receiver; the rows of a wavefront lie 32 bytes more than their length
+    // apart, so that their broadcast reads (same offset in every row) fall on different banks
+    constexpr int DSTRIDE = 16 * CH + 32 / (int)sizeof(F);
+    F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + (size_t)(wave * ROWS + row) * DSTRIDE;
     const int wave_tasks = (a.num_nodes + ROWS - 1) / ROWS;
     __shared__ int task_counter;
     double* fpart = p.fpart + (size_t)slice * p.E * 3;
@@ -551,7 +554,7 @@ static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t
 {
     constexpr int CH = 32 / (int)sizeof(F), ROWS = 64 / RL;
     const int S = (p.a.K + CH - 1) / CH;
-    const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F) + (size_t)(BT / 64) * ROWS * 16 * CH * sizeof(F);
+    const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F) + (size_t)(BT / 64) * ROWS * (16 * CH * sizeof(F) + 32);
     int RG = p.num_cus / S;
     if (RG < 1) RG = 1;
     const long tasks_per_slice = ((long)p.a.num_nodes + ROWS - 1) / ROWS;
@@ -582,7 +585,7 @@ template int slice_edge_row_elements<double>();
 template int slice_edge_row_elements<float>();
 template <typename F> size_t slice_edge_lds_bytes(int spl_nodes)
 {
-    return (size_t)(spl_nodes - 1) * slice_edge_row_elements<F>() * sizeof(F) + (size_t)12 * 4 * 16 * 32;
+    return (size_t)(spl_nodes - 1) * slice_edge_row_elements<F>() * sizeof(F) + (size_t)12 * 4 * (16 * 32 + 32);
 }
 template size_t slice_edge_lds_bytes<double>(int);
 template size_t slice_edge_lds_bytes<float>(int);

@@ -442,6 +442,10 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
 #pragma unroll
                     for (int c = 0; c < CH; ++c) ul[c] = F(0);
                     F py = F(0);
+                    // sender row times radial value / derivative once per order, not once per harmonic
+                    F hv[CH], hd[CH];
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) { hv[c] = h.v[c] * Rv[l][c]; hd[c] = h.v[c] * Rd[l][c]; }
                     static_for<0, 2 * l + 1>([&](auto mc) {
                         constexpr int lm = l * l + decltype(mc)::value;
                         double y, g0, g1, g2;
@@ -451,9 +455,8 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
                         F P = F(0), Q = F(0);
 #pragma unroll
                         for (int c = 0; c < CH; ++c) {
-                            const F dh = dd.v[c] * h.v[c];
-                            P += dh * Rv[l][c];
-                            Q += dh * Rd[l][c];
+                            P += dd.v[c] * hv[c];
+                            Q += dd.v[c] * hd[c];
                             ul[c] += dd.v[c] * yf;
                         }
                         srad += Q * yf;

@@ -403,11 +403,17 @@ struct Engine : EngineBase {
             // adjoint kernel with one lane per edge: CH channels are 32 bytes, table slice and the staged adjoint
             // rows of twelve wavefronts fit the LDS
             edge_lanes = CH * sizeof(F) == 32 && slice_edge_lds_bytes<F>(hm.spl_nodes) <= lds_cap;
-            if (edge_lanes && slice_edge_row_elements<F>() != W) {
+            if (edge_lanes) {
                 const int We = slice_edge_row_elements<F>();
                 std::vector<F> eb((size_t)S * U * R * We, F(0));
-                for (size_t rowi = 0; rowi < (size_t)S * U * R; ++rowi)
-                    std::copy(buf.begin() + rowi * W, buf.begin() + rowi * W + 16 * CH, eb.begin() + rowi * We);
+                // unpadded rows; the 32-byte piece (coefficient, path) of row n is stored at piece index
+                // (4 coefficient + path) ^ (n & 7), which spreads the reads of different rows over the banks
+                for (size_t rowi = 0; rowi < (size_t)S * U * R; ++rowi) {
+                    const int swz = (int)(rowi % R) & 7;
+                    for (int pc = 0; pc < 16; ++pc)
+                        std::copy(buf.begin() + rowi * W + pc * CH, buf.begin() + rowi * W + (pc + 1) * CH,
+                                  eb.begin() + rowi * We + (size_t)(pc ^ swz) * CH);
+                }
                 edst.upload(eb.data(), eb.size(), s);
                 HIPCHK(hipStreamSynchronize(s));
             }
@@ -837,7 +843,13 @@ struct Engine : EngineBase {
             HIPCHK(launch_slice_bwd<F>(sp, stream));
             stage_end(ST_AGG1B);
             stage_begin(ST_FSUM1);
-            HIPCHK(launch_fpart_reduce(E1, E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
+            if (carry_forces && sp.edge_lanes && slice_CH0 == slice_CH1) {
+                // the layer-0 adjoint of the same call adds its share to these partial forces and sums once
+                carried_edges = E1;
+                carried_accumulate = zero_dxyz ? 0 : 1;
+            } else {
+                HIPCHK(launch_fpart_reduce(E1, E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
+            }
             stage_end(ST_FSUM1);
         } else {
             auto p = agg_params(1, N);
@@ -857,6 +869,9 @@ struct Engine : EngineBase {
         }
         stage_end(ST_SRED);
     }
+    bool carry_forces = false;      // compute() lets the layer-1 partial forces wait for the layer-0 adjoint
+    long carried_edges = 0;         // ... and the stage left them in fpart for edges [0, carried_edges)
+    int carried_accumulate = 1;
     bool fuse_reverse_H1 = false;   // compute() wants reverse_H1 folded into the sender-side sum
     bool reverse_H1_done = false;   // ... and the stage did it
     // The same stage for edge lists whose messages do not fit the staging buffer: receivers are taken in
@@ -917,11 +932,19 @@ struct Engine : EngineBase {
             const int S = (K() + sp.CH - 1) / sp.CH;
             fpart.size_to((size_t)S * 3 * E, stream);
             sp.a.d_out = Phi0.p; sp.a.msg = nullptr; sp.fpart = fpart.p;
+            int accumulate = 1;
+            if (carried_edges > 0) {
+                // With carried layer-1 partial forces, edges past them (ghost receivers) have only this stage's share:
+                // the sum below overwrites, so the forces must not hold anything else for them.
+                sp.fpart_carry = carried_edges;
+                accumulate = carried_accumulate;
+                carried_edges = 0;
+            }
             stage_begin(ST_AGG0B);
             HIPCHK(launch_slice_bwd<F>(sp, stream));
             stage_end(ST_AGG0B);
             stage_begin(ST_FSUM0);
-            HIPCHK(launch_fpart_reduce(E, E, S, fpart.p, node_forces.p, 1, forces_copy, stream));
+            HIPCHK(launch_fpart_reduce(E, E, S, fpart.p, node_forces.p, accumulate, forces_copy, stream));
             forces_copy = nullptr;
             stage_end(ST_FSUM0);
             return;
@@ -1076,8 +1099,10 @@ struct Engine : EngineBase {
         st_scale(1, N1, true);
         stage_begin(ST_REVA1); st_A1(N1, true, fuse1); stage_end(ST_REVA1);
         fuse_reverse_H1 = N1 == N; reverse_H1_done = false;
+        // (the density normalisation of layer 0 adds to the forces in between: then they must already hold the layer-1 sum)
+        carry_forces = early_forces || !hm.A0_scaled; carried_edges = 0;
         st_agg1_bwd(N1, !early_forces, false);
-        fuse_reverse_H1 = false;
+        fuse_reverse_H1 = false; carry_forces = false;
         if (N1 < N) node_lists_for(N);
         stage_begin(ST_REVH1); if (!reverse_H1_done) st_H1(N, true); stage_end(ST_REVH1);
         stage_begin(ST_REVM0); if (!fuse0) st_reverse_M0(N); stage_end(ST_REVM0);

@@ -350,10 +350,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     const int row = lane / RL, sub = lane % RL;
     const int kc = slice * CH;
     const bool whole = kc + CH <= K;                        // all channels of the slice exist
-    // staged adjoint rows of this lane's receiver; the rows of a wavefront lie 32 bytes more than their length
-    // apart, so that their broadcast reads (same offset in every row) fall on different banks
-    constexpr int DSTRIDE = 16 * CH + 32 / (int)sizeof(F);
-    F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + (size_t)(wave * ROWS + row) * DSTRIDE;
+    // staged adjoint rows of the wavefront's receivers, [harmonic][receiver][CH]: the receivers' reads of one
+    // harmonic (same instruction, one 32-byte piece each) cover contiguous memory
+    F* dstage = reinterpret_cast<F*>(smem + (size_t)R * 512) + ((size_t)wave * 16 * ROWS + row) * CH;
     const int wave_tasks = (a.num_nodes + ROWS - 1) / ROWS;
     __shared__ int task_counter;
     double* fpart = p.fpart + (size_t)slice * p.E * 3;
@@ -361,7 +360,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     for (int u = 0; u < p.U; ++u) {
         __syncthreads();
         if (threadIdx.x == 0) task_counter = 0;
-        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
+        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * 512);
         __syncthreads();
         for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
              task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
@@ -388,7 +387,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
                 const F cd = (F)p.cdiag[lm];
 #pragma unroll
                 for (int c = 0; c < CH; ++c) v.v[c] *= cd;
-                *reinterpret_cast<V*>(dstage + lm * CH) = v;
+                *reinterpret_cast<V*>(dstage + lm * ROWS * CH) = v;
             }
             wave_lds_sync();
             const int iters = (e1 - e0 + RL - 1) / RL;
@@ -411,25 +410,17 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
                         for (int c = 0; c < CH; ++c) h.v[c] = src[min(c, K - 1 - kc)];
                     }
                 }
+                // partial forces an earlier stage left for this edge: requested now, added at the end
+                double f0 = 0.0, f1 = 0.0, f2 = 0.0;
+                if (e < p.fpart_carry) { f0 = fpart[3 * (size_t)e]; f1 = fpart[3 * (size_t)e + 1]; f2 = fpart[3 * (size_t)e + 2]; }
                 const double dx = cu.dx, dy = cu.dy, dz = cu.dz, r = cu.r;
                 const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
                 const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
                 const int n = spline_interval(r, a.spl_inv_h, R - 1);
                 const F x = (F)(r - a.spl_h * n);
-                const F* rowp = lds + (size_t)n * W;
-                F Rv[4][CH], Rd[4][CH];
-#pragma unroll
-                for (int l = 0; l < 4; ++l) {
-                    const V c0 = *reinterpret_cast<const V*>(rowp + (0 * 4 + l) * CH);
-                    const V c1 = *reinterpret_cast<const V*>(rowp + (1 * 4 + l) * CH);
-                    const V c2 = *reinterpret_cast<const V*>(rowp + (2 * 4 + l) * CH);
-                    const V c3 = *reinterpret_cast<const V*>(rowp + (3 * 4 + l) * CH);
-#pragma unroll
-                    for (int c = 0; c < CH; ++c) {
-                        Rv[l][c] = c0.v[c] + x * (c1.v[c] + x * (c2.v[c] + x * c3.v[c]));
-                        Rd[l][c] = c1.v[c] + x * (F(2) * c2.v[c] + F(3) * x * c3.v[c]);
-                    }
-                }
+                // 32-byte piece (coefficient, path) of row n sits at piece index (16 n + 4 coefficient + path) ^ (n & 7)
+                const unsigned rowb = (((unsigned)n << 4) ^ ((unsigned)n & 7u)) * 32u;
+                auto piece = [&](int q, int l) { return *reinterpret_cast<const V*>(smem + (rowb ^ (unsigned)((q * 4 + l) * 32))); };
                 F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
                 F mg[CH];
 #pragma unroll
@@ -443,14 +434,21 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
                     for (int c = 0; c < CH; ++c) ul[c] = F(0);
                     F py = F(0);
                     // sender row times radial value / derivative once per order, not once per harmonic
-                    F hv[CH], hd[CH];
+                    F Rv[CH], hv[CH], hd[CH];
+                    {
+                        const V c0 = piece(0, l), c1 = piece(1, l), c2 = piece(2, l), c3 = piece(3, l);
 #pragma unroll
-                    for (int c = 0; c < CH; ++c) { hv[c] = h.v[c] * Rv[l][c]; hd[c] = h.v[c] * Rd[l][c]; }
+                        for (int c = 0; c < CH; ++c) {
+                            Rv[c] = c0.v[c] + x * (c1.v[c] + x * (c2.v[c] + x * c3.v[c]));
+                            hv[c] = h.v[c] * Rv[c];
+                            hd[c] = h.v[c] * (c1.v[c] + x * (F(2) * c2.v[c] + F(3) * x * c3.v[c]));
+                        }
+                    }
                     static_for<0, 2 * l + 1>([&](auto mc) {
                         constexpr int lm = l * l + decltype(mc)::value;
                         double y, g0, g1, g2;
                         ylm_g<lm>(vx, vy, vz, y, g0, g1, g2);
-                        const V dd = *reinterpret_cast<const V*>(dstage + lm * CH);
+                        const V dd = *reinterpret_cast<const V*>(dstage + lm * ROWS * CH);
                         const F yf = (F)y;
                         F P = F(0), Q = F(0);
 #pragma unroll
@@ -465,7 +463,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
                     });
                     lterm += py * F(l);
 #pragma unroll
-                    for (int c = 0; c < CH; ++c) mg[c] += Rv[l][c] * ul[c];
+                    for (int c = 0; c < CH; ++c) mg[c] += Rv[c] * ul[c];
                     order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
 #pragma unroll
                     for (int c = 0; c < CH; ++c) pin_value(mg[c]);
@@ -486,9 +484,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
                 // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
                 const double sr = (double)srad, lt = (double)lterm;
                 const double ir = rcp_pos(r);
-                fpart[3 * (size_t)e] = -(dx * ir * sr + ((double)wy - uy * lt) * inv);       // original x is permuted axis 1
-                fpart[3 * (size_t)e + 1] = -(dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
-                fpart[3 * (size_t)e + 2] = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
+                fpart[3 * (size_t)e] = f0 - (dx * ir * sr + ((double)wy - uy * lt) * inv);       // original x is permuted axis 1
+                fpart[3 * (size_t)e + 1] = f1 - (dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
+                fpart[3 * (size_t)e + 2] = f2 - (dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
             }
         }
     }
@@ -552,12 +550,15 @@ hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s)
     default: return hipErrorInvalidValue;
     }
 }
+// threads per block of the lane-per-edge adjoint kernel: three wavefronts per SIMD, 168 registers each (four per
+// SIMD, which the LDS has room for, spill in double precision and gain nothing measurable in single)
+template <typename F> constexpr int kEdgeBlock = 768;
 template <typename F, int BT, int RL>
 static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t s)
 {
     constexpr int CH = 32 / (int)sizeof(F), ROWS = 64 / RL;
     const int S = (p.a.K + CH - 1) / CH;
-    const size_t lds = (size_t)(p.a.spl_nodes - 1) * p.W * sizeof(F) + (size_t)(BT / 64) * ROWS * (16 * CH * sizeof(F) + 32);
+    const size_t lds = (size_t)(p.a.spl_nodes - 1) * 512 + (size_t)(BT / 64) * ROWS * 512;
     int RG = p.num_cus / S;
     if (RG < 1) RG = 1;
     const long tasks_per_slice = ((long)p.a.num_nodes + ROWS - 1) / ROWS;
@@ -577,18 +578,18 @@ static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t
 template <typename F>
 static hipError_t launch_slice_bwd_edge(const SliceParams<F>& p, hipStream_t s)
 {
-    return launch_slice_bwd_edge_cfg<F, 768, 16>(p, s);
+    return launch_slice_bwd_edge_cfg<F, kEdgeBlock<F>, 16>(p, s);
 }
 template <typename F> int slice_edge_row_elements()
 {
-    // [4][4][CH] with CH * sizeof(F) = 32: 512 bytes, plus 16 so that consecutive rows start four banks apart
-    return (512 + 16) / (int)sizeof(F);
+    // [4][4][CH] with CH * sizeof(F) = 32: 512 bytes, no padding (the pieces of a row are permuted instead)
+    return 512 / (int)sizeof(F);
 }
 template int slice_edge_row_elements<double>();
 template int slice_edge_row_elements<float>();
 template <typename F> size_t slice_edge_lds_bytes(int spl_nodes)
 {
-    return (size_t)(spl_nodes - 1) * slice_edge_row_elements<F>() * sizeof(F) + (size_t)12 * 4 * (16 * 32 + 32);
+    return (size_t)(spl_nodes - 1) * 512 + (size_t)(kEdgeBlock<F> / 64) * 4 * 512;
 }
 template size_t slice_edge_lds_bytes<double>(int);
 template size_t slice_edge_lds_bytes<float>(int);

@@ -406,14 +406,8 @@ struct Engine : EngineBase {
             if (edge_lanes) {
                 const int We = slice_edge_row_elements<F>();
                 std::vector<F> eb((size_t)S * U * R * We, F(0));
-                // unpadded rows; the 32-byte piece (coefficient, path) of row n is stored at piece index
-                // (4 coefficient + path) ^ (n & 7), which spreads the reads of different rows over the banks
-                for (size_t rowi = 0; rowi < (size_t)S * U * R; ++rowi) {
-                    const int swz = (int)(rowi % R) & 7;
-                    for (int pc = 0; pc < 16; ++pc)
-                        std::copy(buf.begin() + rowi * W + pc * CH, buf.begin() + rowi * W + (pc + 1) * CH,
-                                  eb.begin() + rowi * We + (size_t)(pc ^ swz) * CH);
-                }
+                for (size_t rowi = 0; rowi < (size_t)S * U * R; ++rowi)
+                    std::copy(buf.begin() + rowi * W, buf.begin() + rowi * W + 16 * CH, eb.begin() + rowi * We);
                 edst.upload(eb.data(), eb.size(), s);
                 HIPCHK(hipStreamSynchronize(s));
             }

@@ -166,7 +166,8 @@ __global__ __launch_bounds__(1024) void k_type_groups(const int* node_types, int
 // Receivers in order of decreasing degree (counting sort on min(degree, 1023), one block).  The edge
 // kernels hand consecutive entries to the rows of a wavefront, which then finish together; the order
 // inside a degree class is whatever the LDS atomics leave and has no influence on any result.
-__device__ void degree_order_body(int N, const int* first_neigh, int* order)
+// `v` holds the CSR offsets (counts == false) or the degrees themselves (counts == true).
+__device__ void degree_order_body(int N, const int* v, int* order, bool counts = false)
 {
     __shared__ int start[1024];
     __shared__ int cur[1024];
@@ -175,7 +176,7 @@ __device__ void degree_order_body(int N, const int* first_neigh, int* order)
     start[tid] = 0; cur[tid] = 0;
     __syncthreads();
     for (int i = tid; i < N; i += 1024) {
-        const int d = min(max(first_neigh[i + 1] - first_neigh[i], 0), 1023);   // a negative count must not index below the table
+        const int d = min(max(counts ? v[i] : v[i + 1] - v[i], 0), 1023);   // a negative count must not index below the table
         atomicAdd(&start[1023 - d], 1);
     }
     __syncthreads();
@@ -195,7 +196,7 @@ __device__ void degree_order_body(int N, const int* first_neigh, int* order)
     start[tid] = base + incl - c;
     __syncthreads();
     for (int i = tid; i < N; i += 1024) {
-        const int b = 1023 - min(max(first_neigh[i + 1] - first_neigh[i], 0), 1023);
+        const int b = 1023 - min(max(counts ? v[i] : v[i + 1] - v[i], 0), 1023);
         order[start[b] + atomicAdd(&cur[b], 1)] = i;
     }
 }
@@ -261,7 +262,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists(const int* num_neigh,
     __syncthreads();
     type_groups_body(node_types, N, T, tstart, perm, sh);
 }
-// The same with the sender histogram in the same launch: block 0 forms the node lists, the other blocks
+// The same with the sender histogram in the same launch: blocks 0, 1, 2 form one node list each, the other blocks
 // count the senders (counters at zero on entry), which does not depend on the node lists.
 // With `chk.status` set the launch also checks everything the later kernels use as an address or a table argument
 // (species, sender rows, edge lengths, counts that add up to the edge totals) and raises bits in the status word.
@@ -271,6 +272,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_
                                                                 InputChecks chk)
 {
     extern __shared__ int sh[];
+    // the three node lists are independent of each other: a block each
     if (blockIdx.x == 0) {
         scan_single_body(num_neigh, first_neigh, N);
         __syncthreads();   // first_neigh, written by this block, is read back below
@@ -280,12 +282,12 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_
             if (threadIdx.x == 0) bad |= (first_neigh[N] != (int)chk.num_edges) | (first_neigh[chk.num_local_nodes] != (int)n);
             if (bad) atomicOr(chk.status, 1);
         }
-        degree_order_body(N, first_neigh, order);
-        __syncthreads();
-        type_groups_body(node_types, N, T, tstart, perm, sh);
         return;
     }
-    for (long i = (long)(blockIdx.x - 1) * SCAN_BLOCK + threadIdx.x; i < n; i += (long)(gridDim.x - 1) * SCAN_BLOCK) {
+    if (blockIdx.x == 1) { degree_order_body(N, num_neigh, order, true); return; }
+    if (blockIdx.x == 2) { type_groups_body(node_types, N, T, tstart, perm, sh); return; }
+    constexpr int LIST_BLOCKS = 3;
+    for (long i = (long)(blockIdx.x - LIST_BLOCKS) * SCAN_BLOCK + threadIdx.x; i < n; i += (long)(gridDim.x - LIST_BLOCKS) * SCAN_BLOCK) {
         const int j = key[i];
         if (j >= 0 && j < rows) rank[i] = atomicAdd(&count[j], 1);   // the entry's place inside its bucket
         else if (chk.status) atomicOr(chk.status, 1);
@@ -293,7 +295,7 @@ __global__ __launch_bounds__(SCAN_BLOCK) void k_node_lists_count(const int* num_
     if (chk.status) {
         // species and length of every edge (layer 0 covers the edges of ghost receivers as well)
         int bad = 0;
-        for (long i = (long)(blockIdx.x - 1) * SCAN_BLOCK + threadIdx.x; i < chk.num_edges; i += (long)(gridDim.x - 1) * SCAN_BLOCK) {
+        for (long i = (long)(blockIdx.x - LIST_BLOCKS) * SCAN_BLOCK + threadIdx.x; i < chk.num_edges; i += (long)(gridDim.x - LIST_BLOCKS) * SCAN_BLOCK) {
             const int t = chk.neigh_types[i];
             const double rr = chk.r[i];
             bad |= (t < 0 || t >= T) ? 1 : 0;
@@ -329,7 +331,7 @@ hipError_t launch_node_lists_count(const int* num_neigh, int N, int* first_neigh
 {
     if (N <= 0 || N > 64 * SCAN_BLOCK || T <= 0) return hipErrorInvalidValue;
     const long work = chk.status ? std::max(n, chk.num_edges) : n;
-    const unsigned nb = 1 + (unsigned)std::max<long>(1, std::min<long>((work + SCAN_BLOCK - 1) / SCAN_BLOCK, 2048));
+    const unsigned nb = 3 + (unsigned)std::max<long>(1, std::min<long>((work + SCAN_BLOCK - 1) / SCAN_BLOCK, 2048));
     hipLaunchKernelGGL(k_node_lists_count, dim3(nb), dim3(SCAN_BLOCK), 2 * T * sizeof(int), s, num_neigh, N, first_neigh,
                        order, node_types, T, tstart, perm, key, n, rows, count, rank, chk);
     return hipGetLastError();

@@ -29,7 +29,7 @@ struct WaveLds {
     static constexpr int NBT = BWD ? 4 * NBP : NBP;
     __host__ __device__ static constexpr size_t per_wave(int EC)
     {
-        size_t b = (size_t)EC * (NY * sizeof(double) + (BWD ? 4 * sizeof(double) : 0) + NBT * sizeof(F));
+        size_t b = (size_t)EC * (NY * sizeof(double) + (BWD ? 12 * sizeof(double) : 0) + NBT * sizeof(F));
         b += (size_t)EC * (sizeof(double) + 2 * sizeof(int));   // x (held as double-sized slot), rows, gather rows
         return (b + 15) / 16 * 16;
     }
@@ -90,11 +90,11 @@ struct BwdSteps {
     static constexpr int MAXLEN = max_len();
 };
 
-// Everything addressed through boffs after this point is scheduled after the four sums are final.
+// Everything addressed through boffs after this point is scheduled after the three sums are final.
 template <typename F>
-__device__ __forceinline__ void order_after(F& gx, F& gy, F& gz, F& srad, int& boffs)
+__device__ __forceinline__ void order_after(F& g1, F& g2, F& srad, int& boffs)
 {
-    asm volatile("" : "+v"(gx), "+v"(gy), "+v"(gz), "+v"(srad), "+v"(boffs));
+    asm volatile("" : "+v"(g1), "+v"(g2), "+v"(srad), "+v"(boffs));
 }
 
 // The value is final here: keeps an accumulation from drifting past the fences (its operands would stay live).
@@ -332,11 +332,14 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
     int* cg_start = cg_lm1 + num_terms;
     unsigned char* base = smem + WL::lists(num_terms) + (size_t)wave * WL::per_wave(EC);
     // the B block below is read with 4 * sizeof(F)-byte accesses: the doubles in front of it must keep that alignment
-    static_assert((EC * (64 + 4 + 1) * sizeof(double)) % (4 * sizeof(F)) == 0, "chunk size breaks the alignment of the B block");
+    static_assert((EC * (64 + 12 + 1) * sizeof(double)) % (4 * sizeof(F)) == 0, "chunk size breaks the alignment of the B block");
     double* Yt = reinterpret_cast<double*>(base);                                 // [EC][4][16]: Y, dY/dx, dY/dy, dY/dz
-    double* us = Yt + EC * 64;                                                    // [EC][4] unit vector xyz/r
-    double* xs = us + EC * 4;                                                     // [EC]
-    F* Bs = reinterpret_cast<F*>(xs + EC);                                        // [EC][NBP][4]: B, dB/dx, dB/dy, dB/dz
+    double* us = Yt + EC * 64;                                                    // [EC][12]: xyz/r, -, tangent t1, tangent t2, -, -
+    double* xs = us + EC * 12;                                                    // [EC]
+    // The harmonics depend on the direction only, so their gradient is tangential: two components in a frame
+    // (t1, t2) orthogonal to the direction carry it, and the contraction below costs three multiply-adds per
+    // entry instead of four.
+    F* Bs = reinterpret_cast<F*>(xs + EC);                                        // [EC][NBP][4]: B, dB.t1, dB.t2, -
     int* rows = reinterpret_cast<int*>(Bs + EC * 4 * NBP);
     int* grows = rows + EC;
 
@@ -382,7 +385,21 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
             const double r = a.r[e];
             // radial direction as the reference forms it: xyz / r with the caller's r
             const double ir = rcp_pos(r);
-            us[lane * 4] = dx * ir; us[lane * 4 + 1] = dy * ir; us[lane * 4 + 2] = dz * ir;
+            us[lane * 12] = dx * ir; us[lane * 12 + 1] = dy * ir; us[lane * 12 + 2] = dz * ir;
+            {
+                // t1 = n x a / |n x a| with a the axis the direction n is least aligned with (|n x a|^2 >= 2/3), t2 = n x t1
+                const double nx = dx * inv, ny = dy * inv, nz = dz * inv;
+                const double ax = fabs(nx), ay = fabs(ny), az = fabs(nz);
+                double t1x, t1y, t1z;
+                if (ax <= ay && ax <= az) { t1x = 0.0; t1y = nz; t1z = -ny; }
+                else if (ay <= az) { t1x = -nz; t1y = 0.0; t1z = nx; }
+                else { t1x = ny; t1y = -nx; t1z = 0.0; }
+                const double tn = rsqrt_pos(t1x * t1x + t1y * t1y + t1z * t1z);
+                t1x *= tn; t1y *= tn; t1z *= tn;
+                double* fr = us + lane * 12 + 4;
+                fr[0] = t1x; fr[1] = t1y; fr[2] = t1z;
+                fr[3] = ny * t1z - nz * t1y; fr[4] = nz * t1x - nx * t1z; fr[5] = nx * t1y - ny * t1x;
+            }
             const int n = spline_interval(r, a.spl_inv_h, a.spl_nodes - 2);
             xs[lane] = r - a.spl_h * n;
             const int tbl = a.pair_table[pair_index(a.T, ti, a.neigh_types[e])];
@@ -406,8 +423,12 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                             const double* y = Yt + le * 64 + cg_lm1[t];
                             s += cc * y[0]; sx += cc * y[16]; sy += cc * y[32]; sz += cc * y[48];
                         }
+                        const double* fr = us + le * 12 + 4;
                         Vec<F, 4> o;
-                        o.v[0] = (F)s; o.v[1] = (F)sx; o.v[2] = (F)sy; o.v[3] = (F)sz;
+                        o.v[0] = (F)s;
+                        o.v[1] = (F)(sx * fr[0] + sy * fr[1] + sz * fr[2]);
+                        o.v[2] = (F)(sx * fr[3] + sy * fr[4] + sz * fr[5]);
+                        o.v[3] = F(0);
                         *reinterpret_cast<Vec<F, 4>*>(Bs + ((size_t)le * NBP + b) * 4) = o;
                     }
                 }
@@ -421,8 +442,12 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                 const double* y = Yt + le * 64 + cg_lm1[t];
                 s += cc * y[0]; sx += cc * y[16]; sy += cc * y[32]; sz += cc * y[48];
             }
+            const double* fr = us + le * 12 + 4;
             Vec<F, 4> o;
-            o.v[0] = (F)s; o.v[1] = (F)sx; o.v[2] = (F)sy; o.v[3] = (F)sz;
+            o.v[0] = (F)s;
+            o.v[1] = (F)(sx * fr[0] + sy * fr[1] + sz * fr[2]);
+            o.v[2] = (F)(sx * fr[3] + sy * fr[4] + sz * fr[5]);
+            o.v[3] = F(0);
             *reinterpret_cast<Vec<F, 4>*>(Bs + ((size_t)le * NBP + b) * 4) = o;
         }
         }
@@ -445,7 +470,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
         // last of the chunk, which runs without: a request under a condition inside one loop body would make the
         // coefficients carried round the loop a merge of old and new registers (a register copy per value and edge).
         auto edge = [&](const int le, auto ahead) {
-            F srad = F(0), gx = F(0), gy = F(0), gz = F(0);
+            F srad = F(0), g1 = F(0), g2 = F(0);
             {
                 const F x = (F)xs[le];
                 const int grow = __builtin_amdgcn_readfirstlane(grows[le]);
@@ -473,14 +498,14 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                     }
                 if constexpr (AHEAD && decltype(ahead)::value) load_cf(le + 1);
                 // The B block of the edge is walked in steps (a few rows m of one path each).  Per path, the rows
-                // are summed first, u[m2][comp] = sum_m d[m] * (B, dB/dx, dB/dy, dB/dz)[m][m2], then one product
+                // are summed first, u[m2][comp] = sum_m d[m] * (B, dB.t1, dB.t2)[m][m2], then one product
                 // with the sender feature per m2.  The LDS reads of the next step are issued before the
                 // arithmetic of the current one (two register buffers); the fence after each step keeps
                 // reads further ahead from being issued (all at once would need several hundred registers).
                 using ST = BwdSteps<LMAXH, sizeof(F) == 8>;
                 constexpr bool LOOKAHEAD = true;
                 Vec<F, 4> buf[LOOKAHEAD ? 2 : 1][ST::MAXLEN];
-                F u[CPL][2 * LMAXH + 1][4];
+                F u[CPL][2 * LMAXH + 1][3];
                 auto load_step = [&](auto sc, Vec<F, 4>* dst) {
                     constexpr int s = decltype(sc)::value, p = ST::path(s), n2 = 2 * PT::l2(p) + 1;
                     const F* B4 = Bs + boffs + (PT::boff(p) + ST::m0(s) * n2) * 4;
@@ -503,8 +528,11 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
 #pragma unroll
                             for (int m2 = 0; m2 < n2; ++m2) {
                                 const Vec<F, 4>& bb = b4[(m - m0) * n2 + m2];
+                                // the unused fourth word counts as used where the others are: the read stays a 16-byte
+                                // one (a 12-byte LDS read is slower) and is not waited for any earlier
+                                asm volatile("" : : "v"(bb.v[3]));
 #pragma unroll
-                                for (int t = 0; t < 4; ++t)   // the first row of a path starts the sums
+                                for (int t = 0; t < 3; ++t)   // the first row of a path starts the sums
                                     u[c][m2][t] = m == 0 ? dd * bb.v[t] : u[c][m2][t] + dd * bb.v[t];
                             }
                         }
@@ -514,22 +542,22 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
 #pragma unroll
                         for (int m2 = 0; m2 < n2; ++m2)
 #pragma unroll
-                            for (int t = 0; t < 4; ++t) tie(u[c][m2][t], boffs);
+                            for (int t = 0; t < 3; ++t) tie(u[c][m2][t], boffs);
                     if constexpr (m1 == 2 * l + 1) {
 #pragma unroll
                         for (int c = 0; c < CPL; ++c) {
                             const F R = Rv[p][c], Rd = Rdv[p][c];
-                            F s0 = F(0), s1 = F(0), s2 = F(0), s3 = F(0);
+                            F s0 = F(0), s1 = F(0), s2 = F(0);
 #pragma unroll
                             for (int m2 = 0; m2 < n2; ++m2) {
                                 const F h = H[l2 * l2 + m2].v[c];
-                                s0 += u[c][m2][0] * h; s1 += u[c][m2][1] * h; s2 += u[c][m2][2] * h; s3 += u[c][m2][3] * h;
+                                s0 += u[c][m2][0] * h; s1 += u[c][m2][1] * h; s2 += u[c][m2][2] * h;
                                 mg[l2 * l2 + m2].v[c] += R * u[c][m2][0];
                             }
                             srad += Rd * s0;
-                            gx += R * s1; gy += R * s2; gz += R * s3;
+                            g1 += R * s1; g2 += R * s2;
                         }
-                        order_after(gx, gy, gz, srad, boffs);
+                        order_after(g1, g2, srad, boffs);
 #pragma unroll
                         for (int m2 = 0; m2 < n2; ++m2)
 #pragma unroll
@@ -542,22 +570,13 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                     for (int q = 0; q < NLM; ++q) *reinterpret_cast<Vec<F, CPL>*>(mrow + q * K) = mg[q];
                 }
             }
-            // Sums over the channels of the wavefront (a fixed tree: bit-reproducible).  Double precision: the three
-            // force components are put together per lane and summed.  Single-precision features: the four partial
-            // sums are added across the lanes in single precision (a third of the instructions) and put together in
-            // double afterwards.
-            double fx, fy, fz;
-            if constexpr (sizeof(F) == 8) {
-                const double sr = (double)srad;
-                fx = wave_sum(-(us[le * 4] * sr + (double)gx));
-                fy = wave_sum(-(us[le * 4 + 1] * sr + (double)gy));
-                fz = wave_sum(-(us[le * 4 + 2] * sr + (double)gz));
-            } else {
-                const double sr = (double)wave_sum(srad);
-                fx = -(us[le * 4] * sr + (double)wave_sum(gx));
-                fy = -(us[le * 4 + 1] * sr + (double)wave_sum(gy));
-                fz = -(us[le * 4 + 2] * sr + (double)wave_sum(gz));
-            }
+            // Sums over the channels of the wavefront (a fixed tree: bit-reproducible): the radial sum and the two
+            // tangential ones, in the feature precision; the force is put together from them in double.
+            const double sr = (double)wave_sum(srad), G1 = (double)wave_sum(g1), G2 = (double)wave_sum(g2);
+            const double* uf = us + le * 12;
+            const double fx = -(uf[0] * sr + uf[4] * G1 + uf[7] * G2);
+            const double fy = -(uf[1] * sr + uf[5] * G1 + uf[8] * G2);
+            const double fz = -(uf[2] * sr + uf[6] * G1 + uf[9] * G2);
             if (lane == 0) {
                 double* f = fout + 3 * (size_t)(eb + le);
                 if (add_forces) { f[0] += fx; f[1] += fy; f[2] += fz; }

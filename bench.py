@@ -33,8 +33,8 @@ sys.path.insert(0, HERE)
 
 HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 
-# kernel behind each edge stage: channel-slice kernels (scalar hidden features and at most four distinct radial
-# tables) / general kernels
+# kernel behind each edge stage: channel-slice kernels (scalar hidden features and one radial table for all
+# species pairs) / general kernels
 SLICE_KERNEL = {"agg0_fwd": "k_slice_fwd", "agg1_fwd": "k_slice_fwd", "agg1_bwd": "k_slice_bwd_edge",
                 "agg0_bwd": "k_slice_bwd_edge", "sender_reduce": "k_sender_reduce_linear"}
 GENERAL_KERNEL = {"agg0_fwd": "k_agg_fwd", "agg1_fwd": "k_agg_fwd", "agg1_bwd": "k_agg_bwd", "agg0_bwd": "k_agg_bwd",
@@ -44,7 +44,7 @@ EDGE_STAGES = ["agg0_fwd", "agg1_fwd", "agg1_bwd", "sender_reduce", "agg0_bwd"]
 
 def stage_kernel(stage, L_max, distinct_tables):
     """Name of the kernel that runs an edge stage for this kind of model."""
-    sliced = distinct_tables <= 4
+    sliced = distinct_tables == 1
     if stage.startswith("agg0"):
         return (SLICE_KERNEL if sliced else GENERAL_KERNEL)[stage]
     if stage == "sender_reduce":
@@ -237,7 +237,7 @@ def main():
                     help="periodic images as explicit ghost nodes that go through layer 0 only (the pair style's "
                          "no_mpi_message_passing layout on one rank) instead of senders mapped to their owners")
     ap.add_argument("--pair-tables", action="store_true",
-                    help="a radial table of its own for every species pair (more than four distinct tables take the "
+                    help="a radial table of its own for every species pair (several distinct tables take the "
                          "general edge kernels)")
     ap.add_argument("--no-second", action="store_true",
                     help="default workload only: skip the second configuration of the metric (mp_medium, float32 features) "

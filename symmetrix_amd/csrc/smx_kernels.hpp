@@ -66,7 +66,6 @@ template <typename F>
 struct SliceParams {
     AggParams<F> a;
     const F* tabS;
-    int U;             // unique radial tables (one pass over the edges per table)
     int W;             // padded row length in elements
     int CH;            // channels per slice
     double cdiag[16];

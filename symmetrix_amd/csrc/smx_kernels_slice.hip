@@ -42,7 +42,7 @@ __device__ __forceinline__ int next_block_task(int* counter)
 
 struct EdgeGeo {
     double dx, dy, dz, r;
-    int g, tj;
+    int g;
 };
 template <typename F>
 __device__ __forceinline__ EdgeGeo load_edge(const AggParams<F>& a, int e)
@@ -51,7 +51,6 @@ __device__ __forceinline__ EdgeGeo load_edge(const AggParams<F>& a, int e)
     q.dx = a.xyz[3 * (size_t)e]; q.dy = a.xyz[3 * (size_t)e + 1]; q.dz = a.xyz[3 * (size_t)e + 2];
     q.r = a.r[e];
     q.g = a.gather[e];
-    q.tj = a.neigh_types[e];
     return q;
 }
 
@@ -111,79 +110,74 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
     const int wave_tasks = (a.num_nodes + 3) / 4;
     __shared__ int task_counter;
 
-    for (int u = 0; u < p.U; ++u) {
-        __syncthreads();
-        if (threadIdx.x == 0) task_counter = 0;
-        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
-        __syncthreads();
-        for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
-             task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
-            const int slot = task * 4 + (lane >> 4);
-            const bool live = slot < a.num_nodes;
-            const int i = live ? p.order[slot] : 0;
-            int e0 = 0, e1 = 0, ti = 0;
-            if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
-            F acc[16][CPLN];
+    if (threadIdx.x == 0) task_counter = 0;
+    copy_slice_to_lds(p.tabS + (size_t)slice * R * W, smem, (size_t)R * W * sizeof(F));
+    __syncthreads();
+    for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
+         task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
+        const int slot = task * 4 + (lane >> 4);
+        const bool live = slot < a.num_nodes;
+        const int i = live ? p.order[slot] : 0;
+        int e0 = 0, e1 = 0;
+        if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; }
+        F acc[16][CPLN];
 #pragma unroll
-            for (int q = 0; q < 16; ++q)
+        for (int q = 0; q < 16; ++q)
 #pragma unroll
-                for (int c = 0; c < CPLN; ++c) acc[q][c] = F(0);
-            // the geometry of the next edge of this lane is loaded while the current one is processed
-            EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0, 0};
-            {
-                const int ef = e0 + e_sub;
-                if (ef < e1) nx = load_edge(a, ef);
+            for (int c = 0; c < CPLN; ++c) acc[q][c] = F(0);
+        // the geometry of the next edge of this lane is loaded while the current one is processed
+        EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0};
+        {
+            const int ef = e0 + e_sub;
+            if (ef < e1) nx = load_edge(a, ef);
+        }
+        for (int e = e0 + e_sub; e < e1; e += EPR) {
+            const EdgeGeo cu = nx;
+            nx = load_edge(a, min(e + EPR, e1 - 1));   // unconditional: a conditional load costs a register copy per value
+            const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
+            const double r = cu.r;
+            const int g = cu.g;
+            const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
+            double Yd[16];
+            sph_l3(dz * inv, dx * inv, dy * inv, Yd);
+            const int n = spline_interval(r, a.spl_inv_h, R - 1);
+            const F x = (F)(r - a.spl_h * n);
+            const F* row = lds + (size_t)n * W + cs * CPLN;
+            // step i reads path (i + rot) & 3, rot = this lane's edge slot in single precision, else 0
+            F t[CPLN][4];
+#pragma unroll
+            for (int c = 0; c < CPLN; ++c) {
+                const F h = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const F* rp = row + poff[i] + c;
+                    const F c0 = rp[0], c1 = rp[4 * CH], c2 = rp[8 * CH], c3 = rp[12 * CH];
+                    t[c][i] = (c0 + x * (c1 + x * (c2 + x * c3))) * h;
+                }
+                if constexpr (slice_rotates<F>()) unrotate4(t[c], rot);
             }
-            for (int e = e0 + e_sub; e < e1; e += EPR) {
-                const EdgeGeo cu = nx;
-                nx = load_edge(a, min(e + EPR, e1 - 1));   // unconditional: a conditional load costs a register copy per value
-                const int tj = cu.tj;
-                if (p.U > 1 && a.pair_table[pair_index(a.T, ti, tj)] != u) continue;
-                const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
-                const double r = cu.r;
-                const int g = cu.g;
-                const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
-                double Yd[16];
-                sph_l3(dz * inv, dx * inv, dy * inv, Yd);
-                const int n = spline_interval(r, a.spl_inv_h, R - 1);
-                const F x = (F)(r - a.spl_h * n);
-                const F* row = lds + (size_t)n * W + cs * CPLN;
-                // step i reads path (i + rot) & 3, rot = this lane's edge slot in single precision, else 0
-                F t[CPLN][4];
 #pragma unroll
-                for (int c = 0; c < CPLN; ++c) {
-                    const F h = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)];
+            for (int q = 0; q < 16; ++q) {
+                const F y = (F)Yd[q];
 #pragma unroll
-                    for (int i = 0; i < 4; ++i) {
-                        const F* rp = row + poff[i] + c;
-                        const F c0 = rp[0], c1 = rp[4 * CH], c2 = rp[8 * CH], c3 = rp[12 * CH];
-                        t[c][i] = (c0 + x * (c1 + x * (c2 + x * c3))) * h;
+                for (int c = 0; c < CPLN; ++c) acc[q][c] += t[c][lm_l(q)] * y;
+            }
+        }
+        // add up the lanes of the row that hold the same channels (they took alternate edges)
+#pragma unroll
+        for (int q = 0; q < 16; ++q)
+#pragma unroll
+            for (int c = 0; c < CPLN; ++c) acc[q][c] = row_sum_strided<CL>(acc[q][c]);
+        if (live && e_sub == 0) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const F cd = (F)p.cdiag[q];
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c)
+                    if (kc + c < K) {
+                        F* o = a.out + ((size_t)i * 16 + q) * K + kc + c;
+                        *o = acc[q][c] * cd;
                     }
-                    if constexpr (slice_rotates<F>()) unrotate4(t[c], rot);
-                }
-#pragma unroll
-                for (int q = 0; q < 16; ++q) {
-                    const F y = (F)Yd[q];
-#pragma unroll
-                    for (int c = 0; c < CPLN; ++c) acc[q][c] += t[c][lm_l(q)] * y;
-                }
-            }
-            // add up the lanes of the row that hold the same channels (they took alternate edges)
-#pragma unroll
-            for (int q = 0; q < 16; ++q)
-#pragma unroll
-                for (int c = 0; c < CPLN; ++c) acc[q][c] = row_sum_strided<CL>(acc[q][c]);
-            if (live && e_sub == 0) {
-#pragma unroll
-                for (int q = 0; q < 16; ++q) {
-                    const F cd = (F)p.cdiag[q];
-#pragma unroll
-                    for (int c = 0; c < CPLN; ++c)
-                        if (kc + c < K) {
-                            F* o = a.out + ((size_t)i * 16 + q) * K + kc + c;
-                            *o = (u == 0) ? acc[q][c] * cd : *o + acc[q][c] * cd;
-                        }
-                }
             }
         }
     }
@@ -210,116 +204,112 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     __shared__ int task_counter;
     double* fpart = p.fpart + (size_t)slice * p.E * 3;
 
-    for (int u = 0; u < p.U; ++u) {
-        __syncthreads();
-        if (threadIdx.x == 0) task_counter = 0;
-        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
-        __syncthreads();
-        for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
-             task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
-            const int slot = task * 4 + (lane >> 4);
-            const bool live = slot < a.num_nodes;
-            const int i = live ? p.order[slot] : 0;
-            int e0 = 0, e1 = 0, ti = 0;
-            if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
-            F d[16][CPLN];
+    if (threadIdx.x == 0) task_counter = 0;
+    copy_slice_to_lds(p.tabS + (size_t)slice * R * W, smem, (size_t)R * W * sizeof(F));
+    __syncthreads();
+    for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
+         task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
+        const int slot = task * 4 + (lane >> 4);
+        const bool live = slot < a.num_nodes;
+        const int i = live ? p.order[slot] : 0;
+        int e0 = 0, e1 = 0;
+        if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; }
+        F d[16][CPLN];
 #pragma unroll
-            for (int q = 0; q < 16; ++q) {
-                const F cd = (F)p.cdiag[q];
+        for (int q = 0; q < 16; ++q) {
+            const F cd = (F)p.cdiag[q];
 #pragma unroll
-                for (int c = 0; c < CPLN; ++c)
-                    d[q][c] = (live && kc + c < K) ? a.d_out[((size_t)i * 16 + q) * K + kc + c] * cd : F(0);
-            }
-            // the lanes of a row iterate together so that the cross-lane sums below see all CL partners
-            const int iters = (e1 - e0 + EPR - 1) / EPR;
-            EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0, 0};
-            {
-                const int ef = e0 + e_sub;
-                if (ef < e1) nx = load_edge(a, ef);
-            }
-            for (int it = 0; it < iters; ++it) {
-                const int e = e0 + it * EPR + e_sub;
-                bool on = e < e1;
-                const EdgeGeo cu = nx;
-                nx = load_edge(a, min(e + EPR, e1 - 1));   // unconditional: a conditional load costs a register copy per value
-                if (on && p.U > 1 && a.pair_table[pair_index(a.T, ti, cu.tj)] != u) on = false;
-                double fx = 0.0, fy = 0.0, fz = 0.0;
-                if (on) {
-                    const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
-                    const double r = cu.r;
-                    const int g = cu.g;
-                    const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
-                    const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
-                    const int n = spline_interval(r, a.spl_inv_h, R - 1);
-                    const F x = (F)(r - a.spl_h * n);
-                    const F* row = lds + (size_t)n * W + cs * CPLN;
-                    F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
-                    F h[CPLN], mg[CPLN], Rv[CPLN][4], Rd[CPLN][4];
+            for (int c = 0; c < CPLN; ++c)
+                d[q][c] = (live && kc + c < K) ? a.d_out[((size_t)i * 16 + q) * K + kc + c] * cd : F(0);
+        }
+        // the lanes of a row iterate together so that the cross-lane sums below see all CL partners
+        const int iters = (e1 - e0 + EPR - 1) / EPR;
+        EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0};
+        {
+            const int ef = e0 + e_sub;
+            if (ef < e1) nx = load_edge(a, ef);
+        }
+        for (int it = 0; it < iters; ++it) {
+            const int e = e0 + it * EPR + e_sub;
+            bool on = e < e1;
+            const EdgeGeo cu = nx;
+            nx = load_edge(a, min(e + EPR, e1 - 1));   // unconditional: a conditional load costs a register copy per value
+            double fx = 0.0, fy = 0.0, fz = 0.0;
+            if (on) {
+                const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
+                const double r = cu.r;
+                const int g = cu.g;
+                const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
+                const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
+                const int n = spline_interval(r, a.spl_inv_h, R - 1);
+                const F x = (F)(r - a.spl_h * n);
+                const F* row = lds + (size_t)n * W + cs * CPLN;
+                F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
+                F h[CPLN], mg[CPLN], Rv[CPLN][4], Rd[CPLN][4];
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c) {
+                    h[c] = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)]; mg[c] = F(0);
+                    // paths read in the rotated order of this lane's edge slot (see the forward kernel)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) {
+                        const F* rp = row + poff[i] + c;
+                        const F c0 = rp[0], c1 = rp[4 * CH], c2 = rp[8 * CH], c3 = rp[12 * CH];
+                        Rv[c][i] = c0 + x * (c1 + x * (c2 + x * c3));
+                        Rd[c][i] = c1 + x * (F(2) * c2 + F(3) * x * c3);
+                    }
+                    if constexpr (slice_rotates<F>()) { unrotate4(Rv[c], rot); unrotate4(Rd[c], rot); }
+                }
+                // One order l at a time: its harmonics are formed, used for all channels of the lane and
+                // dropped; the fence keeps the next order's harmonics from being formed early (all 16
+                // with their derivatives would hold 128 registers).
+                double vx = ux, vy = uy, vz = uz;
+                static_for<0, 4>([&](auto lc) {
+                    constexpr int l = decltype(lc)::value;
+                    F Yl[2 * l + 1], g0[2 * l + 1], g1[2 * l + 1], g2[2 * l + 1];
+                    static_for<0, 2 * l + 1>([&](auto mc) {
+                        constexpr int m = decltype(mc)::value;
+                        double y, a0, a1, a2;
+                        ylm_g<l * l + m>(vx, vy, vz, y, a0, a1, a2);
+                        Yl[m] = (F)y; g0[m] = (F)a0; g1[m] = (F)a1; g2[m] = (F)a2;
+                    });
 #pragma unroll
                     for (int c = 0; c < CPLN; ++c) {
-                        h[c] = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)]; mg[c] = F(0);
-                        // paths read in the rotated order of this lane's edge slot (see the forward kernel)
+                        F ul = F(0), v0 = F(0), v1 = F(0), v2 = F(0);
 #pragma unroll
-                        for (int i = 0; i < 4; ++i) {
-                            const F* rp = row + poff[i] + c;
-                            const F c0 = rp[0], c1 = rp[4 * CH], c2 = rp[8 * CH], c3 = rp[12 * CH];
-                            Rv[c][i] = c0 + x * (c1 + x * (c2 + x * c3));
-                            Rd[c][i] = c1 + x * (F(2) * c2 + F(3) * x * c3);
+                        for (int m = 0; m < 2 * l + 1; ++m) {
+                            const F dd = d[l * l + m][c];
+                            ul += dd * Yl[m];
+                            v0 += dd * g0[m]; v1 += dd * g1[m]; v2 += dd * g2[m];
                         }
-                        if constexpr (slice_rotates<F>()) { unrotate4(Rv[c], rot); unrotate4(Rd[c], rot); }
+                        const F Rh = Rv[c][l] * h[c];
+                        srad += Rd[c][l] * h[c] * ul;
+                        wx += Rh * v0; wy += Rh * v1; wz += Rh * v2;
+                        lterm += Rh * ul * F(l);
+                        mg[c] += Rv[c][l] * ul;
                     }
-                    // One order l at a time: its harmonics are formed, used for all channels of the lane and
-                    // dropped; the fence keeps the next order's harmonics from being formed early (all 16
-                    // with their derivatives would hold 128 registers).
-                    double vx = ux, vy = uy, vz = uz;
-                    static_for<0, 4>([&](auto lc) {
-                        constexpr int l = decltype(lc)::value;
-                        F Yl[2 * l + 1], g0[2 * l + 1], g1[2 * l + 1], g2[2 * l + 1];
-                        static_for<0, 2 * l + 1>([&](auto mc) {
-                            constexpr int m = decltype(mc)::value;
-                            double y, a0, a1, a2;
-                            ylm_g<l * l + m>(vx, vy, vz, y, a0, a1, a2);
-                            Yl[m] = (F)y; g0[m] = (F)a0; g1[m] = (F)a1; g2[m] = (F)a2;
-                        });
+                    order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
 #pragma unroll
-                        for (int c = 0; c < CPLN; ++c) {
-                            F ul = F(0), v0 = F(0), v1 = F(0), v2 = F(0);
+                    for (int c = 0; c < CPLN; ++c) pin_value(mg[c]);
+                });
+                if (a.msg) {
 #pragma unroll
-                            for (int m = 0; m < 2 * l + 1; ++m) {
-                                const F dd = d[l * l + m][c];
-                                ul += dd * Yl[m];
-                                v0 += dd * g0[m]; v1 += dd * g1[m]; v2 += dd * g2[m];
-                            }
-                            const F Rh = Rv[c][l] * h[c];
-                            srad += Rd[c][l] * h[c] * ul;
-                            wx += Rh * v0; wy += Rh * v1; wz += Rh * v2;
-                            lterm += Rh * ul * F(l);
-                            mg[c] += Rv[c][l] * ul;
-                        }
-                        order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
-#pragma unroll
-                        for (int c = 0; c < CPLN; ++c) pin_value(mg[c]);
-                    });
-                    if (a.msg) {
-#pragma unroll
-                        for (int c = 0; c < CPLN; ++c)
-                            if (kc + c < K) a.msg[(size_t)e * K + kc + c] = mg[c];
-                    }
-                    // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
-                    // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
-                    const double sr = (double)srad, lt = (double)lterm;
-                    const double ir = rcp_pos(r);
-                    fx = -(dx * ir * sr + ((double)wy - uy * lt) * inv);   // original x is permuted axis 1
-                    fy = -(dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
-                    fz = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
+                    for (int c = 0; c < CPLN; ++c)
+                        if (kc + c < K) a.msg[(size_t)e * K + kc + c] = mg[c];
                 }
-                // channels of the slice are spread over CL adjacent lanes: add their partial forces
-                if constexpr (CL >= 2) { fx += lane_xor1(fx); fy += lane_xor1(fy); fz += lane_xor1(fz); }
-                if constexpr (CL >= 4) { fx += lane_xor2(fx); fy += lane_xor2(fy); fz += lane_xor2(fz); }
-                if constexpr (CL >= 8) { fx += half_mirror(fx); fy += half_mirror(fy); fz += half_mirror(fz); }
-                if (on && cs == 0) {
-                    fpart[3 * (size_t)e] = fx; fpart[3 * (size_t)e + 1] = fy; fpart[3 * (size_t)e + 2] = fz;
-                }
+                // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
+                // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
+                const double sr = (double)srad, lt = (double)lterm;
+                const double ir = rcp_pos(r);
+                fx = -(dx * ir * sr + ((double)wy - uy * lt) * inv);   // original x is permuted axis 1
+                fy = -(dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
+                fz = -(dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
+            }
+            // channels of the slice are spread over CL adjacent lanes: add their partial forces
+            if constexpr (CL >= 2) { fx += lane_xor1(fx); fy += lane_xor1(fy); fz += lane_xor1(fz); }
+            if constexpr (CL >= 4) { fx += lane_xor2(fx); fy += lane_xor2(fy); fz += lane_xor2(fz); }
+            if constexpr (CL >= 8) { fx += half_mirror(fx); fy += half_mirror(fy); fz += half_mirror(fz); }
+            if (on && cs == 0) {
+                fpart[3 * (size_t)e] = fx; fpart[3 * (size_t)e + 1] = fy; fpart[3 * (size_t)e + 2] = fz;
             }
         }
     }
@@ -357,136 +347,132 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     __shared__ int task_counter;
     double* fpart = p.fpart + (size_t)slice * p.E * 3;
 
-    for (int u = 0; u < p.U; ++u) {
-        __syncthreads();
-        if (threadIdx.x == 0) task_counter = 0;
-        copy_slice_to_lds(p.tabS + ((size_t)slice * p.U + u) * R * W, smem, (size_t)R * W * sizeof(F));
-        __syncthreads();
-        for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
-             task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
-            const int slot = task * ROWS + row;
-            const bool live = slot < a.num_nodes;
-            const int i = live ? p.order[slot] : 0;
-            int e0 = 0, e1 = 0, ti = 0;
-            if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; ti = a.node_types[i]; }
-            // the lanes of the row bring the receiver's adjoint rows, one harmonic each per round
-            wave_lds_sync();                                       // the previous task's reads are done
+    if (threadIdx.x == 0) task_counter = 0;
+    copy_slice_to_lds(p.tabS + (size_t)slice * R * W, smem, (size_t)R * W * sizeof(F));
+    __syncthreads();
+    for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
+         task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
+        const int slot = task * ROWS + row;
+        const bool live = slot < a.num_nodes;
+        const int i = live ? p.order[slot] : 0;
+        int e0 = 0, e1 = 0;
+        if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; }
+        // the lanes of the row bring the receiver's adjoint rows, one harmonic each per round
+        wave_lds_sync();                                       // the previous task's reads are done
 #pragma unroll
-            for (int lm = sub; lm < 16; lm += RL) {
-                V v;
+        for (int lm = sub; lm < 16; lm += RL) {
+            V v;
 #pragma unroll
-                for (int c = 0; c < CH; ++c) v.v[c] = F(0);
-                if (live) {
-                    const F* src = a.d_out + ((size_t)i * 16 + lm) * K + kc;
-                    if (whole) v = *reinterpret_cast<const V*>(src);
-                    else {
+            for (int c = 0; c < CH; ++c) v.v[c] = F(0);
+            if (live) {
+                const F* src = a.d_out + ((size_t)i * 16 + lm) * K + kc;
+                if (whole) v = *reinterpret_cast<const V*>(src);
+                else {
 #pragma unroll
-                        for (int c = 0; c < CH; ++c) if (kc + c < K) v.v[c] = src[c];
-                    }
+                    for (int c = 0; c < CH; ++c) if (kc + c < K) v.v[c] = src[c];
                 }
-                const F cd = (F)p.cdiag[lm];
-#pragma unroll
-                for (int c = 0; c < CH; ++c) v.v[c] *= cd;
-                *reinterpret_cast<V*>(dstage + lm * ROWS * CH) = v;
             }
-            wave_lds_sync();
-            const int iters = (e1 - e0 + RL - 1) / RL;
-            EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0, 0};
-            if (e0 + sub < e1) nx = load_edge(a, e0 + sub);
-            for (int it = 0; it < iters; ++it) {
-                const int e = e0 + it * RL + sub;
-                bool on = e < e1;
-                const EdgeGeo cu = nx;
-                nx = load_edge(a, min(e + RL, e1 - 1));   // unconditional: a conditional load costs a register copy per value
-                if (on && p.U > 1 && a.pair_table[pair_index(a.T, ti, cu.tj)] != u) on = false;
-                if (!on) continue;
-                // sender row first: its latency hides behind the radial part
-                V h;
+            const F cd = (F)p.cdiag[lm];
+#pragma unroll
+            for (int c = 0; c < CH; ++c) v.v[c] *= cd;
+            *reinterpret_cast<V*>(dstage + lm * ROWS * CH) = v;
+        }
+        wave_lds_sync();
+        const int iters = (e1 - e0 + RL - 1) / RL;
+        EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0};
+        if (e0 + sub < e1) nx = load_edge(a, e0 + sub);
+        for (int it = 0; it < iters; ++it) {
+            const int e = e0 + it * RL + sub;
+            bool on = e < e1;
+            const EdgeGeo cu = nx;
+            nx = load_edge(a, min(e + RL, e1 - 1));   // unconditional: a conditional load costs a register copy per value
+            if (!on) continue;
+            // sender row first: its latency hides behind the radial part
+            V h;
+            {
+                const F* src = a.Hsrc + (size_t)cu.g * K + kc;
+                if (whole) h = *reinterpret_cast<const V*>(src);
+                else {
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) h.v[c] = src[min(c, K - 1 - kc)];
+                }
+            }
+            // partial forces an earlier stage left for this edge: requested now, added at the end
+            double f0 = 0.0, f1 = 0.0, f2 = 0.0;
+            if (e < p.fpart_carry) { f0 = fpart[3 * (size_t)e]; f1 = fpart[3 * (size_t)e + 1]; f2 = fpart[3 * (size_t)e + 2]; }
+            const double dx = cu.dx, dy = cu.dy, dz = cu.dz, r = cu.r;
+            const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
+            const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
+            const int n = spline_interval(r, a.spl_inv_h, R - 1);
+            const F x = (F)(r - a.spl_h * n);
+            const F* rowp = lds + (size_t)n * W;
+            auto piece = [&](int q, int l) { return *reinterpret_cast<const V*>(rowp + (q * 4 + l) * CH); };
+            F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
+            F mg[CH];
+#pragma unroll
+            for (int c = 0; c < CH; ++c) mg[c] = F(0);
+            double vx = ux, vy = uy, vz = uz;
+            // one order l at a time (the fence keeps the harmonics of the next order from being formed early)
+            static_for<0, 4>([&](auto lc) {
+                constexpr int l = decltype(lc)::value;
+                F ul[CH];
+#pragma unroll
+                for (int c = 0; c < CH; ++c) ul[c] = F(0);
+                F py = F(0);
+                // sender row times radial value / derivative once per order, not once per harmonic
+                F Rv[CH], hv[CH], hd[CH];
                 {
-                    const F* src = a.Hsrc + (size_t)cu.g * K + kc;
-                    if (whole) h = *reinterpret_cast<const V*>(src);
-                    else {
+                    const V c0 = piece(0, l), c1 = piece(1, l), c2 = piece(2, l), c3 = piece(3, l);
 #pragma unroll
-                        for (int c = 0; c < CH; ++c) h.v[c] = src[min(c, K - 1 - kc)];
+                    for (int c = 0; c < CH; ++c) {
+                        Rv[c] = c0.v[c] + x * (c1.v[c] + x * (c2.v[c] + x * c3.v[c]));
+                        hv[c] = h.v[c] * Rv[c];
+                        hd[c] = h.v[c] * (c1.v[c] + x * (F(2) * c2.v[c] + F(3) * x * c3.v[c]));
                     }
                 }
-                // partial forces an earlier stage left for this edge: requested now, added at the end
-                double f0 = 0.0, f1 = 0.0, f2 = 0.0;
-                if (e < p.fpart_carry) { f0 = fpart[3 * (size_t)e]; f1 = fpart[3 * (size_t)e + 1]; f2 = fpart[3 * (size_t)e + 2]; }
-                const double dx = cu.dx, dy = cu.dy, dz = cu.dz, r = cu.r;
-                const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
-                const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
-                const int n = spline_interval(r, a.spl_inv_h, R - 1);
-                const F x = (F)(r - a.spl_h * n);
-                const F* rowp = lds + (size_t)n * W;
-                auto piece = [&](int q, int l) { return *reinterpret_cast<const V*>(rowp + (q * 4 + l) * CH); };
-                F srad = F(0), wx = F(0), wy = F(0), wz = F(0), lterm = F(0);
-                F mg[CH];
+                static_for<0, 2 * l + 1>([&](auto mc) {
+                    constexpr int lm = l * l + decltype(mc)::value;
+                    double y, g0, g1, g2;
+                    ylm_g<lm>(vx, vy, vz, y, g0, g1, g2);
+                    const V dd = *reinterpret_cast<const V*>(dstage + lm * ROWS * CH);
+                    const F yf = (F)y;
+                    F P = F(0), Q = F(0);
 #pragma unroll
-                for (int c = 0; c < CH; ++c) mg[c] = F(0);
-                double vx = ux, vy = uy, vz = uz;
-                // one order l at a time (the fence keeps the harmonics of the next order from being formed early)
-                static_for<0, 4>([&](auto lc) {
-                    constexpr int l = decltype(lc)::value;
-                    F ul[CH];
-#pragma unroll
-                    for (int c = 0; c < CH; ++c) ul[c] = F(0);
-                    F py = F(0);
-                    // sender row times radial value / derivative once per order, not once per harmonic
-                    F Rv[CH], hv[CH], hd[CH];
-                    {
-                        const V c0 = piece(0, l), c1 = piece(1, l), c2 = piece(2, l), c3 = piece(3, l);
-#pragma unroll
-                        for (int c = 0; c < CH; ++c) {
-                            Rv[c] = c0.v[c] + x * (c1.v[c] + x * (c2.v[c] + x * c3.v[c]));
-                            hv[c] = h.v[c] * Rv[c];
-                            hd[c] = h.v[c] * (c1.v[c] + x * (F(2) * c2.v[c] + F(3) * x * c3.v[c]));
-                        }
+                    for (int c = 0; c < CH; ++c) {
+                        P += dd.v[c] * hv[c];
+                        Q += dd.v[c] * hd[c];
+                        ul[c] += dd.v[c] * yf;
                     }
-                    static_for<0, 2 * l + 1>([&](auto mc) {
-                        constexpr int lm = l * l + decltype(mc)::value;
-                        double y, g0, g1, g2;
-                        ylm_g<lm>(vx, vy, vz, y, g0, g1, g2);
-                        const V dd = *reinterpret_cast<const V*>(dstage + lm * ROWS * CH);
-                        const F yf = (F)y;
-                        F P = F(0), Q = F(0);
-#pragma unroll
-                        for (int c = 0; c < CH; ++c) {
-                            P += dd.v[c] * hv[c];
-                            Q += dd.v[c] * hd[c];
-                            ul[c] += dd.v[c] * yf;
-                        }
-                        srad += Q * yf;
-                        wx += P * (F)g0; wy += P * (F)g1; wz += P * (F)g2;
-                        py += P * yf;
-                    });
-                    lterm += py * F(l);
-#pragma unroll
-                    for (int c = 0; c < CH; ++c) mg[c] += Rv[c] * ul[c];
-                    order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
-#pragma unroll
-                    for (int c = 0; c < CH; ++c) pin_value(mg[c]);
+                    srad += Q * yf;
+                    wx += P * (F)g0; wy += P * (F)g1; wz += P * (F)g2;
+                    py += P * yf;
                 });
-                if (a.msg) {
-                    F* dstm = a.msg + (size_t)e * K + kc;
-                    if (whole) {
-                        V m;
+                lterm += py * F(l);
 #pragma unroll
-                        for (int c = 0; c < CH; ++c) m.v[c] = mg[c];
-                        *reinterpret_cast<V*>(dstm) = m;
-                    } else {
+                for (int c = 0; c < CH; ++c) mg[c] += Rv[c] * ul[c];
+                order_l(srad, wx, wy, wz, lterm, vx, vy, vz);
 #pragma unroll
-                        for (int c = 0; c < CH; ++c) if (kc + c < K) dstm[c] = mg[c];
-                    }
+                for (int c = 0; c < CH; ++c) pin_value(mg[c]);
+            });
+            if (a.msg) {
+                F* dstm = a.msg + (size_t)e * K + kc;
+                if (whole) {
+                    V m;
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) m.v[c] = mg[c];
+                    *reinterpret_cast<V*>(dstm) = m;
+                } else {
+#pragma unroll
+                    for (int c = 0; c < CH; ++c) if (kc + c < K) dstm[c] = mg[c];
                 }
-                // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
-                // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
-                const double sr = (double)srad, lt = (double)lterm;
-                const double ir = rcp_pos(r);
-                fpart[3 * (size_t)e] = f0 - (dx * ir * sr + ((double)wy - uy * lt) * inv);       // original x is permuted axis 1
-                fpart[3 * (size_t)e + 1] = f1 - (dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
-                fpart[3 * (size_t)e + 2] = f2 - (dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
             }
+            // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
+            // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
+            const double sr = (double)srad, lt = (double)lterm;
+            const double ir = rcp_pos(r);
+            fpart[3 * (size_t)e] = f0 - (dx * ir * sr + ((double)wy - uy * lt) * inv);       // original x is permuted axis 1
+            fpart[3 * (size_t)e + 1] = f1 - (dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
+            fpart[3 * (size_t)e + 2] = f2 - (dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
         }
     }
 }

@@ -21,13 +21,25 @@ namespace smx {
 
 namespace {
 
+// The table slice of a block, global memory -> LDS (both sides 16-byte aligned, size a multiple of 16).  Whole
+// kilobytes go through loads that write straight into LDS (16 bytes per lane, the 64 lanes of a wavefront side by
+// side, no registers in between), so that a wavefront has all its pieces in flight at once; the caller's barrier
+// follows the wait for them.
 __device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, size_t bytes)
 {
-    // both sides 16-byte aligned, size a multiple of 16
-    const uint4* s = reinterpret_cast<const uint4*>(src);
-    uint4* d = reinterpret_cast<uint4*>(dst);
-    const size_t n = bytes / 16;
-    for (size_t q = threadIdx.x; q < n; q += blockDim.x) d[q] = s[q];
+    typedef const __attribute__((address_space(1))) void* GlobalPtr;
+    typedef __attribute__((address_space(3))) void* LdsPtr;
+    const char* s = reinterpret_cast<const char*>(src);
+    char* d = reinterpret_cast<char*>(dst);
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6)), lane = threadIdx.x & 63;
+    const int waves = blockDim.x >> 6;
+    const int chunks = (int)(bytes / 1024);
+    for (int q = wave; q < chunks; q += waves)
+        __builtin_amdgcn_global_load_lds((GlobalPtr)(s + (size_t)q * 1024 + lane * 16), (LdsPtr)(d + (size_t)q * 1024), 16, 0, 0);
+    const size_t tail = (size_t)chunks * 1024;
+    for (size_t q = tail + threadIdx.x * 16; q < bytes; q += (size_t)blockDim.x * 16)
+        *reinterpret_cast<uint4*>(d + q) = *reinterpret_cast<const uint4*>(s + q);
+    __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the direct loads have written the LDS
 }
 
 // The tasks of a block (groups of receivers, largest first) are handed to its wavefronts as they become free: an

@@ -33,6 +33,11 @@ struct WaveLds {
         b += (size_t)EC * (sizeof(double) + 2 * sizeof(int));   // x (held as double-sized slot), rows, gather rows
         return (b + 15) / 16 * 16;
     }
+    // Double-precision forward kernel with vector sender features: the coefficients of the first PRE paths of the
+    // next edge wait in LDS, brought there by loads that bypass the registers (32 bytes per lane and path).
+    static constexpr bool PREFETCH = !BWD && sizeof(F) == 8 && LMAXH == 1;
+    static constexpr int PRE = PREFETCH ? PT::P / 2 : 0;
+    __host__ __device__ static constexpr size_t prefetch_per_wave() { return (size_t)PRE * 64 * 32; }
     __host__ __device__ static constexpr size_t lists(int num_terms)
     {
         return ((size_t)num_terms * (sizeof(double) + sizeof(int)) + (PT::NB + 1) * sizeof(int) + 15) / 16 * 16;
@@ -265,6 +270,29 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
                     for (int m2 = 0; m2 < 2 * PT::l2(q) + 1; ++m2) w[q][c][m2] = R * H[PT::l2(q) * PT::l2(q) + m2].v[c];
                 }
         };
+        // coefficient buffer of this wavefront: [PRE paths][2 halves][64 lanes] 16-byte words
+        unsigned char* pre = smem + WL::lists(num_terms) + 4 * WL::per_wave(EC) + (size_t)wave * WL::prefetch_per_wave();
+        constexpr int PRE = WL::PRE;
+        Vec<F, CPL> Hn[NLM];
+        auto request_lds = [&](int le_) {
+            typedef const __attribute__((address_space(1))) void* GlobalPtr;
+            typedef __attribute__((address_space(3))) void* LdsPtr;
+            const int row = __builtin_amdgcn_readfirstlane(rows[le_]);
+            const char* rowp = reinterpret_cast<const char*>(a.tabK + ((size_t)row * P * K + k0) * 4);
+#pragma unroll
+            for (int q = 0; q < PRE; ++q) {
+                const char* src = rowp + (size_t)q * K * 4 * sizeof(F);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)src, (LdsPtr)(pre + (q * 2) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((GlobalPtr)(src + 16), (LdsPtr)(pre + (q * 2 + 1) * 1024), 16, 0, 0);
+            }
+            const int grow = __builtin_amdgcn_readfirstlane(grows[le_]);
+            const F* Hp = a.Hsrc + (size_t)grow * NLM * K + k0;
+#pragma unroll
+            for (int q = 0; q < NLM; ++q) Hn[q] = ldv<F, CPL>(Hp + q * K);
+        };
+        if constexpr (WL::PREFETCH) {
+            if (nE > 0) { request_lds(0); request(0, std::integral_constant<int, PRE>{}, std::integral_constant<int, P>{}, false); }
+        }
         for (int le = 0; le < nE; ++le) {
             const F x = (F)xs[le];
             const F* B = Bs + le * NBP;
@@ -290,6 +318,28 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
             // again): a conditional request makes the values carried round the loop a merge of old and new registers,
             // which costs a register copy per value
             const int le_next = le + 1 < nE ? le + 1 : le;
+            if constexpr (WL::PREFETCH) {
+                constexpr std::integral_constant<int, PRE> cPre{};
+                // first paths from the buffer (filled while the previous edge was worked on), sender row likewise
+#pragma unroll
+                for (int q = 0; q < NLM; ++q) H[q] = Hn[q];
+#pragma unroll
+                for (int q = 0; q < PRE; ++q) {
+                    const Vec<F, 2> lo = *reinterpret_cast<const Vec<F, 2>*>(pre + (q * 2) * 1024 + lane * 16);
+                    const Vec<F, 2> hi = *reinterpret_cast<const Vec<F, 2>*>(pre + (q * 2 + 1) * 1024 + lane * 16);
+                    cf[q][0].v[0] = lo.v[0]; cf[q][0].v[1] = lo.v[1]; cf[q][0].v[2] = hi.v[0]; cf[q][0].v[3] = hi.v[1];
+                }
+                products(x, c0, cPre);
+                static_for<0, PRE>(accumulate);
+                products(x, cPre, cP);                    // the other paths came through registers, requested an edge ago
+                // the next edge's operands: first paths into the buffer (these requests are the older ones, so the
+                // wait for them at the top of the next edge leaves the register loads in flight), the rest into the
+                // registers the products above have just freed
+                request_lds(le_next);
+                request(le_next, cPre, cP, false);
+                static_for<PRE, P>(accumulate);
+                continue;
+            }
             if (!AHEAD && !HALF) request(le, c0, cP, true);
             if (HALF) request(le, cA, cP, false);
             products(x, c0, cA);
@@ -595,7 +645,7 @@ hipError_t launch_agg_t(const AggParams<F>& p, hipStream_t s)
     const int groups = (p.K + 64 * CPL - 1) / (64 * CPL);
     if (p.K % CPL != 0) return hipErrorInvalidValue;
     if (BWD && groups > 1 && !p.fpart) return hipErrorInvalidValue;
-    const size_t lds = WL::lists(p.num_terms) + 4 * WL::per_wave(EC);
+    const size_t lds = WL::lists(p.num_terms) + 4 * WL::per_wave(EC) + 4 * WL::prefetch_per_wave();
     if (!BWD && (p.node_begin != 0 || p.msg_edge_begin != 0)) return hipErrorInvalidValue;
     if (p.node_begin < 0 || p.node_begin > p.num_nodes) return hipErrorInvalidValue;
     dim3 grid((p.num_nodes - p.node_begin + 3) / 4, groups);
@@ -624,7 +674,9 @@ int agg_cpl(int K)
 template <typename F, int LMAXH, bool BWD>
 hipError_t launch_agg_sel(const AggParams<F>& p, hipStream_t s)
 {
-    constexpr int EC = LMAXH == 0 ? 16 : (BWD ? (sizeof(F) == 4 ? 8 : 4) : 16);
+    // edges per chunk; the double-precision forward kernel of the ten-path list takes eight so that two blocks with
+    // their coefficient buffers fit a CU
+    constexpr int EC = LMAXH == 0 ? 16 : (BWD ? (sizeof(F) == 4 ? 8 : 4) : (sizeof(F) == 8 ? 8 : 16));
     // two channels per lane exist for the four-path list only (the ten-path kernels have no registers for them)
     if constexpr (LMAXH == 0) {
         if (agg_cpl<F, LMAXH, BWD>(p.K) == 2) return launch_agg_t<F, LMAXH, 2, EC, BWD>(p, s);

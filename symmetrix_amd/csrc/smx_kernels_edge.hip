@@ -175,9 +175,14 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
     }
 
     const int K = a.K;
-    const int i = blockIdx.x * 4 + wave;
+    // One-dimensional grid, channel group fastest: consecutive blocks go to the dies in turn, so a die only ever
+    // works on the channel groups congruent to its number and its L2 holds that share of the spline table alone
+    // (half of it at two groups of 64 channels).
+    const int groups = (K + 64 * CPL - 1) / (64 * CPL);
+    const int cgroup = blockIdx.x % groups;
+    const int i = (blockIdx.x / groups) * 4 + wave;
     if (i >= a.num_nodes) return;
-    const int k0 = (blockIdx.y * 64 + lane) * CPL;
+    const int k0 = (cgroup * 64 + lane) * CPL;
     const bool active = k0 < K;
     const int e0 = a.first_neigh[i], e1 = a.first_neigh[i + 1], ti = a.node_types[i];
 
@@ -367,7 +372,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
 // Adjoint: per edge force -dE/dxyz_ij (MACE::reverse_A0, mace.cpp:238-269;
 // MACE::reverse_Phi1, mace.cpp:531-574) and the adjoint message to the sender
 // row (mace.cpp:579-604), staged per edge for the deterministic sender-side sum.
-// With more than one channel group (gridDim.y > 1) each group writes its share
+// With more than one channel group each group writes its share
 // of the force to fpart[group][edge][3]; the caller adds the groups up.
 template <typename F, int LMAXH, int CPL, int EC>
 __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const int num_terms)
@@ -406,15 +411,18 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
     }
 
     const int K = a.K;
-    const int i = a.node_begin + blockIdx.x * 4 + wave;
+    // one-dimensional grid, channel group fastest (see k_agg_fwd)
+    const int groups = (K + 64 * CPL - 1) / (64 * CPL);
+    const int cgroup = blockIdx.x % groups;
+    const int i = a.node_begin + (blockIdx.x / groups) * 4 + wave;
     if (i >= a.num_nodes) return;
     // Lanes beyond the last channel work on channel 0 with a zero adjoint (all their sums are zero) and skip the
     // message store: no branch on the lane's channel inside the edge loop, hence no merges of old and new registers.
-    const bool active = (blockIdx.y * 64 + lane) * CPL < K;
-    const int k0 = active ? (blockIdx.y * 64 + lane) * CPL : 0;
+    const bool active = (cgroup * 64 + lane) * CPL < K;
+    const int k0 = active ? (cgroup * 64 + lane) * CPL : 0;
     const int e0 = a.first_neigh[i], e1 = a.first_neigh[i + 1], ti = a.node_types[i];
-    double* fout = gridDim.y > 1 ? a.fpart + (size_t)blockIdx.y * 3 * a.num_edges : a.forces;
-    const bool add_forces = gridDim.y == 1 && a.accumulate_forces;
+    double* fout = groups > 1 ? a.fpart + (size_t)cgroup * 3 * a.num_edges : a.forces;
+    const bool add_forces = groups == 1 && a.accumulate_forces;
 
     F d[CPL][NE];
 #pragma unroll
@@ -648,8 +656,10 @@ hipError_t launch_agg_t(const AggParams<F>& p, hipStream_t s)
     const size_t lds = WL::lists(p.num_terms) + 4 * WL::per_wave(EC) + 4 * WL::prefetch_per_wave();
     if (!BWD && (p.node_begin != 0 || p.msg_edge_begin != 0)) return hipErrorInvalidValue;
     if (p.node_begin < 0 || p.node_begin > p.num_nodes) return hipErrorInvalidValue;
-    dim3 grid((p.num_nodes - p.node_begin + 3) / 4, groups);
-    if (grid.x == 0) return hipSuccess;
+    const long blocks = (long)((p.num_nodes - p.node_begin + 3) / 4) * groups;
+    if (blocks == 0) return hipSuccess;
+    if (blocks > 0x7fffffffL) return hipErrorInvalidValue;
+    dim3 grid((unsigned)blocks);
     void (*kern)(const AggParams<F>, const int);
     if constexpr (BWD) kern = k_agg_bwd<F, LMAXH, CPL, EC>;
     else kern = k_agg_fwd<F, LMAXH, CPL, EC>;

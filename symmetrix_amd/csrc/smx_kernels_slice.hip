@@ -42,6 +42,21 @@ __device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, si
     __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0): the direct loads have written the LDS
 }
 
+// Which slice and which receiver group a block works on.  Blocks go to the eight dies in turn (block b to die
+// b % 8), and every die has its own L2.  The (slice, receiver group) pairs are numbered slice by slice and each die
+// takes one contiguous eighth of that order, i.e. consecutive slices: the 32-byte pieces its blocks read and write
+// in the rows of the feature arrays (sender rows, adjoint rows, messages, sums) then lie side by side in the same
+// cache lines of the same L2, instead of every die touching a quarter of every line.
+struct BlockSlot { int slice, group; };
+__device__ __forceinline__ BlockSlot block_slot(int slots_per_die, int receiver_groups, int num_slots)
+{
+    const int die = blockIdx.x % 8, j = blockIdx.x / 8;
+    const int t = die * slots_per_die + j;
+    if (j >= slots_per_die || t >= num_slots) return {1 << 28, 0};      // no work: the caller sees a slice past the last
+    return {t / receiver_groups, t % receiver_groups};
+}
+static inline int slots_per_die(int S, int RG) { return (S * RG + 7) / 8; }
+
 // The tasks of a block (groups of receivers, largest first) are handed to its wavefronts as they become free: an
 // integer counter in LDS, so that the wavefronts of a block finish together whatever the degrees.  Which wavefront
 // takes a task has no influence on any result (a task's sums are its own).
@@ -110,7 +125,9 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
     const F* lds = reinterpret_cast<const F*>(smem);
     const AggParams<F>& a = p.a;
     constexpr int CPLN = CH / CL, EPR = 16 / CL;
-    const int slice = blockIdx.x, K = a.K;
+    const BlockSlot slot_of_block = block_slot(p.slots_per_die, p.receiver_groups, p.num_slots);
+    const int slice = slot_of_block.slice, K = a.K;
+    if ((long)slice * CH >= K) return;                      // a block without a slot
     const int W = p.W, R = a.spl_nodes - 1;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int sub = lane & 15, e_sub = sub / CL, cs = sub % CL;
@@ -125,8 +142,8 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
     if (threadIdx.x == 0) task_counter = 0;
     copy_slice_to_lds(p.tabS + (size_t)slice * R * W, smem, (size_t)R * W * sizeof(F));
     __syncthreads();
-    for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
-         task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
+    for (int task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter); task < wave_tasks;
+         task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter)) {
         const int slot = task * 4 + (lane >> 4);
         const bool live = slot < a.num_nodes;
         const int i = live ? p.order[slot] : 0;
@@ -203,7 +220,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     const F* lds = reinterpret_cast<const F*>(smem);
     const AggParams<F>& a = p.a;
     constexpr int CPLN = CH / CL, EPR = 16 / CL;
-    const int slice = blockIdx.x, K = a.K;
+    const BlockSlot slot_of_block = block_slot(p.slots_per_die, p.receiver_groups, p.num_slots);
+    const int slice = slot_of_block.slice, K = a.K;
+    if ((long)slice * CH >= K) return;                      // a block without a slot
     const int W = p.W, R = a.spl_nodes - 1;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int sub = lane & 15, e_sub = sub / CL, cs = sub % CL;
@@ -219,8 +238,8 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     if (threadIdx.x == 0) task_counter = 0;
     copy_slice_to_lds(p.tabS + (size_t)slice * R * W, smem, (size_t)R * W * sizeof(F));
     __syncthreads();
-    for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
-         task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
+    for (int task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter); task < wave_tasks;
+         task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter)) {
         const int slot = task * 4 + (lane >> 4);
         const bool live = slot < a.num_nodes;
         const int i = live ? p.order[slot] : 0;
@@ -345,7 +364,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     using V = Vec<F, CH>;
     const F* lds = reinterpret_cast<const F*>(smem);
     const AggParams<F>& a = p.a;
-    const int slice = blockIdx.x, K = a.K;
+    const BlockSlot slot_of_block = block_slot(p.slots_per_die, p.receiver_groups, p.num_slots);
+    const int slice = slot_of_block.slice, K = a.K;
+    if ((long)slice * CH >= K) return;                      // a block without a slot
     const int W = p.W, R = a.spl_nodes - 1;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     constexpr int ROWS = 64 / RL;                            // receivers a wavefront works on at a time
@@ -362,8 +383,8 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     if (threadIdx.x == 0) task_counter = 0;
     copy_slice_to_lds(p.tabS + (size_t)slice * R * W, smem, (size_t)R * W * sizeof(F));
     __syncthreads();
-    for (int task = blockIdx.y + gridDim.y * next_block_task(&task_counter); task < wave_tasks;
-         task = blockIdx.y + gridDim.y * next_block_task(&task_counter)) {
+    for (int task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter); task < wave_tasks;
+         task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter)) {
         const int slot = task * ROWS + row;
         const bool live = slot < a.num_nodes;
         const int i = live ? p.order[slot] : 0;
@@ -511,7 +532,11 @@ hipError_t launch_slice_cfg(const SliceParams<F>& p, hipStream_t s)
     if (RG < 1) RG = 1;
     const long tasks_per_slice = ((long)p.a.num_nodes + 3) / 4;
     if ((long)RG * waves_per_block > tasks_per_slice) RG = (int)((tasks_per_slice + waves_per_block - 1) / waves_per_block);
-    dim3 grid(S, RG);
+    SliceParams<F> q = p;
+    q.slots_per_die = slots_per_die(S, RG);
+    q.receiver_groups = RG;
+    q.num_slots = S * RG;
+    dim3 grid(8u * (unsigned)q.slots_per_die);
     void (*kern)(const SliceParams<F>) = nullptr;
     if constexpr (BWD) kern = k_slice_bwd<F, CH, CL, BT>;
     else kern = k_slice_fwd<F, CH, CL, BT>;
@@ -519,7 +544,7 @@ hipError_t launch_slice_cfg(const SliceParams<F>& p, hipStream_t s)
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(kern, grid, dim3(BT), lds, s, p);
+    hipLaunchKernelGGL(kern, grid, dim3(BT), lds, s, q);
     return hipGetLastError();
 }
 
@@ -565,7 +590,11 @@ static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
     }
-    hipLaunchKernelGGL(kern, dim3(S, RG), dim3(BT), lds, s, p);
+    SliceParams<F> q = p;
+    q.slots_per_die = slots_per_die(S, RG);
+    q.receiver_groups = RG;
+    q.num_slots = S * RG;
+    hipLaunchKernelGGL(kern, dim3(8u * (unsigned)q.slots_per_die), dim3(BT), lds, s, q);
     return hipGetLastError();
 }
 // Twelve wavefronts per block and sixteen lanes per receiver measured best (eight lanes per receiver fill the

@@ -73,7 +73,7 @@ struct SliceParams {
     long E;
     int num_cus;
     const int* order;     // [num_nodes] receivers by decreasing degree: entry 4t+q is row q of task t
-    int slots_per_die, receiver_groups, num_slots;   // set by the launchers: block -> (slice, receiver group)
+    int units_per_die, slot_lines, num_units, receiver_groups;   // set by the launchers: block -> (slice, receiver group)
     long fpart_carry;     // bwd, one lane per edge: edges [0, fpart_carry) add what fpart already holds (an earlier stage's partial forces)
     int edge_lanes;       // bwd: one lane per edge (tabS rows padded to slice_edge_row_elements, CH * sizeof(F) = 32)
 };

@@ -43,19 +43,31 @@ __device__ __forceinline__ void copy_slice_to_lds(const void* src, void* dst, si
 }
 
 // Which slice and which receiver group a block works on.  Blocks go to the eight dies in turn (block b to die
-// b % 8), and every die has its own L2.  The (slice, receiver group) pairs are numbered slice by slice and each die
-// takes one contiguous eighth of that order, i.e. consecutive slices: the 32-byte pieces its blocks read and write
-// in the rows of the feature arrays (sender rows, adjoint rows, messages, sums) then lie side by side in the same
-// cache lines of the same L2, instead of every die touching a quarter of every line.
+// b % 8), and every die has its own L2.  A slice's share of a feature row is 32 bytes, so four consecutive slices
+// share a 128-byte cache line.  The unit that must stay on one die is therefore (line of four slices, receiver
+// group): its four blocks read and write whole lines of the rows of their receivers (adjoint rows, messages, sums)
+// in one L2, where the partial writes merge.  Units are numbered receiver group first, then line, and each die
+// takes a contiguous eighth of them: a die's blocks mostly share their receivers, hence the edge arrays they read.
 struct BlockSlot { int slice, group; };
-__device__ __forceinline__ BlockSlot block_slot(int slots_per_die, int receiver_groups, int num_slots)
+__device__ __forceinline__ BlockSlot block_slot(int units_per_die, int lines, int num_units)
 {
     const int die = blockIdx.x % 8, j = blockIdx.x / 8;
-    const int t = die * slots_per_die + j;
-    if (j >= slots_per_die || t >= num_slots) return {1 << 28, 0};      // no work: the caller sees a slice past the last
-    return {t / receiver_groups, t % receiver_groups};
+    const int unit = die * units_per_die + j / 4;
+    if (j >= 4 * units_per_die || unit >= num_units) return {1 << 28, 0};   // no work: a slice past the last
+    return {4 * (unit % lines) + j % 4, unit / lines};
 }
-static inline int slots_per_die(int S, int RG) { return (S * RG + 7) / 8; }
+// receiver groups of a launch over S slices on num_cus CUs: one block per CU, and no die with more than its 32
+template <typename P>
+static inline void place_blocks(P& q, int S, int& RG, unsigned& blocks)
+{
+    const int lines = (S + 3) / 4;
+    if (RG * lines > 64) RG = 64 / lines > 0 ? 64 / lines : 1;
+    q.slot_lines = lines;
+    q.num_units = lines * RG;
+    q.units_per_die = (q.num_units + 7) / 8;
+    q.receiver_groups = RG;
+    blocks = 8u * 4u * (unsigned)q.units_per_die;
+}
 
 // The tasks of a block (groups of receivers, largest first) are handed to its wavefronts as they become free: an
 // integer counter in LDS, so that the wavefronts of a block finish together whatever the degrees.  Which wavefront
@@ -125,7 +137,7 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
     const F* lds = reinterpret_cast<const F*>(smem);
     const AggParams<F>& a = p.a;
     constexpr int CPLN = CH / CL, EPR = 16 / CL;
-    const BlockSlot slot_of_block = block_slot(p.slots_per_die, p.receiver_groups, p.num_slots);
+    const BlockSlot slot_of_block = block_slot(p.units_per_die, p.slot_lines, p.num_units);
     const int slice = slot_of_block.slice, K = a.K;
     if ((long)slice * CH >= K) return;                      // a block without a slot
     const int W = p.W, R = a.spl_nodes - 1;
@@ -220,7 +232,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
     const F* lds = reinterpret_cast<const F*>(smem);
     const AggParams<F>& a = p.a;
     constexpr int CPLN = CH / CL, EPR = 16 / CL;
-    const BlockSlot slot_of_block = block_slot(p.slots_per_die, p.receiver_groups, p.num_slots);
+    const BlockSlot slot_of_block = block_slot(p.units_per_die, p.slot_lines, p.num_units);
     const int slice = slot_of_block.slice, K = a.K;
     if ((long)slice * CH >= K) return;                      // a block without a slot
     const int W = p.W, R = a.spl_nodes - 1;
@@ -364,7 +376,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     using V = Vec<F, CH>;
     const F* lds = reinterpret_cast<const F*>(smem);
     const AggParams<F>& a = p.a;
-    const BlockSlot slot_of_block = block_slot(p.slots_per_die, p.receiver_groups, p.num_slots);
+    const BlockSlot slot_of_block = block_slot(p.units_per_die, p.slot_lines, p.num_units);
     const int slice = slot_of_block.slice, K = a.K;
     if ((long)slice * CH >= K) return;                      // a block without a slot
     const int W = p.W, R = a.spl_nodes - 1;
@@ -533,10 +545,9 @@ hipError_t launch_slice_cfg(const SliceParams<F>& p, hipStream_t s)
     const long tasks_per_slice = ((long)p.a.num_nodes + 3) / 4;
     if ((long)RG * waves_per_block > tasks_per_slice) RG = (int)((tasks_per_slice + waves_per_block - 1) / waves_per_block);
     SliceParams<F> q = p;
-    q.slots_per_die = slots_per_die(S, RG);
-    q.receiver_groups = RG;
-    q.num_slots = S * RG;
-    dim3 grid(8u * (unsigned)q.slots_per_die);
+    unsigned blocks = 0;
+    place_blocks(q, S, RG, blocks);
+    dim3 grid(blocks);
     void (*kern)(const SliceParams<F>) = nullptr;
     if constexpr (BWD) kern = k_slice_bwd<F, CH, CL, BT>;
     else kern = k_slice_fwd<F, CH, CL, BT>;
@@ -591,10 +602,9 @@ static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t
         if (err != hipSuccess) return err;
     }
     SliceParams<F> q = p;
-    q.slots_per_die = slots_per_die(S, RG);
-    q.receiver_groups = RG;
-    q.num_slots = S * RG;
-    hipLaunchKernelGGL(kern, dim3(8u * (unsigned)q.slots_per_die), dim3(BT), lds, s, q);
+    unsigned blocks = 0;
+    place_blocks(q, S, RG, blocks);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(BT), lds, s, q);
     return hipGetLastError();
 }
 // Twelve wavefronts per block and sixteen lanes per receiver measured best (eight lanes per receiver fill the

@@ -56,12 +56,14 @@ __device__ __forceinline__ BlockSlot block_slot(int units_per_die, int lines, in
     if (j >= 4 * units_per_die || unit >= num_units) return {1 << 28, 0};   // no work: a slice past the last
     return {4 * (unit % lines) + j % 4, unit / lines};
 }
-// receiver groups of a launch over S slices on num_cus CUs: one block per CU, and no die with more than its 32
+// receiver groups of a launch over S slices: one block per CU, and no die with more blocks than it has CUs (an eighth
+// of them; four blocks per unit)
 template <typename P>
 static inline void place_blocks(P& q, int S, int& RG, unsigned& blocks)
 {
     const int lines = (S + 3) / 4;
-    if (RG * lines > 64) RG = 64 / lines > 0 ? 64 / lines : 1;
+    const int max_units = q.num_cus / 4 > 0 ? q.num_cus / 4 : 1;
+    if (RG * lines > max_units) RG = max_units / lines > 0 ? max_units / lines : 1;
     q.slot_lines = lines;
     q.num_units = lines * RG;
     q.units_per_die = (q.num_units + 7) / 8;

@@ -35,7 +35,7 @@ HBM_PEAK = 8.0e12  # bytes/s, MI355X HBM3E
 
 # kernel behind each edge stage: channel-slice kernels (scalar hidden features and one radial table for all
 # species pairs) / general kernels
-SLICE_KERNEL = {"agg0_fwd": "k_slice_fwd", "agg1_fwd": "k_slice_fwd", "agg1_bwd": "k_slice_bwd_edge",
+SLICE_KERNEL = {"agg0_fwd": "k_slice_fwd_halves", "agg1_fwd": "k_slice_fwd_halves", "agg1_bwd": "k_slice_bwd_edge",
                 "agg0_bwd": "k_slice_bwd_edge", "sender_reduce": "k_sender_reduce_linear"}
 GENERAL_KERNEL = {"agg0_fwd": "k_agg_fwd", "agg1_fwd": "k_agg_fwd", "agg1_bwd": "k_agg_bwd", "agg0_bwd": "k_agg_bwd",
                   "sender_reduce": "k_sender_reduce"}

@@ -170,6 +170,7 @@ struct Engine : EngineBase {
     // the same slices with the row padding of the adjoint kernel that gives every edge a lane of its own
     // (empty when the forward table already has that row length, or when the kernel does not apply)
     DVec<F> tabE0, tabE1;
+    DVec<F> tabF0, tabF1;   // forward-kernel layout of the same slices (when a slice is 32 bytes of channels)
     bool edge_lanes = false;
     double cdiag1[16] = {};
     DVec<double> fpart;
@@ -366,7 +367,8 @@ struct Engine : EngineBase {
     }
 
     // Regroup a radial table per channel slice, or return 0 when the slice path does not apply.
-    int build_slice_table(const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst, DVec<F>& edst, hipStream_t s)
+    int build_slice_table(const std::vector<std::vector<double>>& tables, int nspl, DVec<F>& dst, DVec<F>& edst, DVec<F>& fdst,
+                          hipStream_t s)
     {
         // One radial table only (species-independent radial functions, as models without a distance transform
         // have).  A slice kernel holds one table at a time: with several, every table is a pass over all edges of
@@ -413,6 +415,24 @@ struct Engine : EngineBase {
                     std::copy(buf.begin() + rowi * W, buf.begin() + rowi * W + 16 * CH, eb.begin() + rowi * We);
                 edst.upload(eb.data(), eb.size(), s);
                 HIPCHK(hipStreamSynchronize(s));
+                // forward kernel of such slices: per row [4 paths][2 halves][4 lanes][channels of the lane][2], the pair
+                // being coefficients (2 half, 2 half + 1)
+                const int cpln = CH / 4, Wf = 512 / (int)sizeof(F);
+                std::vector<F> fb((size_t)S * R * Wf, F(0));
+                for (int sl = 0; sl < S; ++sl)
+                    for (int n = 0; n < R; ++n)
+                        for (int pth = 0; pth < 4; ++pth)
+                            for (int hf = 0; hf < 2; ++hf)
+                                for (int ln = 0; ln < 4; ++ln)
+                                    for (int c = 0; c < cpln; ++c)
+                                        for (int j = 0; j < 2; ++j) {
+                                            const int k = sl * CH + ln * cpln + c;
+                                            if (k < Kc)
+                                                fb[((size_t)sl * R + n) * Wf + ((((pth * 2 + hf) * 4 + ln) * cpln + c) * 2 + j)] =
+                                                    (F)tables[0][((size_t)n * 4 + 2 * hf + j) * nspl + pth * Kc + k];
+                                        }
+                fdst.upload(fb.data(), fb.size(), s);
+                HIPCHK(hipStreamSynchronize(s));
             }
             return CH;
         }
@@ -420,7 +440,7 @@ struct Engine : EngineBase {
     }
     void build_slices(hipStream_t s)
     {
-        slice_CH0 = build_slice_table(hm.tables0, hm.nspl0, tabS0, tabE0, s);
+        slice_CH0 = build_slice_table(hm.tables0, hm.nspl0, tabS0, tabE0, tabF0, s);
         if (hm.L_max == 0) {
             // layer 1 qualifies when every output slot lm is fed by harmonic lm alone
             bool diag = hm.num_B == 16;
@@ -432,7 +452,7 @@ struct Engine : EngineBase {
                 }
             }
             if (diag) {
-                slice_CH1 = build_slice_table(hm.tables1, hm.nspl1, tabS1, tabE1, s);
+                slice_CH1 = build_slice_table(hm.tables1, hm.nspl1, tabS1, tabE1, tabF1, s);
             }
         }
     }
@@ -442,6 +462,7 @@ struct Engine : EngineBase {
         p.a = agg_params(layer, N);
         p.tabS = layer == 0 ? tabS0.p : tabS1.p;
         p.W = slice_W;
+        if (!adjoint && edge_lanes) p.tabF = layer == 0 ? tabF0.p : tabF1.p;
         if (adjoint && edge_lanes) {
             p.edge_lanes = 1;
             DVec<F>& te = layer == 0 ? tabE0 : tabE1;

@@ -66,6 +66,7 @@ template <typename F>
 struct SliceParams {
     AggParams<F> a;
     const F* tabS;
+    const F* tabF;     // forward kernel of 32-byte slices: rows [4 paths][2 halves][4 lanes][16 bytes], or null
     int W;             // padded row length in elements
     int CH;            // channels per slice
     double cdiag[16];

@@ -227,6 +227,117 @@ __global__ __launch_bounds__(BT) void k_slice_fwd(const SliceParams<F> p)
 }
 
 // ---------------------------------------------------------------------------
+// Forward kernel for slices of 32 bytes of channels (four lanes per edge, CH / 4 channels each) with a table layout
+// made for the LDS banks.  A row is [4 paths][2 halves][4 lanes][16 bytes]: the 16 bytes hold, for the lane's
+// channels, the coefficient pair (c0, c1) in half 0 and (c2, c3) in half 1, so that the four lanes of an edge read 64
+// contiguous bytes per instruction.  Rows are 512 bytes, so every edge's 64 bytes would fall on the same half of the
+// banks; edges in odd slots therefore read the halves in the opposite order, an even and an odd edge fill one 128-byte
+// bank row per cycle, and no read conflicts with another whatever the rows.  The cubic is evaluated as
+// (c0 + c1 x) + x^2 (c2 + c3 x): the two brackets are formed from whichever half arrived first and second, and
+// the lane's factors (1, x^2) or (x^2, 1), already multiplied with the sender feature, put them together.
+template <typename F, int BT>
+__global__ __launch_bounds__(BT) void k_slice_fwd_halves(const SliceParams<F> p)
+{
+    constexpr int CH = 32 / (int)sizeof(F), CL = 4, CPLN = CH / CL, EPR = 16 / CL;
+    using V = Vec<F, 2 * CPLN>;                            // 16 bytes
+    extern __shared__ __align__(16) unsigned char smem[];
+    const F* lds = reinterpret_cast<const F*>(smem);
+    const AggParams<F>& a = p.a;
+    const BlockSlot slot_of_block = block_slot(p.units_per_die, p.slot_lines, p.num_units);
+    const int slice = slot_of_block.slice, K = a.K;
+    if ((long)slice * CH >= K) return;                      // a block without a slot
+    constexpr int WF = 512 / (int)sizeof(F);               // row length in elements
+    const int R = a.spl_nodes - 1;
+    const int lane = threadIdx.x & 63;
+    const int sub = lane & 15, e_sub = sub / CL, cs = sub % CL;
+    const int kc = slice * CH + cs * CPLN;                 // first channel of this lane
+    const int par = e_sub & 1;
+    const int off_first = (par * 4 + cs) * 2 * CPLN, off_second = ((par ^ 1) * 4 + cs) * 2 * CPLN;
+    const int wave_tasks = (a.num_nodes + 3) / 4;
+    __shared__ int task_counter;
+
+    if (threadIdx.x == 0) task_counter = 0;
+    copy_slice_to_lds(p.tabF + (size_t)slice * R * WF, smem, (size_t)R * 512);
+    __syncthreads();
+    for (int task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter); task < wave_tasks;
+         task = slot_of_block.group + p.receiver_groups * next_block_task(&task_counter)) {
+        const int slot = task * 4 + (lane >> 4);
+        const bool live = slot < a.num_nodes;
+        const int i = live ? p.order[slot] : 0;
+        int e0 = 0, e1 = 0;
+        if (live) { e0 = a.first_neigh[i]; e1 = a.first_neigh[i + 1]; }
+        F acc[16][CPLN];
+#pragma unroll
+        for (int q = 0; q < 16; ++q)
+#pragma unroll
+            for (int c = 0; c < CPLN; ++c) acc[q][c] = F(0);
+        // the geometry of the next edge of this lane is loaded while the current one is processed
+        EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0};
+        {
+            const int ef = e0 + e_sub;
+            if (ef < e1) nx = load_edge(a, ef);
+        }
+        for (int e = e0 + e_sub; e < e1; e += EPR) {
+            const EdgeGeo cu = nx;
+            nx = load_edge(a, min(e + EPR, e1 - 1));   // unconditional: a conditional load costs a register copy per value
+            const int g = cu.g;
+            const double dx = cu.dx, dy = cu.dy, dz = cu.dz;
+            const double r = cu.r;
+            const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
+            double Yd[16];
+            sph_l3(dz * inv, dx * inv, dy * inv, Yd);
+            const int n = spline_interval(r, a.spl_inv_h, R - 1);
+            const F x = (F)(r - a.spl_h * n);
+            const F x2 = x * x;
+            const F* row = lds + (size_t)n * WF;
+            F s_first[CPLN], s_second[CPLN];
+#pragma unroll
+            for (int c = 0; c < CPLN; ++c) {
+                const F h = a.Hsrc[(size_t)g * K + min(kc + c, K - 1)];
+                const F hx = h * x2;
+                s_first[c] = par ? hx : h;
+                s_second[c] = par ? h : hx;
+            }
+            F t[CPLN][4];
+#pragma unroll
+            for (int l = 0; l < 4; ++l) {
+                const V first = *reinterpret_cast<const V*>(row + l * 16 * CPLN + off_first);
+                const V second = *reinterpret_cast<const V*>(row + l * 16 * CPLN + off_second);
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c) {
+                    const F u = first.v[2 * c] + first.v[2 * c + 1] * x;
+                    const F v = second.v[2 * c] + second.v[2 * c + 1] * x;
+                    t[c][l] = u * s_first[c] + v * s_second[c];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const F y = (F)Yd[q];
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c) acc[q][c] += t[c][lm_l(q)] * y;
+            }
+        }
+        // add up the lanes of the row that hold the same channels (they took alternate edges)
+#pragma unroll
+        for (int q = 0; q < 16; ++q)
+#pragma unroll
+            for (int c = 0; c < CPLN; ++c) acc[q][c] = row_sum_strided<CL>(acc[q][c]);
+        if (live && e_sub == 0) {
+#pragma unroll
+            for (int q = 0; q < 16; ++q) {
+                const F cd = (F)p.cdiag[q];
+#pragma unroll
+                for (int c = 0; c < CPLN; ++c)
+                    if (kc + c < K) {
+                        F* o = a.out + ((size_t)i * 16 + q) * K + kc + c;
+                        *o = acc[q][c] * cd;
+                    }
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------
 template <typename F, int CH, int CL, int BT>
 __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
 {
@@ -574,10 +685,33 @@ hipError_t launch_slice_t(const SliceParams<F>& p, hipStream_t s)
 
 }  // namespace
 
+template <typename F, int BT>
+static hipError_t launch_slice_fwd_halves(const SliceParams<F>& p, hipStream_t s)
+{
+    constexpr int CH = 32 / (int)sizeof(F);
+    const int S = (p.a.K + CH - 1) / CH;
+    const size_t lds = (size_t)(p.a.spl_nodes - 1) * 512;
+    int RG = p.num_cus / S;
+    if (RG < 1) RG = 1;
+    const long tasks_per_slice = ((long)p.a.num_nodes + 3) / 4;
+    if ((long)RG * (BT / 64) > tasks_per_slice) RG = (int)((tasks_per_slice + BT / 64 - 1) / (BT / 64));
+    auto kern = k_slice_fwd_halves<F, BT>;
+    if (lds > 64 * 1024) {
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (err != hipSuccess) return err;
+    }
+    SliceParams<F> q = p;
+    unsigned blocks = 0;
+    place_blocks(q, S, RG, blocks);
+    hipLaunchKernelGGL(kern, dim3(blocks), dim3(BT), lds, s, q);
+    return hipGetLastError();
+}
+
 template <typename F>
 hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s)
 {
     if (p.a.num_nodes <= 0) return hipSuccess;
+    if (p.tabF) return launch_slice_fwd_halves<F, 1024>(p, s);
     switch (p.CH) {
     case 2: return launch_slice_t<F, 2, false>(p, s);
     case 4: return launch_slice_t<F, 4, false>(p, s);

@@ -86,8 +86,8 @@ def test_pipeline_matches_oracle(gpu, tmp_models, K, L_max, natoms, pair, dtype)
 @pytest.mark.parametrize("dtype", ["float64", "float32"])
 @pytest.mark.parametrize("K,natoms", [(20, 70), (96, 200), (33, 9)])
 def test_two_species_three_radial_tables(gpu, tmp_models, K, natoms, dtype):
-    """Scalar hidden features with a few distinct pair tables: the channel-slice
-    kernels make one pass over the edges per table."""
+    """Scalar hidden features with a few distinct pair tables: the general edge kernels
+    (the channel-slice kernels hold one table)."""
     model = H.tiny_model(K=K, L_max=0, T=(1, 8), n_pts=50, seed=K, pair=True)
     path = H.write_model(model, tmp_models / f"two_{K}.json")
     orc = _oracle()(model)
@@ -98,6 +98,26 @@ def test_two_species_three_radial_tables(gpu, tmp_models, K, natoms, dtype):
     orc.compute_node_energies_forces(*H.call_args(ea))
     eng.compute_node_energies_forces(*H.call_args(ea))
     _compare(orc, eng, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("K,natoms", [(24, 60), (7, 33)])
+def test_long_spline_tables_take_the_narrow_slice_kernels(gpu, tmp_models, K, natoms, dtype):
+    """One radial table with 400 nodes: a slice of 32 bytes of channels no longer fits the LDS, so the slices
+    are half as wide and the four-lanes-per-edge kernels of both directions run instead of the 32-byte ones."""
+    model = H.tiny_model(K=K, L_max=0, n_pts=400, seed=K, pair=False)
+    path = H.write_model(model, tmp_models / f"long_{K}.json")
+    orc = _oracle()(model)
+    eng = gpu(path, dtype)
+    pos, cell, sp = H.small_system(natoms, seed=natoms)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K={K} atoms={natoms} edges={len(ea['r'])} {dtype} 400 spline nodes", flush=True)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    _compare(orc, eng, dtype)
+    f1, e1 = eng.node_forces, eng.node_energies
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    assert np.array_equal(f1, eng.node_forces) and np.array_equal(e1, eng.node_energies)
 
 
 @pytest.mark.parametrize("dtype", ["float64", "float32"])

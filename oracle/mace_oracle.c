@@ -33,6 +33,18 @@
  *                         of each stage vs central differences; total energy
  *                         vs per-edge finite differences; rotation,
  *                         translation and permutation invariance of E.
+ *   compute_* index conventions (which finite differences and invariances
+ *                         cannot see): tests/test_oracle_stage_pins.py --
+ *                         pair-table index, radial function index, sender
+ *                         species of H0_weights, row-major [kp][k] weights of
+ *                         A0 / H1 / A1 (rows e K + kp), transposed H2 weights,
+ *                         readout layouts, (species, LM, k) of the M0 / M1
+ *                         polynomials and their gradient slots, the sender-row
+ *                         gather of Phi1, and the forward chain in numpy.
+ *   orc_zbl_*, *_scaled   the two known answers of symmetrix/test/test_zbl.py
+ *                         through the reference object code; special cases
+ *                         fixed by the mathematics (tests/test_oracle_pipeline.py).
+ * No function here is left without such a pin.
  */
 #include <math.h>
 #include <stdlib.h>

@@ -95,6 +95,14 @@ __device__ __forceinline__ EdgeGeo load_edge(const AggParams<F>& a, int e)
     return q;
 }
 
+// cu <- nx with moves the compiler cannot postpone: where this stands, the wait for nx stands
+__device__ __forceinline__ void take_edge(EdgeGeo& cu, const EdgeGeo& nx)
+{
+    asm volatile("v_mov_b64 %0, %4\n\tv_mov_b64 %1, %5\n\tv_mov_b64 %2, %6\n\tv_mov_b64 %3, %7"
+                 : "=&v"(cu.dx), "=&v"(cu.dy), "=&v"(cu.dz), "=&v"(cu.r) : "v"(nx.dx), "v"(nx.dy), "v"(nx.dz), "v"(nx.r));
+    asm volatile("v_mov_b32 %0, %1" : "=v"(cu.g) : "v"(nx.g));
+}
+
 // Scheduling fences without instructions: what is computed from vx, vy, vz after order_l cannot start
 // before the five sums are final; pin_value ends the live range of an accumulation's operands here.
 template <typename F>
@@ -481,7 +489,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd(const SliceParams<F> p)
 // rows d[16][CH] (times the coupling constant) are staged per wavefront in the LDS left free by the table slice
 // and read back as broadcasts, one harmonic at a time.  tabS rows here are [4 coefficients][4 paths][CH] padded to
 // W elements with W * sizeof(F) = 16 (mod 32), so that the rows of 16 edges spread over the banks.
-template <typename F, int CH, int BT, int RL>
+template <typename F, int CH, int BT, int RL, bool MSG, bool CARRY, bool WHOLE>
 __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
 {
     static_assert(CH * sizeof(F) == 32, "a lane moves its channels as two 16-byte words");
@@ -497,7 +505,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     constexpr int ROWS = 64 / RL;                            // receivers a wavefront works on at a time
     const int row = lane / RL, sub = lane % RL;
     const int kc = slice * CH;
-    const bool whole = kc + CH <= K;                        // all channels of the slice exist
+    const bool whole = WHOLE || kc + CH <= K;               // all channels of the slice exist (WHOLE: of every slice)
     // staged adjoint rows of the wavefront's receivers, [harmonic][receiver][CH]: the receivers' reads of one
     // harmonic (same instruction, one 32-byte piece each) cover contiguous memory
     F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + ((size_t)wave * 16 * ROWS + row) * CH;
@@ -537,27 +545,41 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
         }
         wave_lds_sync();
         const int iters = (e1 - e0 + RL - 1) / RL;
-        EdgeGeo nx = {1.0, 0.0, 0.0, 1.0, 0};
-        if (e0 + sub < e1) nx = load_edge(a, e0 + sub);
+        auto sender_row = [&](int g) {
+            V h;
+            const F* src = a.Hsrc + (size_t)g * K + kc;
+            if (whole) h = *reinterpret_cast<const V*>(src);
+            else {
+#pragma unroll
+                for (int c = 0; c < CH; ++c) h.v[c] = src[min(c, K - 1 - kc)];
+            }
+            return h;
+        };
+        // Loads and stores share one in-order counter: a wait for a load that was requested after a store also waits
+        // for the store to be acknowledged.  So everything the next iteration needs early is requested before this
+        // iteration's stores: the next edge one iteration ahead (nx, copied into cu before the stores), the sender's
+        // row and the partial forces an earlier stage left for the edge right before the stores, into the
+        // registers the finished edge has just given up.
+        EdgeGeo cu = {1.0, 0.0, 0.0, 1.0, 0}, nx = cu;
+        V h;
+#pragma unroll
+        for (int c = 0; c < CH; ++c) h.v[c] = F(0);
+        double f0 = 0.0, f1 = 0.0, f2 = 0.0;
+        if (e0 + sub < e1) {
+            const int ef = e0 + sub;
+            cu = load_edge(a, ef);
+            if constexpr (CARRY) { f0 = fpart[3 * (size_t)ef]; f1 = fpart[3 * (size_t)ef + 1]; f2 = fpart[3 * (size_t)ef + 2]; }
+            h = sender_row(cu.g);
+        }
+        // nothing outstanding on entry: the waits inside the loop are then counted along the loop alone (merged with a
+        // way in that has loads in flight and no stores, they would assume fewer operations behind a load than the loop
+        // has, and wait for its stores)
+        __builtin_amdgcn_s_waitcnt(0x0F70);   // vmcnt(0)
         for (int it = 0; it < iters; ++it) {
             const int e = e0 + it * RL + sub;
-            bool on = e < e1;
-            const EdgeGeo cu = nx;
-            nx = load_edge(a, min(e + RL, e1 - 1));   // unconditional: a conditional load costs a register copy per value
-            if (!on) continue;
-            // sender row first: its latency hides behind the radial part
-            V h;
-            {
-                const F* src = a.Hsrc + (size_t)cu.g * K + kc;
-                if (whole) h = *reinterpret_cast<const V*>(src);
-                else {
-#pragma unroll
-                    for (int c = 0; c < CH; ++c) h.v[c] = src[min(c, K - 1 - kc)];
-                }
-            }
-            // partial forces an earlier stage left for this edge: requested now, added at the end
-            double f0 = 0.0, f1 = 0.0, f2 = 0.0;
-            if (e < p.fpart_carry) { f0 = fpart[3 * (size_t)e]; f1 = fpart[3 * (size_t)e + 1]; f2 = fpart[3 * (size_t)e + 2]; }
+            const int en = min(e + RL, e1 - 1);
+            nx = load_edge(a, en);   // unconditional: a conditional load costs a register copy per value
+            if (e >= e1) continue;
             const double dx = cu.dx, dy = cu.dy, dz = cu.dz, r = cu.r;
             const double inv = rsqrt_pos(dx * dx + dy * dy + dz * dz);
             const double ux = dz * inv, uy = dx * inv, uz = dy * inv;   // permuted unit vector
@@ -612,7 +634,19 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
 #pragma unroll
                 for (int c = 0; c < CH; ++c) pin_value(mg[c]);
             });
-            if (a.msg) {
+            // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
+            // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
+            const double sr = (double)srad, lt = (double)lterm;
+            const double ir = rcp_pos(r);
+            const bool carried = CARRY && e < p.fpart_carry;    // edges past fpart_carry hold nothing yet (read, not used)
+            const double res0 = (carried ? f0 : 0.0) - (dx * ir * sr + ((double)wy - uy * lt) * inv);   // original x is permuted axis 1
+            const double res1 = (carried ? f1 : 0.0) - (dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
+            const double res2 = (carried ? f2 : 0.0) - (dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
+            // the next edge (this very edge again after the last one: not used), then the stores
+            take_edge(cu, nx);
+            h = sender_row(cu.g);
+            if constexpr (CARRY) { f0 = fpart[3 * (size_t)en]; f1 = fpart[3 * (size_t)en + 1]; f2 = fpart[3 * (size_t)en + 2]; }
+            if constexpr (MSG) {
                 F* dstm = a.msg + (size_t)e * K + kc;
                 if (whole) {
                     V m;
@@ -624,13 +658,7 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
                     for (int c = 0; c < CH; ++c) if (kc + c < K) dstm[c] = mg[c];
                 }
             }
-            // gradient with respect to the edge vector: (w - u (l-weighted sum)) / |v|, axes unpermuted;
-            // radial part along xyz / r with the caller's r (mace.cpp:256-264, 558-566)
-            const double sr = (double)srad, lt = (double)lterm;
-            const double ir = rcp_pos(r);
-            fpart[3 * (size_t)e] = f0 - (dx * ir * sr + ((double)wy - uy * lt) * inv);       // original x is permuted axis 1
-            fpart[3 * (size_t)e + 1] = f1 - (dy * ir * sr + ((double)wz - uz * lt) * inv);   // original y is permuted axis 2
-            fpart[3 * (size_t)e + 2] = f2 - (dz * ir * sr + ((double)wx - ux * lt) * inv);   // original z is permuted axis 0
+            fpart[3 * (size_t)e] = res0; fpart[3 * (size_t)e + 1] = res1; fpart[3 * (size_t)e + 2] = res2;
         }
     }
 }
@@ -722,7 +750,7 @@ hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s)
 // threads per block of the lane-per-edge adjoint kernel: three wavefronts per SIMD, 168 registers each (four per
 // SIMD, which the LDS has room for, spill in double precision and gain nothing measurable in single)
 template <typename F> constexpr int kEdgeBlock = 768;
-template <typename F, int BT, int RL>
+template <typename F, int BT, int RL, bool MSG, bool CARRY, bool WHOLE>
 static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t s)
 {
     constexpr int CH = 32 / (int)sizeof(F), ROWS = 64 / RL;
@@ -732,7 +760,7 @@ static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t
     if (RG < 1) RG = 1;
     const long tasks_per_slice = ((long)p.a.num_nodes + ROWS - 1) / ROWS;
     if ((long)RG * (BT / 64) > tasks_per_slice) RG = (int)((tasks_per_slice + BT / 64 - 1) / (BT / 64));
-    auto kern = k_slice_bwd_edge<F, CH, BT, RL>;
+    auto kern = k_slice_bwd_edge<F, CH, BT, RL, MSG, CARRY, WHOLE>;
     if (lds > 64 * 1024) {
         hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(kern), hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
         if (err != hipSuccess) return err;
@@ -750,7 +778,22 @@ static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t
 template <typename F>
 static hipError_t launch_slice_bwd_edge(const SliceParams<F>& p, hipStream_t s)
 {
-    return launch_slice_bwd_edge_cfg<F, kEdgeBlock<F>, 16>(p, s);
+    // with or without messages and carried forces, every slice complete or not: compiled apart, so that the loop
+    // body has no branches (a wait for a load counts the memory operations requested after it; where paths merge
+    // it assumes the shorter one, and would wait for stores of the longer)
+    constexpr int CH = 32 / (int)sizeof(F);
+    const int variant = (p.a.msg ? 4 : 0) + (p.fpart_carry > 0 ? 2 : 0) + (p.a.K % CH == 0 ? 1 : 0);
+    constexpr int BT = kEdgeBlock<F>;
+    switch (variant) {
+    case 0: return launch_slice_bwd_edge_cfg<F, BT, 16, false, false, false>(p, s);
+    case 1: return launch_slice_bwd_edge_cfg<F, BT, 16, false, false, true>(p, s);
+    case 2: return launch_slice_bwd_edge_cfg<F, BT, 16, false, true, false>(p, s);
+    case 3: return launch_slice_bwd_edge_cfg<F, BT, 16, false, true, true>(p, s);
+    case 4: return launch_slice_bwd_edge_cfg<F, BT, 16, true, false, false>(p, s);
+    case 5: return launch_slice_bwd_edge_cfg<F, BT, 16, true, false, true>(p, s);
+    case 6: return launch_slice_bwd_edge_cfg<F, BT, 16, true, true, false>(p, s);
+    default: return launch_slice_bwd_edge_cfg<F, BT, 16, true, true, true>(p, s);
+    }
 }
 template <typename F> int slice_edge_row_elements()
 {

@@ -473,42 +473,71 @@ struct alignas(16) PolyVec {
 constexpr int POLY_VG = POLY_GROUPS;
 static_assert(16 % POLY_VG == 0 && POLY_BLOCK % 64 == 0 && POLY_SPARE_CHUNKS >= 2, "list layout and the kernel's walk must agree");
 
-template <typename F>
-__global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<F> a)
+// Threads of a block: POLY_VG variable groups of PB threads each; thread `tid` of a group owns channel tid % CB of
+// atom group tid / CB (AG atom groups of poly_nb atoms per block, PB = AG * CB rounded up to whole wavefronts).
+// With K = 96 two atom groups fill three wavefronts exactly, where one group alone would leave a third of two
+// wavefronts without a channel.
+struct PolyShape {
+    int CB, AG, PB;   // channels per block, atom groups per block, threads per variable group
+};
+static PolyShape poly_shape(int K, long atom_groups)
+{
+    PolyShape sh;
+    sh.CB = K <= POLY_BLOCK ? K : POLY_BLOCK;
+    sh.AG = 1;
+    double best = 1e30;   // idle lanes per used lane; ties keep the smaller block
+    for (int a = 1; a <= 4; a *= 2) {
+        const int used = a * sh.CB, pb = (used + 63) / 64 * 64;
+        if (a > 1 && pb > 192) break;
+        if (a > 1 && atom_groups / a < 2 * 256) break;   // fewer than two blocks per CU: the lanes gained do not pay
+        const double waste = (double)(pb - used) / used;
+        if (waste < best - 1e-12) { best = waste; sh.AG = a; }
+    }
+    sh.PB = (sh.AG * sh.CB + 63) / 64 * 64;
+    return sh;
+}
+
+template <typename F, int PB>
+__global__ __launch_bounds__(PB * POLY_VG) void k_poly(const PolyParams<F> a, const PolyShape sh)
 {
     constexpr int NB = poly_nb<F>();
-    __shared__ PolyVec<F, NB> X[17][POLY_BLOCK];
-    __shared__ PolyVec<F, NB> fsum[POLY_VG][POLY_BLOCK];
+    extern __shared__ __align__(16) unsigned char poly_smem[];
+    PolyVec<F, NB>* Xs = reinterpret_cast<PolyVec<F, NB>*>(poly_smem);          // [17][PB]
+    PolyVec<F, NB>* fsum = Xs + 17 * PB;                                         // [POLY_VG][PB]
+    auto X = [&](int q) { return Xs + q * PB; };
     // the group index is the same for a whole wavefront: as a scalar it keeps the walk through the lists
     // (indices, chunk counts, coefficient rows) in scalar registers and scalar loads
-    const int tid = threadIdx.x % POLY_BLOCK, vg = __builtin_amdgcn_readfirstlane(threadIdx.x / POLY_BLOCK);
+    const int tid = threadIdx.x % PB, vg = __builtin_amdgcn_readfirstlane(threadIdx.x / PB);
+    const int ag = tid / sh.CB, kloc = tid - ag * sh.CB;
+    const bool tlive = ag < sh.AG;
     constexpr int VPG = 16 / POLY_VG;   // variables per group
-    // species segment and group of atoms of this block row
-    const int kblocks = (a.K + POLY_BLOCK - 1) / POLY_BLOCK;
-    int type = -1, grp = blockIdx.x / kblocks, seg0 = 0, seg_n = 0;
+    // species segment and atom groups of this block row
+    const int kblocks = (a.K + sh.CB - 1) / sh.CB;
+    int type = -1, sg = blockIdx.x / kblocks, seg0 = 0, seg_n = 0;
     for (int t = 0; t < a.T; ++t) {
         const int n_t = a.tstart[t + 1] - a.tstart[t];
-        const int groups = (n_t + NB - 1) / NB;
-        if (grp < groups) { type = t; seg0 = a.tstart[t]; seg_n = n_t; break; }
-        grp -= groups;
+        const int sgroups = ((n_t + NB - 1) / NB + sh.AG - 1) / sh.AG;
+        if (sg < sgroups) { type = t; seg0 = a.tstart[t]; seg_n = n_t; break; }
+        sg -= sgroups;
     }
     if (type < 0) return;
-    const int k = (blockIdx.x % kblocks) * POLY_BLOCK + tid;
-    const bool klive = k < a.K;
+    const int grp = sg * sh.AG + (tlive ? ag : 0);
+    const int k = (blockIdx.x % kblocks) * sh.CB + kloc;
+    const bool klive = tlive && k < a.K;
     const unsigned kk = klive ? k : a.K - 1;
     int node[NB];
     bool nlive[NB];
 #pragma unroll
     for (int b = 0; b < NB; ++b) {
         const int j = grp * NB + b;
-        nlive[b] = j < seg_n;
-        node[b] = a.perm[seg0 + (nlive[b] ? j : seg_n - 1)];
+        nlive[b] = tlive && j < seg_n;
+        node[b] = a.perm[seg0 + (j < seg_n ? j : seg_n - 1)];
     }
     for (int q = vg; q < 17; q += POLY_VG) {
         PolyVec<F, NB> x;
 #pragma unroll
         for (int b = 0; b < NB; ++b) x.v[b] = q < 16 ? a.A[((size_t)node[b] * 16 + q) * a.K + kk] : F(1);
-        X[q][tid] = x;
+        X(q)[tid] = x;
     }
     __syncthreads();
     for (int pl = 0; pl < a.NP; ++pl) {
@@ -554,7 +583,7 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
 #pragma unroll
                 for (int q = 0; q < 4; ++q) {
                     const int ia = (e4[q] >> 16) & 0xff, ib = (e4[q] >> 24) & 0xff;
-                    const PolyVec<F, NB> xa = X[ia][tid], xb = X[ib][tid];
+                    const PolyVec<F, NB> xa = X(ia)[tid], xb = X(ib)[tid];
 #pragma unroll
                     for (int b = 0; b < NB; ++b) g[b] += w[q] * (xa.v[b] * xb.v[b]);
                 }
@@ -563,7 +592,7 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
                 for (int q = 0; q < 4; ++q) w[q] = wn[q];
                 if (i + 1 == n0) {
                     // the monomials that start with v are done: their sum times x_v is v's share of P
-                    const PolyVec<F, NB> xv = X[v][tid];
+                    const PolyVec<F, NB> xv = X(v)[tid];
 #pragma unroll
                     for (int b = 0; b < NB; ++b) f[b] += xv.v[b] * g[b];
                 }
@@ -582,7 +611,7 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
             PolyVec<F, NB> fv;
 #pragma unroll
             for (int b = 0; b < NB; ++b) fv.v[b] = f[b];
-            fsum[vg][tid] = fv;
+            fsum[vg * PB + tid] = fv;
         }
         __syncthreads();
         if (vg == 0) {
@@ -590,7 +619,7 @@ __global__ __launch_bounds__(POLY_BLOCK * POLY_VG) void k_poly(const PolyParams<
             for (int b = 0; b < NB; ++b) {
                 F t = F(0);
 #pragma unroll
-                for (int g2 = 0; g2 < POLY_VG; ++g2) t += fsum[g2][tid].v[b];
+                for (int g2 = 0; g2 < POLY_VG; ++g2) t += fsum[g2 * PB + tid].v[b];
                 if (klive && nlive[b]) a.M[((size_t)node[b] * a.NP + pl) * a.K + k] = t;
             }
         }
@@ -630,10 +659,28 @@ template <typename F>
 hipError_t launch_poly(const PolyParams<F>& p, hipStream_t s)
 {
     if (p.num_nodes <= 0) return hipSuccess;
-    const int kblocks = (p.K + POLY_BLOCK - 1) / POLY_BLOCK;
-    const unsigned groups = (unsigned)((p.num_nodes + poly_nb<F>() - 1) / poly_nb<F>() + p.T);
-    hipLaunchKernelGGL(k_poly<F>, dim3(groups * kblocks), dim3(POLY_BLOCK * POLY_VG), 0, s, p);
-    return hipGetLastError();
+    const PolyShape sh = poly_shape(p.K, (p.num_nodes + poly_nb<F>() - 1) / poly_nb<F>());
+    const int kblocks = (p.K + sh.CB - 1) / sh.CB;
+    const int per_block = poly_nb<F>() * sh.AG;
+    const unsigned sgroups = (unsigned)((p.num_nodes + per_block - 1) / per_block + p.T);
+    const size_t lds = (size_t)(17 + POLY_VG) * sh.PB * 16;
+    auto go = [&](auto pbc) -> hipError_t {
+        constexpr int PB = decltype(pbc)::value;
+        static bool attr_done = false;   // per instantiation
+        if (!attr_done) {
+            hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_poly<F, PB>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024);
+            if (err != hipSuccess) return err;
+            attr_done = true;
+        }
+        hipLaunchKernelGGL((k_poly<F, PB>), dim3(sgroups * kblocks), dim3(PB * POLY_VG), lds, s, p, sh);
+        return hipGetLastError();
+    };
+    switch (sh.PB) {
+    case 64: return go(std::integral_constant<int, 64>{});
+    case 128: return go(std::integral_constant<int, 128>{});
+    case 192: return go(std::integral_constant<int, 192>{});
+    default: return hipErrorInvalidValue;
+    }
 }
 template hipError_t launch_poly<double>(const PolyParams<double>&, hipStream_t);
 template hipError_t launch_poly<float>(const PolyParams<float>&, hipStream_t);

@@ -54,6 +54,28 @@ def test_tiny_configuration_at_full_size_against_the_oracle(gpu, tmp_models, pai
     assert np.abs(F - H.atom_forces(nl, orc.node_forces, len(pos))).max() <= TOL[dtype]["F"] * 10
 
 
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+def test_headline_configuration_at_full_size_against_the_oracle(gpu, tmp_models, dtype):
+    """3 000 atoms H/C/N/O, K = 96, scalar hidden features, one radial table: the benchmark's headline workload,
+    whole, against the oracle (about two seconds of CPU).  At this size the symmetric contraction takes two atom
+    groups per block in double precision (96 channels fill three wavefronts only in pairs), which small cases never do."""
+    from oracle.oracle import OracleMACE
+    from symmetrix_amd import neighbors, systems
+    path, cfg = _model_file(tmp_models, "off_small", pair_dependent_radial=False)
+    pos, cell, sp = systems.config_system("off_small")
+    assert len(pos) == 3000 and cfg["num_channels"] == 96
+    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"]); ea = neighbors.edge_arrays(nl, sp)
+    print(f"off_small: {len(pos)} atoms, {len(ea['r'])} edges, {dtype}", flush=True)
+    orc = OracleMACE(path)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng = gpu(path, dtype)
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    Eo = orc.node_energies.sum()
+    assert abs(eng.node_energies.sum() - Eo) <= TOL[dtype]["E"] * abs(Eo)
+    assert np.abs(eng.node_energies - orc.node_energies).max() <= TOL[dtype]["E"] * max(1.0, np.abs(orc.node_energies).max()) * 10
+    assert np.abs(eng.node_forces - orc.node_forces).max() <= TOL[dtype]["F"]
+
+
 def test_water_box_with_ghost_nodes_at_full_size(gpu, tmp_models):
     """25 002 atoms, K = 128, hidden features up to l = 1, r_cut 5.0 A, through the full neighbour list with ghost
     atoms as extra nodes (the pair style's no_mpi_message_passing layout on one rank): node energies bit-equal to

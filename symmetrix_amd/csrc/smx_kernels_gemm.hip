@@ -228,10 +228,14 @@ constexpr int ROWS_KMAX = 128;
 constexpr int ROWS_MMAX = 8;                     // 16-row tiles per wavefront at most
 constexpr size_t ROWS_OFFS_BYTES = 8 * ROWS_MMAX * 16 * sizeof(int2);
 
-template <typename TA, typename TC, typename CT, int NTW, bool SCALED>
+// KQ: the inner sizes the instantiation takes, in quarters of ROWS_KMAX (3: up to 96, 4: up to 128).  Rows are held
+// whole in registers (this tile's, the next one's, with SCALED the next one's factors), so K = 96 in the 128-wide
+// instantiation pays a quarter more loads and registers than it needs (256 registers with SCALED in fp64).
+template <typename TA, typename TC, typename CT, int NTW, bool SCALED, int KQ>
 __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> g, const int m)
 {
-    constexpr int VL = rows_vl<CT>(), KG = 4 * VL, KJ = ROWS_KMAX / KG;
+    constexpr int VL = rows_vl<CT>(), KG = 4 * VL, KMAXT = ROWS_KMAX * KQ / 4, KJ = KMAXT / KG;
+    static_assert(KMAXT % KG == 0, "whole groups of k");
     constexpr int GN = 32 * NTW, SW = rows_sw<CT, NTW>();
     extern __shared__ __align__(16) unsigned char smem_raw[];
     CT* Wl = reinterpret_cast<CT*>(smem_raw);          // [Kp][SW], rows Kd..Kp-1 zero
@@ -312,7 +316,7 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
     // A weight block goes to LDS in two steps: all loads (four-element groups, WQ per thread at most), later
     // the writes.  The first block's loads are issued before anything else: they are answered from L2 while
     // the species permutation, on which the first rows' addresses depend, is still on its way.
-    constexpr int WQ = ROWS_KMAX * (GN / 4) / 512;
+    constexpr int WQ = (KMAXT * (GN / 4) + 511) / 512;
     auto w_issue = [&](const CT* W, int trans, int Kw, int Kp, Vec4<CT> (&w)[WQ]) {
         const int groups = Kp * (GN / 4);
 #pragma unroll
@@ -453,14 +457,14 @@ __global__ __launch_bounds__(512) void k_gemm_rows(const GemmParams<TA, TC, CT> 
     }
 }
 
-template <typename TA, typename TC, typename CT, int NTW, bool SCALED>
-hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, size_t lds, long total_rows,
+template <typename TA, typename TC, typename CT, int NTW, bool SCALED, int KQ>
+hipError_t launch_gemm_rows_q(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, size_t lds, long total_rows,
                               hipStream_t s)
 {
     constexpr int GN = 32 * NTW;
     static bool attr_done = false;   // per instantiation
     if (!attr_done) {
-        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_rows<TA, TC, CT, NTW, SCALED>),
+        hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_gemm_rows<TA, TC, CT, NTW, SCALED, KQ>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (err != hipSuccess) return err;
         attr_done = true;
@@ -470,7 +474,7 @@ hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int 
     // rows are resident at once.  Blocks go to the eight dies in turn, whatever they find there, so the
     // count leaves an eighth of the block slots free for an uneven split.
     int per_cu = 1;
-    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemm_rows<TA, TC, CT, NTW, SCALED>, 512, lds) != hipSuccess || per_cu < 1)
+    if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, k_gemm_rows<TA, TC, CT, NTW, SCALED, KQ>, 512, lds) != hipSuccess || per_cu < 1)
         per_cu = 1;
     if (!p.perm) {
         // exact block count: every slot can be used
@@ -482,7 +486,7 @@ hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int 
         };
         long m = 1;
         while (m < ROWS_MMAX && blocks_for(m) > 256L * per_cu) ++m;
-        hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW, SCALED>), dim3((unsigned)blocks_for(m)), dim3(512), lds, s, p, (int)m);
+        hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW, SCALED, KQ>), dim3((unsigned)blocks_for(m)), dim3(512), lds, s, p, (int)m);
         return hipGetLastError();
     }
     const long slots = 224L * per_cu;
@@ -491,8 +495,21 @@ hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int 
     while (m < ROWS_MMAX && (total_rows + 64 * m - 1) / (64 * m) * gy + slack > slots) ++m;
     const long rows = (long)p.num_nodes * max_sub;
     const unsigned gx = (unsigned)((rows + 64 * m - 1) / (64 * m) + p.T);
-    hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW, SCALED>), dim3(gx, gy, p.nprob), dim3(512), lds, s, p, (int)m);
+    hipLaunchKernelGGL((k_gemm_rows<TA, TC, CT, NTW, SCALED, KQ>), dim3(gx, gy, p.nprob), dim3(512), lds, s, p, (int)m);
     return hipGetLastError();
+}
+
+template <typename TA, typename TC, typename CT, int NTW, bool SCALED>
+hipError_t launch_gemm_rows_t(const GemmParams<TA, TC, CT>& p, int max_sub, int max_n, size_t lds, long total_rows,
+                              hipStream_t s)
+{
+    // the narrower instantiation for the working precisions (the mixed ones serve inspection calls only)
+    if constexpr (std::is_same<TA, CT>::value && std::is_same<TC, CT>::value) {
+        int kmax = 0;
+        for (int z = 0; z < p.nprob; ++z) kmax = std::max(kmax, std::max(p.prob[z].Kd, p.prob[z].A2 ? p.prob[z].Kd2 : 0));
+        if (kmax <= ROWS_KMAX * 3 / 4) return launch_gemm_rows_q<TA, TC, CT, NTW, SCALED, 3>(p, max_sub, max_n, lds, total_rows, s);
+    }
+    return launch_gemm_rows_q<TA, TC, CT, NTW, SCALED, 4>(p, max_sub, max_n, lds, total_rows, s);
 }
 
 template <typename TA, typename TC, typename CT, int NT>

@@ -505,7 +505,9 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
     constexpr int ROWS = 64 / RL;                            // receivers a wavefront works on at a time
     const int row = lane / RL, sub = lane % RL;
     const int kc = slice * CH;
-    const bool whole = WHOLE || kc + CH <= K;               // all channels of the slice exist (WHOLE: of every slice)
+    // all channels of the slice exist (WHOLE: of every slice) and rows of K elements keep its 32-byte pieces on
+    // 16-byte addresses: only then are they moved as vectors
+    const bool whole = WHOLE || (kc + CH <= K && (K * sizeof(F)) % 16 == 0);
     // staged adjoint rows of the wavefront's receivers, [harmonic][receiver][CH]: the receivers' reads of one
     // harmonic (same instruction, one 32-byte piece each) cover contiguous memory
     F* dstage = reinterpret_cast<F*>(smem + (size_t)R * W * sizeof(F)) + ((size_t)wave * 16 * ROWS + row) * CH;

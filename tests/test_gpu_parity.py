@@ -121,6 +121,28 @@ def test_long_spline_tables_take_the_narrow_slice_kernels(gpu, tmp_models, K, na
 
 
 @pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("K,natoms", [(6, 41), (7, 33), (20, 52)])
+def test_channel_counts_that_leave_the_last_slice_incomplete(gpu, tmp_models, K, natoms, dtype):
+    """One radial table that fits the LDS in 32-byte slices (4 doubles or 8 floats of channels), scalar hidden
+    features, and a channel count that is no multiple of the slice: the last slice of the 32-byte kernels of both
+    directions has channels missing (K = 20 only in single precision), which they handle by element-wise loads and
+    stores compiled apart from the whole-slice code."""
+    model = H.tiny_model(K=K, L_max=0, n_pts=64, seed=100 + K, pair=False)
+    path = H.write_model(model, tmp_models / f"partial_{K}.json")
+    orc = _oracle()(model)
+    eng = gpu(path, dtype)
+    pos, cell, sp = H.small_system(natoms, seed=natoms)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K={K} atoms={natoms} edges={len(ea['r'])} {dtype} incomplete last slice", flush=True)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    _compare(orc, eng, dtype)
+    f1, e1 = eng.node_forces, eng.node_energies
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    assert np.array_equal(f1, eng.node_forces) and np.array_equal(e1, eng.node_energies)
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
 def test_golden_fixture(gpu, dtype):
     z = np.load(os.path.join(GOLD, "tiny_case.npz"))
     eng = gpu(os.path.join(GOLD, "tiny_model.json"), dtype)

@@ -76,6 +76,27 @@ def test_headline_configuration_at_full_size_against_the_oracle(gpu, tmp_models,
     assert np.abs(eng.node_forces - orc.node_forces).max() <= TOL[dtype]["F"]
 
 
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("L_max", [0, 1])
+def test_contraction_blocks_of_several_atom_groups(gpu, tmp_models, L_max, dtype):
+    """4 400 atoms with K = 32: enough atoms that the symmetric contraction packs two atom groups of 32 channels into
+    one wavefront per variable group, in either precision (single precision takes four atoms per thread and needs
+    more than 4 096 atoms for it), with one polynomial (scalar hidden features) and with four."""
+    from oracle.oracle import OracleMACE
+    model = H.tiny_model(K=32, L_max=L_max, n_pts=64, seed=40 + L_max, pair=False)
+    path = H.write_model(model, tmp_models / f"groups_{L_max}.json")
+    pos, cell, sp = H.small_system(4400, seed=9)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K=32 L_max={L_max} atoms=4400 edges={len(ea['r'])} {dtype}", flush=True)
+    orc = OracleMACE(path)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng = gpu(path, dtype)
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    Eo = orc.node_energies.sum()
+    assert abs(eng.node_energies.sum() - Eo) <= TOL[dtype]["E"] * max(abs(Eo), np.abs(orc.node_energies).sum() * 1e-3)
+    assert np.abs(eng.node_forces - orc.node_forces).max() <= TOL[dtype]["F"] * max(1.0, np.abs(orc.node_forces).max())
+
+
 def test_water_box_with_ghost_nodes_at_full_size(gpu, tmp_models):
     """25 002 atoms, K = 128, hidden features up to l = 1, r_cut 5.0 A, through the full neighbour list with ghost
     atoms as extra nodes (the pair style's no_mpi_message_passing layout on one rank): node energies bit-equal to

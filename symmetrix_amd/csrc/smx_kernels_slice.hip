@@ -749,8 +749,9 @@ hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s)
     default: return hipErrorInvalidValue;
     }
 }
-// threads per block of the lane-per-edge adjoint kernel: three wavefronts per SIMD, 168 registers each (four per
-// SIMD, which the LDS has room for, spill in double precision and gain nothing measurable in single)
+// threads per block of the lane-per-edge adjoint kernel: three wavefronts per SIMD, up to 168 registers each (four
+// per SIMD would need the table rows without their padding to fit the LDS, and plain 512-byte rows put every lane's
+// piece on the same banks: twice the time)
 template <typename F> constexpr int kEdgeBlock = 768;
 template <typename F, int BT, int RL, bool MSG, bool CARRY, bool WHOLE>
 static hipError_t launch_slice_bwd_edge_cfg(const SliceParams<F>& p, hipStream_t s)

@@ -9,6 +9,9 @@ HBM.  Metric: atom-steps/s = atoms / seconds per step.
 Prints ONE JSON line.  Besides the driver's fields it carries
   roofline      the slowest edge kernel of the step against the HBM roofline
                 (algorithmic bytes per launch / HIP-event duration of that kernel's stage)
+  roofline_stages   the same figures for every edge stage (aggregations, their adjoints, the sender-side sum)
+  mfma          the dense channel-mixing stages against the matrix-core peak (algorithmic flops / stage time), with the
+                matrix-pipe busy share rocprofv3 counted for the stage's kernel (profiles/)
   cpu_baseline  the CPU oracle (serial fp64 restatement of the reference path)
                 timed on this host on the same workload
   stages_ms     HIP-event time of every stage of the pipeline
@@ -16,6 +19,8 @@ Prints ONE JSON line.  Besides the driver's fields it carries
   second_config     (default run) the metric's second configuration: 50 000-atom alloy, K = 128, l <= 1 hidden
                     features, float32 features, with its own roofline
   pair_dependent_tables   (default run) the headline workload with one radial table per species pair
+  capacity_config   (default run) the capacity configuration: a million-atom water box, MD-style steps with the
+                    neighbour list searched and filtered on the device
 """
 from __future__ import annotations
 
@@ -67,6 +72,43 @@ def measured_traffic(workload, dtype, stage, kernel):
             try:
                 return float(cols[k + 3]) * 1e6      # columns after the stage: fetch MB, write MB, traffic MB
             except (ValueError, IndexError):
+                return None
+    return None
+
+
+MFMA_PEAK = {"float64": 78.6e12, "float32": 157.3e12}   # dense matrix-core peaks of MI355X, flop/s
+# kernel behind each dense stage (as the kernel trace names it) when it runs in feature precision F
+DENSE_KERNEL = {"A0_lin": "k_gemm_rows<{F}, {F}, {F}, 3, false", "A1": "k_gemm_rows<{F}, {F}, {F}, 3, false",
+                "H1": "k_gemm_rows<{F}, {F}, {F}, 1, false", "H2": "k_tail_fused<{F}",
+                "rev_A1": "k_gemm_rows<{F}, {F}, {F}, 3, true", "rev_A0_lin": "k_gemm_rows<{F}, {F}, {F}, 3, true",
+                "rev_H1": "k_gemm_rows<{F}, {F}, {F}, 1, false"}
+
+
+def dense_flops(stage, N, K, n_LM, n_e):
+    """Algorithmic flops per evaluation of a dense stage: 2 x rows x K x K multiply-adds per atom for the products
+    (A0 linear: 16 rows; H1: n_LM; A1: n_e rows of K into 16 / n_e, i.e. 2 n_e K^2; H2: two K x K products), the
+    readout network 2 x 16 K each way, and as much again for each adjoint."""
+    per_atom = {
+        "A0_lin": 32 * K * K, "rev_A0_lin": 32 * K * K,
+        "H1": 2 * n_LM * K * K, "rev_H1": 2 * n_LM * K * K,
+        "A1": 2 * n_e * K * K, "rev_A1": 2 * n_e * K * K,
+        "H2": 8 * K * K + 128 * K,      # H2, readout network with its gradient, reverse_H2: one launch
+    }
+    return per_atom[stage] * N
+
+
+def measured_mfma_busy(workload, dtype, stage):
+    """Matrix-pipe busy share of the kernel behind a dense stage (SQ_VALU_MFMA_BUSY_CYCLES over SIMD cycles), from
+    the rocprofv3 counter summary kept under profiles/; None when the file has no line for that kernel."""
+    path = os.path.join(HERE, "profiles", f"bench_{workload}_shader_counters.txt")
+    if not os.path.exists(path) or stage not in DENSE_KERNEL:
+        return None
+    name = DENSE_KERNEL[stage].format(F="double" if dtype == "float64" else "float")
+    for line in open(path):
+        if line.startswith(name) and line.rstrip().endswith("%"):
+            try:
+                return float(line.split()[-1].rstrip("%")) / 100.0
+            except ValueError:
                 return None
     return None
 
@@ -194,6 +236,21 @@ def run_capacity(args):
     free_b, total_b = torch.cuda.mem_get_info()
     ms = 1e3 * float(np.mean(t_step))
     K, L_max = cfg["num_channels"], cfg["L_max"]
+    # stage times of two more evaluations on the last list (HIP events on the kernels' stream)
+    eng.set_profiling(True)
+    acc = {}
+    for _ in range(2):
+        evaluate(E)
+        for k, v in eng.stage_times().items():
+            acc[k] = acc.get(k, 0.0) + v / 2
+    eng.set_profiling(False)
+    n_LM, n_e, s_b = (L_max + 1) ** 2, 16 if L_max == 0 else 40, 8 if args.dtype == "float64" else 4
+    # When the adjoint messages exceed the staging buffer, the layer-1 adjoint and the sender-side sum alternate per
+    # receiver chunk inside one stage: the roofline then prices both kernels' bytes against the stage's time.
+    chunked = acc.get("sender_reduce", 0.0) < 0.01 * acc.get("agg1_bwd", 1.0)
+    b_bwd = algorithmic_bytes("agg1_bwd", N, E, K, s_b, n_LM, n_e) + (algorithmic_bytes("sender_reduce", N, E, K, s_b, n_LM, n_e) if chunked else 0)
+    t_bwd = acc.get("agg1_bwd", 0.0) * 1e-3
+    ach = b_bwd / t_bwd / 1e9 if t_bwd > 0 else 0.0
     line = {
         "metric": "atom-steps/s per MI355X (energy+forces)", "value": N / (ms * 1e-3), "unit": "atom-steps/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "ms_per_step": ms, "higher_is_better": True,
@@ -209,14 +266,21 @@ def run_capacity(args):
             "evaluation": 1e3 * float(np.mean(t_eval)),
             "move_and_list_search": 1e3 * float(np.mean(t_list_build)) if t_list_build else None,
             "move_and_list_filter": 1e3 * float(np.mean(t_list_update)) if t_list_update else None,
+            "list_searches_timed": len(t_list_build), "list_filters_timed": len(t_list_update),
         },
         "evaluation_only_value": N / float(np.mean(t_eval)),
         "hbm_in_use_GB": (total_b - free_b) / 1e9,
         "copies_check": {"energy_max_abs_diff": e_dev, "energy_scale": e_scale, "atom_force_max_abs_diff": f_dev, "atom_force_scale": f_scale,
                          "note": "64 periodic copies of the small box before the first move: equal up to summation order"},
         "energy_first": energy0,
+        "stages_ms": acc,
+        "roofline": {"bound": "hbm", "kernel": "k_agg_bwd" + (" + k_sender_reduce, alternating per receiver chunk" if chunked else ""),
+                     "stage": "agg1_bwd", "achieved": ach, "peak": HBM_PEAK / 1e9, "unit": "GB/s", "frac": ach / (HBM_PEAK / 1e9),
+                     "traffic": None, "algorithmic_bytes_per_launch": b_bwd, "kernel_ms": acc.get("agg1_bwd", 0.0)},
     }
-    print(json.dumps(line))
+    del eng, nl, out_E, out_F, dpos, dty
+    torch.cuda.empty_cache()
+    return line
 
 
 def main():
@@ -263,7 +327,8 @@ def main():
         sys.exit(1)
     dev = torch.device("cuda:0")
     if args.workload == "water_capacity":
-        return run_capacity(args)
+        print(json.dumps(run_capacity(args)))
+        return
 
     def measure(workload, dtype, steps, warmup, pair_tables=False, ghosts=False, scale=1.0, both=True, host_leg=True):
         """One workload in one precision (and, with `both`, in the other): model file, synthetic system, timing."""
@@ -373,6 +438,32 @@ def main():
         achieved = dom_bytes / dom_s / 1e9 if dom_s > 0 else 0.0
         total_bytes = sum(stage_bytes(k) for k in EDGE_STAGES) + (32 * E + 24 * N)
         kernel = stage_kernel(dom, L_max, res["tables"])
+        prof_name = workload + ("_pairs" if pair_tables else "")
+        profiled = scale == 1.0 and not ghosts
+        stages_rl = {}
+        for k in EDGE_STAGES:
+            ms_k = res["stages"].get(k, 0.0)
+            if ms_k <= 0.0:
+                continue
+            b_k = stage_bytes(k)
+            kern_k = stage_kernel(k, L_max, res["tables"])
+            ach = b_k / (ms_k * 1e-3) / 1e9
+            stages_rl[k] = {"kernel": kern_k, "algorithmic_bytes": b_k, "kernel_ms": ms_k, "achieved": ach,
+                            "frac": ach / (HBM_PEAK / 1e9),
+                            "traffic": measured_traffic(prof_name, dtype, k, kern_k) if profiled else None}
+        mfma = {}
+        for k in ("A0_lin", "H1", "A1", "H2", "rev_A1", "rev_H1", "rev_A0_lin"):
+            ms_k = res["stages"].get(k, 0.0)
+            n_k = (N + N_ghost) if k in ("A0_lin", "H1", "rev_H1", "rev_A0_lin") else N
+            fl = dense_flops(k, n_k, K, n_LM, n_e)
+            # the tail works in double whatever the feature precision; a stage folded into another launch has no time of its own
+            peak = MFMA_PEAK["float64"] if k == "H2" else MFMA_PEAK[dtype]
+            if ms_k < 0.006:
+                mfma[k] = {"flops": fl, "note": "folded into another launch (sender_reduce carries reverse_H1 for scalar hidden features)"}
+                continue
+            mfma[k] = {"flops": fl, "kernel_ms": ms_k, "achieved_tflops": fl / (ms_k * 1e-3) / 1e12, "peak_tflops": peak / 1e12,
+                       "frac": fl / (ms_k * 1e-3) / peak,
+                       "mfma_busy_profiled": measured_mfma_busy(workload, dtype, k) if profiled and not pair_tables else None}
         out = dict(
             cfg=cfg, model_path=model_path, ea=ea, N=N, E=E, N_ghost=N_ghost, E_local=E_local, res=res,
             value=N / (res["ms"] * 1e-3),
@@ -382,11 +473,12 @@ def main():
             roofline={
                 "bound": "hbm", "kernel": kernel, "stage": dom, "achieved": achieved, "peak": HBM_PEAK / 1e9, "unit": "GB/s",
                 "frac": achieved / (HBM_PEAK / 1e9),
-                "traffic": measured_traffic(workload, dtype, dom, kernel) if scale == 1.0 and not ghosts and not pair_tables else None,
+                "traffic": measured_traffic(prof_name, dtype, dom, kernel) if profiled else None,
                 "algorithmic_bytes_per_launch": dom_bytes, "kernel_ms": res["stages"][dom],
                 "whole_step_algorithmic_bytes": total_bytes,
                 "whole_step_frac": (total_bytes / HBM_PEAK) / (res["ms"] * 1e-3),
             },
+            roofline_stages=stages_rl, mfma=mfma,
         )
         if both:
             other = "float32" if dtype == "float64" else "float64"
@@ -424,6 +516,8 @@ def main():
             "scale": args.scale, "ghost_nodes": m["N_ghost"], "edges_of_local_receivers": m["E_local"],
         },
         "roofline": m["roofline"],
+        "roofline_stages": m["roofline_stages"],
+        "mfma": m["mfma"],
         "stages_ms": res["stages"],
         "ms_per_step_with_event_readback": res["ms_sync"],
         "host_arrays": {"ms_per_step": res["ms_host"], "value": N / (res["ms_host"] * 1e-3),
@@ -441,6 +535,7 @@ def main():
         line["second_config"] = {
             "workload": m2["workload"], "dtype": "f32-features/f64-accumulation", "steps": s2, "warmup": 2,
             "ms_per_step": m2["res"]["ms"], "value": m2["value"], "unit": "atom-steps/s", "roofline": m2["roofline"],
+            "roofline_stages": m2["roofline_stages"], "mfma": m2["mfma"],
             "stages_ms": m2["res"]["stages"], "energy": m2["res"]["energy"],
         }
         # the headline workload with one radial table per species pair (ten tables for four species): more than four
@@ -448,8 +543,19 @@ def main():
         m3 = measure("off_small", args.dtype, max(5, args.steps // 2), args.warmup, pair_tables=True, both=False, host_leg=False)
         line["pair_dependent_tables"] = {
             "workload": m3["workload"], "dtype": line["dtype"], "ms_per_step": m3["res"]["ms"], "value": m3["value"],
-            "unit": "atom-steps/s", "roofline": m3["roofline"], "stages_ms": m3["res"]["stages"],
+            "unit": "atom-steps/s", "roofline": m3["roofline"], "roofline_stages": m3["roofline_stages"],
+            "stages_ms": m3["res"]["stages"],
         }
+        # the capacity configuration at its size, a short MD-style loop (two list searches); freed before the CPU leg
+        del m2, m3
+        torch.cuda.empty_cache()
+        free_b, _ = torch.cuda.mem_get_info()
+        if free_b > 200e9:
+            cargs = argparse.Namespace(**vars(args))
+            cargs.steps, cargs.warmup, cargs.dtype, cargs.rebuild_every = 20, 2, "float32", 10
+            line["capacity_config"] = run_capacity(cargs)
+        else:
+            line["capacity_config"] = {"skipped": f"needs about 185 GB of free HBM, {free_b / 1e9:.0f} GB are free"}
 
     # ---- CPU baseline: the oracle (serial fp64 port of the reference path) on this host
     if not args.no_cpu:

@@ -212,8 +212,12 @@ int smx_reduce_forces_device(smx_model* m, int num_atoms, const int* d_sender_at
  * without synchronising.  The per-atom sender lists and the partial virial sums live in a fixed array of about
  * 20 MiB that every GPU holds from the first model load to the end of the process, so sizes beyond
  * SMX_NOALLOC_MAX_ATOMS atoms or SMX_NOALLOC_MAX_EDGES edges are refused with SMX_EINVAL, and calls that overlap on
- * one GPU race (all of them share that GPU's array).  A sender index outside [0, num_atoms) cannot be reported
- * without a synchronisation: the outputs are NaN then.  Calls no hipMalloc / hipFree and no allocating routine. */
+ * one GPU race (all of them share that GPU's array).  `stream` must be the stream of the evaluation whose forces
+ * are reduced, or be ordered after it by the caller (an event wait): the call reads the model's node_forces and
+ * edge arrays without any ordering of its own.  The model's GPU must be the current device (SMX_EINVAL otherwise).
+ * A sender index outside [0, num_atoms) cannot be reported without a synchronisation: the outputs are NaN then, as
+ * they are after an evaluation that its input checks skipped.  Calls no hipMalloc / hipFree and no allocating
+ * routine. */
 #define SMX_NOALLOC_MAX_ATOMS 262144
 #define SMX_NOALLOC_MAX_EDGES 4194304
 int smx_reduce_forces_device_noalloc(smx_model* m, int num_atoms, const int* d_sender_atom, double* d_atom_forces,

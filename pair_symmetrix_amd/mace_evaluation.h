@@ -45,7 +45,9 @@ void evaluate_mpi_message_passing(MACE& mace, const EdgeList& e, int num_atom_ro
 // launches and host round trips; kept for cross-checking).
 void evaluate_no_mpi_message_passing(MACE& mace, const EdgeList& e, bool staged = false);
 
-// Sum of node energies of the local nodes (:324-332, 499-502, 702-704).
+// Sum of node energies of the local nodes (:324-332, 499-502, 702-704).  With `eatom`, node ii's energy is written
+// to eatom[node_i[ii]], the atom row of the node (the reference writes eatom[ii], :329-331, 504-507: the same entry
+// while ilist[ii] == ii).
 double total_energy(MACE& mace, const EdgeList& e, double* eatom = nullptr);
 
 // f[node_i] -= f_ij, f[neigh_j] += f_ij over all edges (:334-347, 509-522, 710-723) into f[num_atom_rows][3],

@@ -249,7 +249,8 @@ void PairSymmetrixMACE::compute(int eflag, int vflag)
       for (int i = 0; i < nall; ++i) eatom[i] += eatom_nodes[i];
     // f[i] -= f_ij, f[j] += f_ij and the virial, summed on the device in a fixed order; forces on ghost rows go back
     // to their owners with LAMMPS' reverse communication (newton pair on)
-    symmetrix_amd::scatter_forces(*mace, edges, nall, &atom->f[0][0], vflag_global ? virial : nullptr);
+    if (nall > 0)   // an empty rank has no force array to point into
+      symmetrix_amd::scatter_forces(*mace, edges, nall, &atom->f[0][0], vflag_global ? virial : nullptr);
   } catch (const std::exception &e) {
     error->one(FLERR, "symmetrix/mace: {}", e.what());
   }

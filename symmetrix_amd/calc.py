@@ -22,12 +22,30 @@ from .mace import MACE
 class SymmetrixCalculator:
     implemented_properties = ["energy", "free_energy", "energies", "forces", "stress"]
 
-    def __init__(self, model_file, dtype="float64", neighbor_list="device"):
+    # keywords the reference hands to its on-the-fly conversion of a torch checkpoint (symmetrix_calc.py:58-61)
+    EXTRACT_KEYWORDS = ("species", "head", "num_spline_points")
+
+    def __init__(self, model_file, dtype="float64", use_kokkos=True, neighbor_list="device", **kwargs):
+        """Signature and defaults of the reference's `Symmetrix.__init__` (symmetrix_calc.py:39).  `use_kokkos`
+        selects between two back ends there; here there is one, for both dtypes, and the flag is ignored."""
         if dtype not in ("float32", "float64"):
             raise ValueError(f"Unsupported dtype '{dtype}'. Supported dtypes are 'float64' and 'float32'.")
         if neighbor_list not in ("device", "host"):
             raise ValueError("neighbor_list is 'device' or 'host'")
-        self.evaluator = MACE(str(model_file), dtype)
+        self.use_kokkos = use_kokkos
+        self.extract_kwargs = {k: v for k, v in kwargs.items() if k in self.EXTRACT_KEYWORDS}
+        unknown = sorted(set(kwargs) - set(self.EXTRACT_KEYWORDS))
+        if unknown:
+            raise TypeError(f"unexpected keyword arguments {unknown}")
+        try:
+            self.evaluator = MACE(str(model_file), dtype)
+        except RuntimeError as exc:
+            # The reference converts a torch-MACE checkpoint here (symmetrix_calc.py:54-68); that needs mace-torch,
+            # e3nn and ase, and this package holds no extractor: say what to run instead of failing on the parse error.
+            raise RuntimeError(
+                f"'{model_file}' is not a symmetrix JSON model ({exc}).  Convert the checkpoint once with the "
+                f"reference's extractor, e.g. `symmetrix_extract_mace {model_file}` with {self.extract_kwargs or 'its defaults'}, "
+                f"and pass the JSON file it writes.") from exc
         self.cutoff = self.evaluator.r_cut
         self.results = {}
         self._nlist = neighbors.DeviceNeighborList() if neighbor_list == "device" else None
@@ -74,9 +92,11 @@ try:  # pragma: no cover - ase is not installed in the build image
     class Symmetrix(Calculator):
         implemented_properties = SymmetrixCalculator.implemented_properties
 
-        def __init__(self, model_file, dtype="float64", use_kokkos=False, **kwargs):
-            Calculator.__init__(self, **kwargs)
-            self._impl = SymmetrixCalculator(model_file, dtype)
+        def __init__(self, model_file, dtype="float64", use_kokkos=True, **kwargs):
+            Calculator.__init__(self, **kwargs)     # symmetrix_calc.py:40: every keyword goes to the base class
+            extract = {k: v for k, v in kwargs.items() if k in SymmetrixCalculator.EXTRACT_KEYWORDS}
+            self._impl = SymmetrixCalculator(model_file, dtype, use_kokkos, **extract)
+            self.use_kokkos = use_kokkos
             self.evaluator = self._impl.evaluator
             self.cutoff = self._impl.cutoff
 

@@ -121,6 +121,7 @@ struct EngineBase {
     }
     HostModel hm;
     int precision = 0;
+    int device = 0;                 // ordinal of the GPU the model was loaded on
     hipStream_t stream = nullptr;   // stream of the current call
     bool profiling = false;
     hipEvent_t ev0[ST_COUNT] = {}, ev1[ST_COUNT] = {};
@@ -236,6 +237,7 @@ struct Engine : EngineBase {
     {
         hm = std::move(m);
         precision = prec;
+        HIPCHK(hipGetDevice(&device));
         hipStream_t s = nullptr;
         auto cat = [](const std::vector<std::vector<double>>& t) {
             std::vector<double> out;
@@ -333,18 +335,20 @@ struct Engine : EngineBase {
     }
 
     // ---- input checks of device-resident evaluations.  flags[0]: host-array calls (read back at once);
-    // flags[1]: sticky status of device-resident calls, read by the next synchronising call; flags[2], flags[3]:
-    // status word of the running / the next device-resident evaluation, taken in turn (an evaluation clears the
-    // other word for its successor; a captured graph keeps the word it was captured with, so after a failed
-    // evaluation one replay of an older graph may be skipped as well: the sticky word reports either).
+    // flags[1]: sticky status of device-resident calls, read by the next synchronising call; flags[2]: the word the
+    // checks of the running device-resident evaluation raise; flags[3]: its copy for the kernels after the list
+    // preparation ("live": raised -> energies and forces are NaN).  The evaluation clears flags[2] again in its
+    // readout launch, after the last reader, so every evaluation, eager or a replayed graph, starts from a clean word.
     long device_calls = 0;
-    int* guard_status = nullptr;   // status word of the running evaluation (nullptr: host-array call, checked already)
+    int* guard_status = nullptr;   // check word of the running evaluation (nullptr: host-array call, checked already)
+    bool guard_clear_enqueued = false;   // ... and a launch that clears it again is in the stream
+    const int* guard_live() const { return guard_status ? flags.p + 3 : nullptr; }
     InputGuard input_guard(int N)
     {
         InputGuard g;
         if (!guard_status) return g;
         g.status = guard_status;
-        g.next_status = flags.p + 2 + (guard_status == flags.p + 2 ? 1 : 0);
+        g.live = flags.p + 3;
         g.sticky = flags.p + 1;
         g.first_neigh = first_neigh.p; g.n_first = N + 1;
         g.tstart = t_start.p; g.n_tstart = hm.T + 1;
@@ -361,9 +365,9 @@ struct Engine : EngineBase {
         if (f & 1)
             throw Error(SMX_EINVAL, "a device-resident evaluation was skipped: node_types / neigh_types / neigh_indices hold an "
                                     "index outside the model or the node range, or num_neigh does not add up to the number "
-                                    "of edges (its node energies are NaN)");
+                                    "of edges (its node energies and forces are NaN)");
         throw Error(SMX_ERANGE, "a device-resident evaluation was skipped: an edge length lies outside (0, r_cut) "
-                                "(its node energies are NaN)");
+                                "(its node energies and forces are NaN)");
     }
 
     // Regroup a radial table per channel slice, or return 0 when the slice path does not apply.
@@ -800,8 +804,9 @@ struct Engine : EngineBase {
         p.H1 = H1.p; p.M1 = M1.p; p.W_H1 = H2w_H1.p; p.W_M1 = H2w_M1.p;
         p.H2 = H2.p; p.H2_adj = H2_adj.p; p.H1_adj = H1_adj.p; p.M1_adj = M1_adj.p;
         p.node_energies = node_energies.p; p.zero_energies = zero_energies ? 1 : 0; p.energies_copy = energies_copy;
-        p.guard = guard_status;
+        p.guard = guard_live(); p.guard_clear = guard_status;
         HIPCHK(launch_tail_fused<F>(p, stream));
+        if (guard_status && rows > 0) guard_clear_enqueued = true;
         energies_copy = nullptr;
     }
     void st_readouts(int N, bool zero_energies)
@@ -814,7 +819,8 @@ struct Engine : EngineBase {
         if (rows < N || H2.n < (size_t)N * k) throw Error(SMX_EINVAL, "readouts called before H1 and H2 exist for these nodes");
         HIPCHK(launch_readout_fused<F>(N, rows, k, nlm, node_types, E0.p, ro1.p, ro2_w1.p, ro2_w2.p, hm.readout_2_scale,
                                        H1.p, H2.p, H2_adj.p, H1_adj.p, node_energies.p, zero_energies ? 1 : 0,
-                                       energies_copy, guard_status, stream));
+                                       energies_copy, guard_live(), guard_status, stream));
+        if (guard_status && rows > 0) guard_clear_enqueued = true;
         energies_copy = nullptr;
     }
     // node counts for which compute() left A1_adj / A0_adj unwritten (-1: they are current)
@@ -884,6 +890,7 @@ struct Engine : EngineBase {
         }
         stage_end(ST_SRED);
     }
+    bool forces_poisoned = false;   // the last force launch of compute() looked at the guard itself
     bool carry_forces = false;      // compute() lets the layer-1 partial forces wait for the layer-0 adjoint
     long carried_edges = 0;         // ... and the stage left them in fpart for edges [0, carried_edges)
     int carried_accumulate = 1;
@@ -959,8 +966,9 @@ struct Engine : EngineBase {
             HIPCHK(launch_slice_bwd<F>(sp, stream));
             stage_end(ST_AGG0B);
             stage_begin(ST_FSUM0);
-            HIPCHK(launch_fpart_reduce(E, E, S, fpart.p, node_forces.p, accumulate, forces_copy, stream));
+            HIPCHK(launch_fpart_reduce(E, E, S, fpart.p, node_forces.p, accumulate, forces_copy, stream, guard_live()));
             forces_copy = nullptr;
+            forces_poisoned = true;
             stage_end(ST_FSUM0);
             return;
         }
@@ -995,8 +1003,12 @@ struct Engine : EngineBase {
             compute_impl(N, nt, nn, ni, nty, x, rr, E_, on_device, d_energies, d_forces, N_local, E_local);
         } catch (...) {
             // whatever was half built is not trusted by the next call
-            senders_counted = false; counters_clean = 0; sender_rows = -1; guard_status = nullptr;
+            senders_counted = false; counters_clean = 0; sender_rows = -1;
             energies_copy = nullptr; forces_copy = nullptr;
+            carried_edges = 0; carry_forces = false; fuse_reverse_H1 = false;
+            // checks of the failed call may have raised the word that only its readout launch would have cleared
+            if (guard_status && !guard_clear_enqueued) (void)launch_fill<int>(guard_status, 1, 0, stream);
+            guard_status = nullptr;
             throw;
         }
         guard_status = nullptr;
@@ -1029,9 +1041,9 @@ struct Engine : EngineBase {
         // range checks come before any kernel that uses these integers as indices: host arrays are checked with a
         // read-back below; device arrays inside the list preparation, whose last launch empties the lists when a
         // check failed (input_guard)
-        guard_status = nullptr;
+        guard_status = nullptr; guard_clear_enqueued = false; forces_poisoned = false;
         if (on_device) {
-            guard_status = flags.p + 2 + (int)(device_calls & 1);
+            guard_status = flags.p + 2;
             ++device_calls;
         }
         if (on_device && N <= 65536) {
@@ -1125,6 +1137,9 @@ struct Engine : EngineBase {
         st_scale(0, N, true);
         stage_begin(ST_REVA0LIN); st_A0_lin(N, true, fuse0); stage_end(ST_REVA0LIN);
         st_agg0_bwd(N);
+        // a skipped evaluation (inputs failed the checks on the device) wrote no force: NaN says so, as for the energies
+        if (guard_status && !forces_poisoned) HIPCHK(launch_poison_forces(guard_live(), node_forces.p, nullptr, 3 * E, stream));
+        if (guard_status && !guard_clear_enqueued) HIPCHK(launch_fill<int>(guard_status, 1, 0, stream));
 
         if (energies_copy) HIPCHK(hipMemcpyAsync(energies_copy, node_energies.p, (size_t)N1 * sizeof(double), hipMemcpyDeviceToDevice, stream));
         if (forces_copy && E) HIPCHK(hipMemcpyAsync(forces_copy, node_forces.p, (size_t)3 * E * sizeof(double), hipMemcpyDeviceToDevice, stream));
@@ -1140,6 +1155,7 @@ struct Engine : EngineBase {
     {
         const std::string s(name);
         energies_copy = nullptr; forces_copy = nullptr;
+        carried_edges = 0; carry_forces = false; fuse_reverse_H1 = false; guard_status = nullptr;
         materialise_adjoints();
         if (N < 0) throw Error(SMX_EINVAL, "negative num_nodes");
         // A stage may cover the leading nodes of a longer edge list (the pair style runs layer 1 on its local
@@ -1294,7 +1310,7 @@ struct Engine : EngineBase {
     void forces_view(ForcesView* v) override
     {
         v->node_forces = node_forces.p; v->forces_len = (long)node_forces.n; v->xyz = xyz; v->first_neigh = first_neigh.p;
-        v->num_edges = E; v->num_receivers = N_geo;
+        v->num_edges = E; v->num_receivers = N_geo; v->device = device;
     }
     // size a named array to n entries, all equal to `value`, without a host copy
     void fill_array(const char* name, long n, double value) override
@@ -1872,11 +1888,17 @@ int smx_synchronize(smx_model* m)
 int smx_reduce_forces(smx_model* m, int num_atoms, const int* sender_atom, const int* receiver_atom,
                       double* atom_forces, double* virial)
 {
-    return guarded([&] { E(m).reduce_forces(num_atoms, sender_atom, receiver_atom, atom_forces, virial, false); });
+    return guarded([&] {
+        E(m).reduce_forces(num_atoms, sender_atom, receiver_atom, atom_forces, virial, false);
+        E(m).check_device_status();   // forces of a skipped device-resident evaluation are NaN: say why
+    });
 }
 int smx_reduce_forces_device(smx_model* m, int num_atoms, const int* d_sender_atom, double* atom_forces, double* virial)
 {
-    return guarded([&] { E(m).reduce_forces(num_atoms, d_sender_atom, nullptr, atom_forces, virial, true); });
+    return guarded([&] {
+        E(m).reduce_forces(num_atoms, d_sender_atom, nullptr, atom_forces, virial, true);
+        E(m).check_device_status();
+    });
 }
 
 smx_nlist* smx_nlist_create(void)

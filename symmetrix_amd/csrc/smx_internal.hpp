@@ -14,6 +14,7 @@ struct ForcesView {
     const int* first_neigh;      // [num_receivers + 1]
     long num_edges, forces_len;
     int num_receivers;
+    int device;                  // ordinal of the GPU that holds the model and these arrays
 };
 int engine_forces_view(smx_model* m, ForcesView* out, std::string* err);
 void set_last_error(const std::string& msg);

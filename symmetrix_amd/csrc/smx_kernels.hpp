@@ -86,9 +86,12 @@ template <typename F> int slice_row_elements(int CH);
 template <typename F> hipError_t launch_slice_fwd(const SliceParams<F>& p, hipStream_t s);
 template <typename F> hipError_t launch_slice_bwd(const SliceParams<F>& p, hipStream_t s);
 // forces (+)= sum over slices of fpart, slices added in ascending order
-// (`copy`, if not null, receives the same sums: the caller's output array of the whole-pipeline call)
+// (`copy`, if not null, receives the same sums: the caller's output array of the whole-pipeline call;
+// `guard`, if not null and raised, makes every force NaN instead: the evaluation was skipped)
 hipError_t launch_fpart_reduce(long edges, long E, int nslices, const double* fpart, double* forces, int accumulate,
-                               double* copy, hipStream_t s);
+                               double* copy, hipStream_t s, const int* guard = nullptr);
+// forces[0, n) and copy[0, n) (may be null) become NaN when *guard is raised
+hipError_t launch_poison_forces(const int* guard, double* forces, double* copy, long n, hipStream_t s);
 
 // H1_adj[j] (+)= sum over edges with sender j of msg[e], in ascending edge order.
 // H_adj[j] (+)= sum of msg[e - e_lo] over the edges e of sender j with e_lo <= e < e_hi, in ascending edge order
@@ -158,13 +161,15 @@ hipError_t launch_degree_order(int N, const int* first_neigh, int* order, hipStr
 // counters_are_zero: 0 = clear count and cursor first, 1 = they are zero, 2 = the histogram is already in count and
 // rank[E] holds every entry's place inside its bucket (launch_node_lists_count);
 // count and cursor are zero again when the launches have run
-// Guard of a device-resident evaluation, carried by the last launch of the sender-list build: when this
-// evaluation's status word is raised, first_neigh[n_first] and tstart[n_tstart] are zeroed (no edges, no species
-// groups: the kernels that follow then touch no unchecked index), the status is ORed into the sticky word the host
-// reads later, and the status word of the next evaluation is cleared.  status == nullptr: no guard.
+// Guard of a device-resident evaluation, carried by the last launch of the sender-list build: when the checks of
+// this evaluation raised the status word, first_neigh[n_first] and tstart[n_tstart] are zeroed (no edges, no species
+// groups: the kernels that follow then touch no unchecked index) and the status is ORed into the sticky word the
+// host reads later.  Raised or not, the status is copied into the `live` word, which the kernels after this launch
+// read (energies and forces become NaN); the status word itself is cleared again by the readout kernel of the same
+// evaluation, after every reader of it has run, so that a replayed graph starts clean.  status == nullptr: no guard.
 struct InputGuard {
     const int* status = nullptr;
-    int* next_status = nullptr;
+    int* live = nullptr;
     int* sticky = nullptr;
     int* first_neigh = nullptr; int n_first = 0;
     int* tstart = nullptr; int n_tstart = 0;
@@ -270,7 +275,7 @@ template <typename F>
 hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,
                                 const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
-                                double* energies_copy, const int* guard, hipStream_t s);
+                                double* energies_copy, const int* guard, int* guard_clear, hipStream_t s);
 // H2 (mace.cpp:820-845), the readout tail and reverse_H2 (mace.cpp:847-874) in one launch; K a multiple of 16
 // up to 128 (tail_fused_ok).  Atoms grouped by species (perm, tstart); H1_adj [rows][num_LM][K] is written
 // whole (seed plus the adjoint of H2 in the scalar block, zero elsewhere), M1_adj [N][K] too.
@@ -284,7 +289,8 @@ struct TailParams {
     const double* W_M1;      // [K][K]
     double* H2; double* H2_adj; F* H1_adj; F* M1_adj;
     double* node_energies; int zero_energies; double* energies_copy;
-    const int* guard;        // status word of a device-resident evaluation (or null): raised -> energies are NaN
+    const int* guard;        // live status of a device-resident evaluation (or null): raised -> energies are NaN
+    int* guard_clear;        // the word the input checks of the next evaluation raise (or null): cleared here
 };
 bool tail_fused_ok(int K);
 template <typename F> hipError_t launch_tail_fused(const TailParams<F>& p, hipStream_t s);

@@ -97,7 +97,7 @@ constexpr int SORT_LDS = 1024;
 // With a guard (device-resident callers, whose arrays no host code has looked at): when the checks of this
 // evaluation raised its status word, the CSR offsets and the species groups are set to "no edges, no nodes", so
 // that no later kernel of the evaluation uses an unchecked integer as an address; the status goes into the sticky
-// word the host reads at its next synchronising call, and the word of the next evaluation is cleared.
+// word the host reads at its next synchronising call and, raised or not, into the word the later kernels read.
 __global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows, int* list, int* count, int* cursor,
                                                      InputGuard g)
 {
@@ -110,7 +110,7 @@ __global__ __launch_bounds__(64) void k_sort_buckets(const int* start, int rows,
             for (int i = j * 64 + threadIdx.x; i < g.n_tstart; i += gridDim.x * 64) g.tstart[i] = 0;
             if (j == 0 && threadIdx.x == 0) atomicOr(g.sticky, st);
         }
-        if (j == 0 && threadIdx.x == 0) *g.next_status = 0;
+        if (j == 0 && threadIdx.x == 0) *g.live = st;
     }
     if (threadIdx.x == 0) { count[j] = 0; cursor[j] = 0; }
     const int s0 = start[j], n = start[j + 1] - s0;
@@ -713,9 +713,12 @@ __global__ __launch_bounds__(256) void k_readout_fused(int N, int rows, int K, i
                                                        const double* E0, const double* w1, const double* W1,
                                                        const double* w2, double scale, const F* H1, const double* H2,
                                                        double* H2_adj, F* H1_adj, double* node_energies,
-                                                       int zero_energies, double* energies_copy, const int* guard)
+                                                       int zero_energies, double* energies_copy, const int* guard,
+                                                       int* guard_clear)
 {
     extern __shared__ double rsm[];
+    // every reader of the check word has run (the sender lists come before the readout): clean for the next evaluation
+    if (guard_clear && blockIdx.x == 0 && threadIdx.x == 0) *guard_clear = 0;
     if (guard && *guard) {
         // unchecked species indices: no table lookup, the energies say so
         const int i = blockIdx.x * 16 + (threadIdx.x >> 4);
@@ -804,6 +807,8 @@ __global__ __launch_bounds__(TAIL_BLOCK) void k_tail_fused(const TailParams<F> p
     __shared__ int node_s[16];
     const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int width = p.num_LM * K;
+    // every reader of the check word has run (the sender lists come before the readout): clean for the next evaluation
+    if (p.guard_clear && blockIdx.x == 0 && tid == 0) *p.guard_clear = 0;
     if (p.guard && *p.guard) {
         // the inputs of this evaluation failed their checks and the species groups are empty: the energies say so
         const int i = blockIdx.x * 16 + tid;
@@ -978,7 +983,7 @@ template <typename F>
 hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,
                                 const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
-                                double* energies_copy, const int* guard, hipStream_t s)
+                                double* energies_copy, const int* guard, int* guard_clear, hipStream_t s)
 {
     if (rows < N) return hipErrorInvalidValue;
     if (rows <= 0) return hipSuccess;
@@ -991,11 +996,11 @@ hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* n
     }
     hipLaunchKernelGGL(k_readout_fused<F>, dim3((rows + 15) / 16), dim3(256), lds, s, N, rows, K, num_LM, node_types,
                        atomic_energies, w1, W1, w2, scale, H1, H2, H2_adj, H1_adj, node_energies, zero_energies,
-                       energies_copy, guard);
+                       energies_copy, guard, guard_clear);
     return hipGetLastError();
 }
-template hipError_t launch_readout_fused<double>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const double*, const double*, double*, double*, double*, int, double*, const int*, hipStream_t);
-template hipError_t launch_readout_fused<float>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const float*, const double*, double*, float*, double*, int, double*, const int*, hipStream_t);
+template hipError_t launch_readout_fused<double>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const double*, const double*, double*, double*, double*, int, double*, const int*, int*, hipStream_t);
+template hipError_t launch_readout_fused<float>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const float*, const double*, double*, float*, double*, int, double*, const int*, int*, hipStream_t);
 
 
 // ===========================================================================

@@ -17,6 +17,8 @@
 #include "smx_device.hpp"
 #include "smx_kernels.hpp"
 
+#include <algorithm>
+
 namespace smx {
 
 namespace {
@@ -666,12 +668,14 @@ __global__ __launch_bounds__(BT) void k_slice_bwd_edge(const SliceParams<F> p)
 }
 
 __global__ void k_fpart_reduce(long n3, long stride3, int nslices, const double* fpart, double* forces, int accumulate,
-                               double* copy)
+                               double* copy, const int* guard)
 {
     const long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
     if (t >= n3) return;
     double s = accumulate ? forces[t] : 0.0;
     for (int q = 0; q < nslices; ++q) s += fpart[(size_t)q * stride3 + t];
+    // a skipped evaluation (inputs failed their checks) left nothing in fpart: its forces say so
+    if (guard && *guard) s = __builtin_nan("");
     forces[t] = s;
     if (copy) copy[t] = s;
 }
@@ -842,12 +846,30 @@ template hipError_t launch_slice_bwd<double>(const SliceParams<double>&, hipStre
 template hipError_t launch_slice_bwd<float>(const SliceParams<float>&, hipStream_t);
 
 hipError_t launch_fpart_reduce(long edges, long E, int nslices, const double* fpart, double* forces, int accumulate,
-                               double* copy, hipStream_t s)
+                               double* copy, hipStream_t s, const int* guard)
 {
     const long n3 = 3 * edges;
     if (n3 <= 0 || edges > E) return n3 <= 0 ? hipSuccess : hipErrorInvalidValue;
     hipLaunchKernelGGL(k_fpart_reduce, dim3((unsigned)((n3 + 255) / 256)), dim3(256), 0, s, n3, 3 * E, nslices, fpart,
-                       forces, accumulate, copy);
+                       forces, accumulate, copy, guard);
+    return hipGetLastError();
+}
+
+namespace {
+__global__ void k_poison_forces(const int* guard, double* forces, double* copy, long n)
+{
+    if (!*guard) return;
+    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (long)gridDim.x * blockDim.x) {
+        forces[t] = __builtin_nan("");
+        if (copy) copy[t] = __builtin_nan("");
+    }
+}
+}  // namespace
+hipError_t launch_poison_forces(const int* guard, double* forces, double* copy, long n, hipStream_t s)
+{
+    if (!guard || n <= 0) return hipSuccess;
+    hipLaunchKernelGGL(k_poison_forces, dim3((unsigned)std::min<long>((n + 255) / 256, 2048)), dim3(256), 0, s, guard,
+                       forces, copy, n);
     return hipGetLastError();
 }
 

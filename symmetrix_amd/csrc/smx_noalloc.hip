@@ -111,6 +111,11 @@ extern "C" int smx_reduce_forces_device_noalloc(smx_model* m, int num_atoms, con
     if (rc != SMX_OK) { smx::set_last_error(err); return rc; }
     int dev = 0;
     (void)hipGetDevice(&dev);
+    if (dev != v.device) {
+        smx::set_last_error("smx_reduce_forces_device_noalloc: the current device (" + std::to_string(dev) +
+                            ") is not the one the model lives on (" + std::to_string(v.device) + ")");
+        return SMX_EINVAL;
+    }
     unsigned char* base = g_scratch_ptr[dev];
     hipStream_t s = static_cast<hipStream_t>(stream);
     int* flag = reinterpret_cast<int*>(base + kOffFlag);

@@ -1,7 +1,8 @@
 """The benchmark configurations that the other GPU tests do not run as such: the 192-atom H/C/O case at full size
-against the oracle, the 25 002-atom water-like box through the pair style's ghost-node layout, and the capacity
-run's molecular-dynamics loop (positions moved on the device, neighbour list searched or filtered on the device,
-evaluation on device-resident arrays) at a size that takes seconds."""
+against the oracle, the 25 002-atom water-like box through the pair style's ghost-node layout, the 50 000-atom
+alloy's model on a small box against the oracle, and the capacity run's molecular-dynamics loop (positions moved on
+the device, neighbour list searched or filtered on the device, evaluation on device-resident arrays) at a size that
+takes seconds and at its full size of a million atoms."""
 import numpy as np
 import pytest
 
@@ -217,3 +218,106 @@ def test_capacity_loop_at_reduced_size(gpu, tmp_models, dtype):
     fs = max(1.0, np.abs(F).max()) if dtype == "float32" else 1.0
     assert abs(e_host.sum() - en.sum()) <= tol["E"] * abs(en.sum())
     assert np.abs(F_host - F).max() <= tol["F"] * 10 * fs
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+def test_alloy_configuration_model_against_the_oracle(gpu, tmp_models, dtype):
+    """The model of the 50 000-atom alloy workload (5 species, K = 128, hidden features up to l = 1, 10 Bessel
+    functions, r_cut 6.0 A, 256 spline points) on a 4 x 4 x 3-cell box of the same lattice, displacements and species
+    draw (192 atoms, about 80 neighbours each; the box is shorter than two cutoffs along z, so a pair also meets
+    through a periodic image), against the oracle."""
+    from oracle.oracle import OracleMACE
+    from symmetrix_amd import neighbors, systems
+    path, cfg = _model_file(tmp_models, "mp_medium", pair_dependent_radial=False)
+    assert cfg["num_channels"] == 128 and cfg["L_max"] == 1 and cfg["r_cut"] == 6.0
+    pos, cell, sp = systems.config_system("mp_medium", scale=0.004)
+    assert len(pos) == 192 and len(set(sp.tolist())) == 5
+    nl = neighbors.neighbor_list(pos, cell, cfg["r_cut"]); ea = neighbors.edge_arrays(nl, sp)
+    print(f"alloy model: {len(pos)} atoms, {len(ea['r'])} edges, {dtype}", flush=True)
+    orc = OracleMACE(path)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng = gpu(path, dtype)
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    Eo = orc.node_energies.sum()
+    assert abs(eng.node_energies.sum() - Eo) <= TOL[dtype]["E"] * abs(Eo)
+    assert np.abs(eng.node_energies - orc.node_energies).max() <= TOL[dtype]["E"] * max(1.0, np.abs(orc.node_energies).max()) * 10
+    assert np.abs(eng.node_forces - orc.node_forces).max() <= TOL[dtype]["F"]
+    F = eng.reduce_forces(len(pos), nl["j"])
+    assert np.abs(F - H.atom_forces(nl, orc.node_forces, len(pos))).max() <= TOL[dtype]["F"] * 10
+
+
+def test_capacity_configuration_at_full_size(gpu, tmp_models):
+    """The capacity configuration at its size: the l <= 1 water model on 1 000 128 atoms (4 x 4 x 4 copies of a
+    15 627-atom water box, about 5.4e7 edges), float32 features.  Device list search, evaluation, two steps with the
+    cutoff filter and one with a new search, every atom moved by N(0, 0.01^2) A per step on the device.  Before the
+    first move the 64 copies of an atom must agree in energy and force (equal up to summation order: the copies'
+    edges are the same vectors); afterwards energies and forces stay finite and the energy moves smoothly.  The
+    adjoint messages (2 KB per edge) do not fit the staging buffer, so the receiver-chunked path runs."""
+    import torch
+    from symmetrix_amd import neighbors, systems
+    free_b, _ = torch.cuda.mem_get_info()
+    if free_b < 200e9:
+        pytest.skip(f"needs about 185 GB of free HBM, {free_b / 1e9:.0f} GB are free")
+    path, cfg = _model_file(tmp_models, "off_medium", pair_dependent_radial=False)
+    dev = torch.device("cuda:0")
+    reps, n_mol = 4, 5209
+    bpos, bcell, bsp = systems.water_box(n_mol, seed=0)
+    nb = len(bpos)
+    offs = np.array([[a, b, c] for a in range(reps) for b in range(reps) for c in range(reps)], dtype=np.float64) * bcell
+    pos = (offs[:, None, :] + bpos[None, :, :]).reshape(-1, 3)
+    species = np.tile(bsp, reps ** 3).astype(np.int32)
+    cell = bcell * reps
+    N = len(pos)
+    assert N == 1000128
+    r_cut, skin = cfg["r_cut"], 0.6
+    dpos = torch.from_numpy(np.ascontiguousarray(pos)).to(dev)
+    dty = torch.from_numpy(species).to(dev)
+    del pos
+    eng = gpu(path, "float32")
+    dnl = neighbors.DeviceNeighborList()
+    stream = torch.cuda.current_stream().cuda_stream
+    out_E = torch.zeros(N, dtype=torch.float64, device=dev)
+    out_F = None
+
+    def evaluate(E):
+        nonlocal out_F
+        if out_F is None or out_F.numel() < 3 * E:
+            out_F = torch.zeros(int(3 * E * 1.02), dtype=torch.float64, device=dev)
+        p = dnl.ptr
+        eng.compute_device(N, dty.data_ptr(), p["num_neigh"], p["neigh_indices"], p["neigh_types"], p["xyz"], p["r"], E,
+                           out_E.data_ptr(), out_F.data_ptr(), stream)
+        eng.synchronize()
+        return eng.reduce_forces_device(N, p["neigh_indices"])
+
+    E = dnl.build(N, dpos.data_ptr(), dty.data_ptr(), cell, r_cut, skin=skin)
+    print(f"capacity configuration: {N} atoms, {E} edges", flush=True)
+    assert E > 5.0e7
+    F = evaluate(E)
+    free_after, total_b = torch.cuda.mem_get_info()
+    print(f"  first evaluation done, {(total_b - free_after) / 1e9:.0f} GB of HBM in use", flush=True)
+    assert (total_b - free_after) < 288e9
+    en = out_E.cpu().numpy()
+    e_rep, f_rep = en.reshape(reps ** 3, nb), F.reshape(reps ** 3, nb, 3)
+    e_scale, f_scale = np.abs(e_rep[0]).max(), np.abs(f_rep[0]).max()
+    e_dev, f_dev = np.abs(e_rep - e_rep[0]).max(), np.abs(f_rep - f_rep[0]).max()
+    print(f"  64 copies: energy differs by {e_dev:.2e} (scale {e_scale:.2f}), force by {f_dev:.2e} (scale {f_scale:.1f})", flush=True)
+    # float32 features: 1e-5 relative in energy, 1e-4 eV/A in force relative to the largest force of the box (the
+    # recipe drops hydrogens next to other molecules: forces of a hundred eV/A)
+    assert e_dev <= 2e-5 * e_scale and f_dev <= 2e-4 * max(1.0, f_scale)
+    assert np.abs(F.sum(0)).max() <= 1e-6 * N ** 0.5 * max(1.0, f_scale)     # Newton's third law
+    e_prev = en.sum()
+    gen = torch.Generator(device=dev); gen.manual_seed(0)
+    for it, search in enumerate((False, False, True)):
+        dpos.add_(torch.randn(dpos.shape, dtype=torch.float64, device=dev, generator=gen), alpha=0.01)
+        if search:
+            E = dnl.build(N, dpos.data_ptr(), dty.data_ptr(), cell, r_cut, skin=skin)
+        else:
+            E = dnl.update(dpos.data_ptr(), dty.data_ptr(), r_cut)
+        F = evaluate(E)
+        e_now = float(out_E.sum().item())
+        print(f"  step {it} ({'search' if search else 'filter'}): {E} edges, E = {e_now:.3f}", flush=True)
+        assert np.isfinite(F).all() and np.isfinite(e_now)
+        assert abs(e_now - e_prev) <= 0.05 * abs(e_prev)
+        e_prev = e_now
+    del eng, dnl, out_F, out_E, dpos, dty
+    torch.cuda.empty_cache()

@@ -31,11 +31,15 @@ def _case(f, mode, Nl, Ng, rows, nt, nn, node_i, ni, nty, nj, halo_ghost, halo_o
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("L_max,dtype", [(0, "float64"), (1, "float64"), (1, "float32")])
-def test_cpp_caller_runs_the_three_pair_style_modes(tmp_path, L_max, dtype):
+@pytest.mark.parametrize("L_max,dtype,one_table,density", [(0, "float64", False, False), (1, "float64", False, True),
+                                                            (1, "float32", False, True), (0, "float64", True, False),
+                                                            (0, "float32", True, True)])
+def test_cpp_caller_runs_the_three_pair_style_modes(tmp_path, L_max, dtype, one_table, density):
+    """`one_table`: one radial table for all species pairs, so that the channel-slice kernels run (the layer-1
+    partial forces wait for the layer-0 adjoint there, beside the ZBL and density-normalisation forces)."""
     if not os.path.exists(DRIVER):
         pytest.fail("tests/cpp/pair_modes_driver is not built: python -c 'import __graft_entry__ as g; g.build()'")
-    model = H.tiny_model(K=16, L_max=L_max, n_pts=48, seed=12, zbl=True, density=(L_max == 1))
+    model = H.tiny_model(K=16, L_max=L_max, n_pts=48, seed=12, pair=not one_table, zbl=True, density=density)
     path = H.write_model(model, tmp_path / "m.json")
     pos, cell, sp = H.small_system(36, seed=21)
     nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])

@@ -356,7 +356,13 @@ def test_calculator_energy_forces_stress(gpu, tmp_models):
     from symmetrix_amd.calc import SymmetrixCalculator
     model = H.tiny_model(K=16, L_max=1, n_pts=64, seed=21)
     path = H.write_model(model, tmp_models / "calc.json")
-    calc = SymmetrixCalculator(path)
+    calc = SymmetrixCalculator(path, species=["H", "C", "O"], num_spline_points=64)   # conversion keywords are accepted
+    # a file that is no symmetrix JSON: RuntimeError, as the reference's loader raises before it converts
+    # (symmetrix_calc.py:54-56); the message names the conversion to run
+    bad = tmp_models / "checkpoint.model"
+    bad.write_bytes(b"PK\x03\x04 not json")
+    with pytest.raises(RuntimeError, match="symmetrix_extract_mace"):
+        SymmetrixCalculator(str(bad))
     pos, cell, sp = H.small_system(14, density=0.09, seed=8)
     Z = np.array(model["atomic_numbers"])[sp]
     res = calc.compute(pos, cell, Z)
@@ -513,21 +519,36 @@ def test_receiver_chunks_of_the_layer1_adjoint_change_nothing(gpu, tmp_models, d
         eng.compute_node_energies_forces(*H.call_args(ea))
 
 
+# (L_max, dtype, one radial table for all pairs, ZBL, density normalisation).  One table and scalar hidden features
+# take the channel-slice kernels, whose layer-1 partial forces wait in the staging array for the layer-0 adjoint
+# (K = 16 is a whole number of 32-byte slices in both precisions): with ghost nodes, ZBL or the density
+# normalisation the force array has other contributions before, between and beside those two.
+MODE_CASES = [(0, "float64", False, False, False), (1, "float64", False, True, True), (0, "float32", False, True, False),
+              (1, "float32", False, True, True)]
+MODE_CASES += [(0, dt, True, zbl, dens) for dt in ("float64", "float32")
+               for zbl, dens in ((False, False), (True, False), (False, True), (True, True))]
+
+
 @pytest.mark.gpu
-@pytest.mark.parametrize("L_max,dtype", [(0, "float64"), (1, "float64"), (0, "float32"), (1, "float32")])
-def test_pair_style_modes_agree(gpu, tmp_models, L_max, dtype):
+@pytest.mark.parametrize("L_max,dtype,one_table,zbl,density", MODE_CASES)
+def test_pair_style_modes_agree(gpu, tmp_models, L_max, dtype, one_table, zbl, density):
     """The three ways the pair style feeds the engine on one rank give one answer (the reference's
     tests/test_pair_symmetrix_mace.py:28-39): owners as senders (no_domain_decomposition), ghost nodes that go
     through layer 0 (no_mpi_message_passing, one call), and ghost rows of H1 filled by a forward copy with the
-    adjoint summed back (mpi_message_passing, stage calls as pair_symmetrix_mace.cpp:372-550 issues them)."""
+    adjoint summed back (mpi_message_passing, stage calls as pair_symmetrix_mace.cpp:372-550 issues them).  The
+    first is compared with the oracle, the others with the first."""
     from symmetrix_amd import neighbors
-    model = H.tiny_model(K=16, L_max=L_max, n_pts=48, seed=12, zbl=(dtype == "float32" or L_max == 1), density=(L_max == 1))
-    path = H.write_model(model, tmp_models / f"modes{L_max}{dtype}.json")
+    model = H.tiny_model(K=16, L_max=L_max, n_pts=48, seed=12, pair=not one_table, zbl=zbl, density=density)
+    path = H.write_model(model, tmp_models / f"modes{L_max}{dtype}{int(one_table)}{int(zbl)}{int(density)}.json")
     pos, cell, sp = H.small_system(36, seed=21)
     nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
     N = len(sp)
     eng = gpu(path, dtype)
+    assert eng._int("num_radial_tables_0") == (1 if one_table else 6)
     eng.compute_node_energies_forces(*H.call_args(ea))
+    orc = _oracle()(model)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    _compare(orc, eng, dtype, names=[])
     e_ref = eng.node_energies.copy()
     f_ref = eng.reduce_forces(N, ea["neigh_indices"])
     ga = neighbors.ghost_edge_arrays(nl, sp)
@@ -541,6 +562,12 @@ def test_pair_style_modes_agree(gpu, tmp_models, L_max, dtype):
     ftol = 1e-11 if dtype == "float64" else 2e-5
     assert np.array_equal(e_g, e_ref)      # same edges in the same order for every local receiver
     assert np.abs(f_g - f_ref).max() <= ftol * max(1.0, np.abs(f_ref).max())
+    assert np.abs(f_g - H.atom_forces(nl, orc.node_forces, N)).max() <= TOL[dtype]["F"]
+    # the same call again, and after an evaluation of the owner layout in between: bit for bit
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    eng.compute_ghosted(Nl, Ng, ga["node_types"], ga["num_neigh"], ga["neigh_indices"], ga["neigh_types"], ga["xyz"], ga["r"])
+    assert np.array_equal(eng.node_energies, e_g)
+    assert np.array_equal(eng.reduce_forces(N, ga["sender_atom"], ga["receiver_atom"]), f_g)
 
     # message-passing mode: local nodes only; H1 of the ghosts copied from their owners, H1_adj summed back
     El = int(ga["num_neigh"][:Nl].sum())
@@ -653,16 +680,19 @@ def test_a_step_captured_in_a_hip_graph_replays_bitwise(gpu, tmp_models, L_max):
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("L_max,big", [(0, False), (1, False), (0, True)])
-def test_device_resident_call_checks_its_inputs_on_the_device(gpu, tmp_models, L_max, big):
+@pytest.mark.parametrize("L_max,big,one_table", [(0, False, False), (1, False, False), (0, True, False), (0, False, True)])
+def test_device_resident_call_checks_its_inputs_on_the_device(gpu, tmp_models, L_max, big, one_table):
     """Arrays handed over as device addresses are checked inside the list preparation; when a check fails, the
-    evaluation runs on emptied lists (no unchecked integer is used as an address), the node energies come back as
-    NaN and the next synchronising call raises.  Every kernel exits normally; the call after is unaffected.
-    `big`: more than 65 536 atoms, where the preparation is made of separate launches."""
+    evaluation runs on emptied lists (no unchecked integer is used as an address), node energies and edge forces come
+    back as NaN and the next synchronising call (synchronize, get_array, reduce_forces) raises.  Every kernel exits
+    normally; the call after is unaffected, also when both are replays of one captured graph.
+    `big`: more than 65 536 atoms, where the preparation is made of separate launches; `one_table`: the
+    channel-slice kernels, whose forces come out of the sum over slices."""
     import torch
     from symmetrix_amd import neighbors, systems
-    model = H.tiny_model(K=16 if big else 32, L_max=L_max, n_pts=48, seed=40 + L_max, r_cut=3.0 if big else 4.0)
-    path = H.write_model(model, tmp_models / f"guard{L_max}{int(big)}.json")
+    model = H.tiny_model(K=16 if big else 32, L_max=L_max, n_pts=48, seed=40 + L_max, r_cut=3.0 if big else 4.0,
+                         pair=not one_table)
+    path = H.write_model(model, tmp_models / f"guard{L_max}{int(big)}{int(one_table)}.json")
     if big:
         pos, cell, sp = systems.fcc_alloy((26, 26, 25), n_species=3, seed=1)     # 67 600 atoms
     else:
@@ -684,18 +714,57 @@ def test_device_resident_call_checks_its_inputs_on_the_device(gpu, tmp_models, L
     run(good)
     eng.synchronize()
     e_ref, f_ref = oE.clone(), oF.clone()
-    assert torch.isfinite(e_ref).all()
+    F_ref = eng.reduce_forces(N, ea["neigh_indices"])
+    assert torch.isfinite(e_ref).all() and torch.isfinite(f_ref).all()
     bad_cases = {"sender row": ("neigh_indices", 5, N + 3), "edge species": ("neigh_types", 0, 3),
                  "node species": ("node_types", 1, -1), "counts": ("num_neigh", 0, int(ea["num_neigh"][0]) + 1),
                  "edge length": ("r", 3, 2.0 * model["r_cut"])}
-    for what, (key, pos_, value) in bad_cases.items():
+    for n_case, (what, (key, pos_, value)) in enumerate(bad_cases.items()):
         d = dict(good); d[key] = good[key].clone(); d[key][pos_] = value
         print(f"bad {what} (L_max {L_max}, {N} atoms)", flush=True)
+        oF.zero_()
         run(d)
         assert torch.isnan(oE).all(), what
+        assert torch.isnan(oF).all(), what
         with pytest.raises(ValueError):
-            eng.synchronize()
+            if n_case % 2 == 0:
+                eng.synchronize()
+            else:
+                eng.reduce_forces(N, ea["neigh_indices"])     # the per-atom sums of NaN forces are not handed out silently
         eng.synchronize()                       # reported once
         run(good)
         eng.synchronize()
         assert torch.equal(oE, e_ref) and torch.equal(oF, f_ref), what
+        assert np.array_equal(eng.reduce_forces(N, ea["neigh_indices"]), F_ref)
+    if big:
+        return
+    # one captured graph, replayed on bad and then on good inputs: a skipped replay leaves nothing behind
+    live = {k: good[k].clone() for k in names}
+    s = torch.cuda.Stream()
+
+    def step():
+        eng.compute_device(N, *[live[k].data_ptr() for k in names], E, oE.data_ptr(), oF.data_ptr(), s.cuda_stream)
+
+    with torch.cuda.stream(s):
+        step()
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g, stream=s):
+        step()
+    torch.cuda.synchronize()
+    for rep in range(2):
+        live["neigh_indices"][5] = N + 3
+        torch.cuda.synchronize()
+        print(f"graph replay {rep}: bad, then good", flush=True)
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.isnan(oE).all() and torch.isnan(oF).all()
+        live["neigh_indices"].copy_(good["neigh_indices"])
+        oE.zero_(); oF.zero_()
+        torch.cuda.synchronize()
+        g.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(oE, e_ref) and torch.equal(oF, f_ref)
+        with pytest.raises(ValueError):
+            eng.synchronize()                   # the skipped replay is still reported, once
+        eng.synchronize()

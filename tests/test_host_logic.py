@@ -186,3 +186,20 @@ def test_neighbor_list_of_atoms_outside_the_cell(triclinic):
     assert np.array_equal(d["i"], e["i"]) and np.array_equal(d["j"], e["j"]) and np.array_equal(d["S"], e["S"])
     w, off = neighbors.wrap_positions(moved, cell)
     assert np.allclose(w + off @ cell, moved, atol=1e-12) and np.all((w @ np.linalg.inv(cell) > -1e-9) & (w @ np.linalg.inv(cell) < 1 + 1e-9))
+
+
+def test_calculator_keeps_the_reference_signature():
+    """symmetrix_calc.py:39: Symmetrix(model_file, dtype="float64", use_kokkos=True, **kwargs), and the keywords it
+    forwards to the conversion of a torch checkpoint (:58-61) are accepted."""
+    import inspect
+    from symmetrix_amd.calc import Symmetrix, SymmetrixCalculator
+    for cls in (Symmetrix, SymmetrixCalculator):
+        sig = inspect.signature(cls.__init__)
+        names = list(sig.parameters)
+        assert names[:4] == ["self", "model_file", "dtype", "use_kokkos"]
+        assert sig.parameters["dtype"].default == "float64" and sig.parameters["use_kokkos"].default is True
+        assert any(p.kind is inspect.Parameter.VAR_KEYWORD for p in sig.parameters.values())
+    assert SymmetrixCalculator.implemented_properties == ["energy", "free_energy", "energies", "forces", "stress"]
+    assert SymmetrixCalculator.EXTRACT_KEYWORDS == ("species", "head", "num_spline_points")
+    with pytest.raises(ValueError):
+        SymmetrixCalculator("x.json", dtype="float16")

@@ -244,7 +244,7 @@ def run_capacity(args):
         for k, v in eng.stage_times().items():
             acc[k] = acc.get(k, 0.0) + v / 2
     eng.set_profiling(False)
-    n_LM, n_e, s_b = (L_max + 1) ** 2, 16 if L_max == 0 else 40, 8 if args.dtype == "float64" else 4
+    n_LM, n_e, s_b = (L_max + 1) ** 2, {0: 16, 1: 40, 2: 71}[L_max], 8 if args.dtype == "float64" else 4
     # When the adjoint messages exceed the staging buffer, the layer-1 adjoint and the sender-side sum alternate per
     # receiver chunk inside one stage: the roofline then prices both kernels' bytes against the stage's time.
     chunked = acc.get("sender_reduce", 0.0) < 0.01 * acc.get("agg1_bwd", 1.0)
@@ -288,7 +288,7 @@ def main():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="off_small", choices=["tiny", "off_small", "off_medium", "mp_medium", "water_capacity"])
+    ap.add_argument("--workload", default="off_small", choices=["tiny", "off_small", "off_medium", "off_medium_l2", "mp_medium", "water_capacity"])
     ap.add_argument("--atoms", type=int, default=1000000, help="water_capacity: target atom count")
     ap.add_argument("--rebuild-every", type=int, default=10, help="water_capacity: steps between neighbour searches")
     ap.add_argument("--staging-gb", type=float, default=0.0,
@@ -424,7 +424,7 @@ def main():
         res = run_mode(dtype, steps, warmup)
         K, L_max = cfg["num_channels"], cfg["L_max"]
         n_LM = (L_max + 1) ** 2
-        n_e = 16 if L_max == 0 else 40
+        n_e = {0: 16, 1: 40, 2: 71}[L_max]
         s_bytes = 8 if dtype == "float64" else 4
 
         def stage_bytes(k):   # layer-0 stages run over all nodes and edges, layer-1 stages over the local ones

@@ -219,7 +219,7 @@ HostModel load_host_model(const std::string& path)
     if ((int)m.atomic_numbers.size() != T || (int)m.atomic_energies.size() != T)
         throw JsonError("model file: atomic_numbers/atomic_energies do not have num_elements entries");
     if (m.l_max != 3) unsupported("l_max = " + std::to_string(m.l_max) + " (the harmonics kernels implement l_max = 3, as the reference's extractor requires)");
-    if (m.L_max < 0 || m.L_max > 1) unsupported("L_max = " + std::to_string(m.L_max) + " (device kernels exist for hidden features up to L_max = 1)");
+    if (m.L_max < 0 || m.L_max > 2) unsupported("L_max = " + std::to_string(m.L_max) + " (device kernels exist for hidden features up to L_max = 2)");
 
     // ZBL, mace.cpp:922-930
     m.has_zbl = file.at("has_zbl").as_bool();

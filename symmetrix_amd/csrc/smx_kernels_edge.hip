@@ -55,7 +55,7 @@ struct BwdSteps {
     static constexpr int group(int p)
     {
         if (NARROW) return PT::l2(p) == 0 ? (rows(p) < 3 ? rows(p) : 3) : 1;
-        return PT::l2(p) == 0 ? rows(p) : 3;
+        return PT::l2(p) == 0 ? rows(p) : (PT::l2(p) == 1 ? 3 : 1);
     }
     static constexpr int groups(int p) { return (rows(p) + group(p) - 1) / group(p); }
     static constexpr int count()
@@ -143,8 +143,10 @@ __device__ __forceinline__ BlockEntry block_entry(int b, int NB, const int* cg_s
 }
 
 // ---------------------------------------------------------------------------
+// (Hidden features up to l = 2: 17 paths and 71 sums per channel.  Those instantiations take one block per CU, so
+// that a wavefront has the whole register file of its SIMD.)
 template <typename F, int LMAXH, int CPL, int EC>
-__global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const int num_terms)
+__global__ __launch_bounds__(256, LMAXH >= 2 ? 1 : 2) void k_agg_fwd(const AggParams<F> a, const int num_terms)
 {
     using PT = Paths<LMAXH>;
     using WL = WaveLds<F, LMAXH, false>;
@@ -239,7 +241,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
         // row of an edge.  In single precision those of the next edge are requested while the current edge is
         // worked on (AHEAD).  In double precision there are registers for half of that at most (HALF: the first
         // five paths and the sender row requested an edge ahead, the other five at the start of the edge).
-        constexpr bool AHEAD = sizeof(F) == 4 && (CPL == 1 || LMAXH == 0);
+        constexpr bool AHEAD = sizeof(F) == 4 && (CPL == 1 || LMAXH == 0) && LMAXH <= 1;
         constexpr bool HALF = false;   // measured slower than requesting all ten at the start of the edge (10.4 against 9.1 ms)
         constexpr int PA = HALF ? P / 2 : P;     // paths of the first part
         Vec<F, 4> cf[P][CPL];
@@ -375,7 +377,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_fwd(const AggParams<F> a, const 
 // With more than one channel group each group writes its share
 // of the force to fpart[group][edge][3]; the caller adds the groups up.
 template <typename F, int LMAXH, int CPL, int EC>
-__global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const int num_terms)
+__global__ __launch_bounds__(256, LMAXH >= 2 ? 1 : 2) void k_agg_bwd(const AggParams<F> a, const int num_terms)
 {
     using PT = Paths<LMAXH>;
     using WL = WaveLds<F, LMAXH, true>;
@@ -513,7 +515,7 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
         // Spline coefficients of one edge: P x CPL 16-byte loads, contiguous across the lanes for one path.  In single
         // precision the next edge's coefficients are requested while the current edge is worked on (40
         // registers in flight); in double precision they are requested together at the start of the edge.
-        constexpr bool AHEAD = sizeof(F) == 4;
+        constexpr bool AHEAD = sizeof(F) == 4 && LMAXH <= 1;
         Vec<F, 4> cf[P][CPL];
         auto load_cf = [&](int le_) {
             const int row = __builtin_amdgcn_readfirstlane(rows[le_]);
@@ -565,10 +567,10 @@ __global__ __launch_bounds__(256, 2) void k_agg_bwd(const AggParams<F> a, const 
                 Vec<F, 4> buf[LOOKAHEAD ? 2 : 1][ST::MAXLEN];
                 F u[CPL][2 * LMAXH + 1][3];
                 auto load_step = [&](auto sc, Vec<F, 4>* dst) {
-                    constexpr int s = decltype(sc)::value, p = ST::path(s), n2 = 2 * PT::l2(p) + 1;
+                    constexpr int s = decltype(sc)::value, p = ST::path(s), n2 = 2 * PT::l2(p) + 1, len = ST::len(s);
                     const F* B4 = Bs + boffs + (PT::boff(p) + ST::m0(s) * n2) * 4;
 #pragma unroll
-                    for (int q = 0; q < ST::len(s); ++q) dst[q] = ldv<F, 4>(B4 + 4 * q);
+                    for (int q = 0; q < len; ++q) dst[q] = ldv<F, 4>(B4 + 4 * q);
                 };
                 if constexpr (LOOKAHEAD) load_step(std::integral_constant<int, 0>{}, buf[0]);
                 static_for<0, ST::count()>([&](auto sc) {
@@ -686,7 +688,8 @@ hipError_t launch_agg_sel(const AggParams<F>& p, hipStream_t s)
 {
     // edges per chunk; the double-precision forward kernel of the ten-path list takes eight so that two blocks with
     // their coefficient buffers fit a CU
-    constexpr int EC = LMAXH == 0 ? 16 : (BWD ? (sizeof(F) == 4 ? 8 : 4) : (sizeof(F) == 8 ? 8 : 16));
+    // (l = 2 hidden features: the coupling block has 243 entries per edge, four edges of the adjoint fill the LDS share of a wavefront)
+    constexpr int EC = LMAXH == 0 ? 16 : (BWD ? (sizeof(F) == 4 && LMAXH == 1 ? 8 : 4) : (sizeof(F) == 8 ? 8 : 16));
     // two channels per lane exist for the four-path list only (the ten-path kernels have no registers for them)
     if constexpr (LMAXH == 0) {
         if (agg_cpl<F, LMAXH, BWD>(p.K) == 2) return launch_agg_t<F, LMAXH, 2, EC, BWD>(p, s);
@@ -701,6 +704,7 @@ hipError_t launch_agg_fwd(int L_max_H, const AggParams<F>& p, hipStream_t s)
 {
     if (L_max_H == 0) return launch_agg_sel<F, 0, false>(p, s);
     if (L_max_H == 1) return launch_agg_sel<F, 1, false>(p, s);
+    if (L_max_H == 2) return launch_agg_sel<F, 2, false>(p, s);
     return hipErrorInvalidValue;
 }
 template <typename F>
@@ -708,12 +712,13 @@ hipError_t launch_agg_bwd(int L_max_H, const AggParams<F>& p, hipStream_t s)
 {
     if (L_max_H == 0) return launch_agg_sel<F, 0, true>(p, s);
     if (L_max_H == 1) return launch_agg_sel<F, 1, true>(p, s);
+    if (L_max_H == 2) return launch_agg_sel<F, 2, true>(p, s);
     return hipErrorInvalidValue;
 }
 template <typename F>
 int agg_bwd_groups(int L_max_H, int K)
 {
-    const int cpl = L_max_H == 0 ? agg_cpl<F, 0, true>(K) : agg_cpl<F, 1, true>(K);
+    const int cpl = L_max_H == 0 ? agg_cpl<F, 0, true>(K) : 1;
     return (K + 64 * cpl - 1) / (64 * cpl);
 }
 // This file is compiled four times (SMX_EDGE_PART = 0..3), one object per

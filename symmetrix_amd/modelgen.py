@@ -264,6 +264,8 @@ CONFIGS = {
     "tiny": dict(atomic_numbers=[1, 6, 8], num_channels=32, L_max=0, r_cut=5.0, n_bessel=8),
     "off_small": dict(atomic_numbers=[1, 6, 7, 8], num_channels=96, L_max=0, r_cut=4.5, n_bessel=8),
     "off_medium": dict(atomic_numbers=[1, 6, 7, 8], num_channels=128, L_max=1, r_cut=5.0, n_bessel=8),
+    # hidden features up to l = 2 (128x0e+128x1o+128x2e), otherwise the model above
+    "off_medium_l2": dict(atomic_numbers=[1, 6, 7, 8], num_channels=128, L_max=2, r_cut=5.0, n_bessel=8),
     "mp_medium": dict(atomic_numbers=[13, 22, 26, 28, 29], num_channels=128, L_max=1, r_cut=6.0,
                       n_bessel=10, avg_num_neighbors=80.0),
 }

@@ -89,7 +89,7 @@ def config_system(name, seed=0, scale=1.0):
         return random_box(max(8, int(192 * scale)), 0.10, [1 / 3, 1 / 3, 1 / 3], seed=seed)
     if name == "off_small":       # 3000 atoms, H/C/N/O 0.5/0.3/0.1/0.1
         return random_box(max(8, int(3000 * scale)), 0.10, [0.5, 0.3, 0.1, 0.1], seed=seed)
-    if name == "off_medium":      # 25 002 atoms water-like (8334 molecules)
+    if name in ("off_medium", "off_medium_l2"):      # 25 002 atoms water-like (8334 molecules)
         return water_box(max(4, int(8334 * scale)), seed=seed)
     if name == "mp_medium":       # 25 x 25 x 20 fcc cells = 50 000 atoms
         s = scale ** (1.0 / 3.0)

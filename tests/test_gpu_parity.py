@@ -54,6 +54,8 @@ CASES = [
     (20, 0, 17, True), (64, 1, 30, False), (128, 0, 30, True),
     # wider than one block of channels: several channel groups, column tiles and slices
     (256, 0, 20, False), (192, 1, 16, False),
+    # hidden features up to l = 2 (128x0e+128x1o+128x2e and the like): 17 paths, 9 polynomials
+    (16, 2, 30, True), (128, 2, 20, False), (40, 2, 26, True),
 ]
 
 
@@ -158,7 +160,8 @@ def test_golden_fixture(gpu, dtype):
 
 @pytest.mark.parametrize("dtype", ["float64", "float32"])
 @pytest.mark.parametrize("K,L_max,natoms,zbl,density", [(32, 0, 40, True, False), (96, 0, 48, True, True),
-                                                        (48, 1, 30, True, True), (128, 1, 24, False, True)])
+                                                        (48, 1, 30, True, True), (128, 1, 24, False, True),
+                                                        (32, 2, 22, True, True)])
 def test_pair_terms_match_oracle(gpu, tmp_models, K, L_max, natoms, zbl, density, dtype):
     """Models with ZBL repulsion and / or density-normalised layers (mace.cpp:27-35, 273-346, 681-757)."""
     model = H.tiny_model(K=K, L_max=L_max, n_pts=64, seed=K + L_max, pair=(K != 96), zbl=zbl, density=density)

@@ -32,7 +32,7 @@ def numerical_gradient(f, x, h=1e-4):
     return g
 
 
-@pytest.fixture(scope="module", params=[0, 1], ids=["Lmax0", "Lmax1"])
+@pytest.fixture(scope="module", params=[0, 1, 2], ids=["Lmax0", "Lmax1", "Lmax2"])
 def setup(request):
     model = H.tiny_model(K=3, L_max=request.param, n_pts=40)
     orc = OracleMACE(model)
@@ -175,7 +175,7 @@ def test_total_energy_per_edge_forces(setup):
 # ---------------------------------------------------------------------------
 # ZBL and density normalisation (mace.cpp:27-35, 273-346, 681-757).  The reference holds no stored value for
 # these stages that can be used here; they are pinned by what the mathematics fixes.
-@pytest.mark.parametrize("L_max", [0, 1])
+@pytest.mark.parametrize("L_max", [0, 1, 2])
 def test_pair_terms_forces_are_the_energy_gradient(L_max):
     """Whole pipeline with ZBL and both normalisations switched on: node_forces[ij] = -dE/dxyz_ij."""
     model = H.tiny_model(K=3, L_max=L_max, n_pts=40, zbl=True, density=True)

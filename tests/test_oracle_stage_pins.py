@@ -43,7 +43,7 @@ def _elementary(rows, cols, r, c):
     return E.ravel().tolist()
 
 
-@pytest.fixture(scope="module", params=[0, 1], ids=["Lmax0", "Lmax1"])
+@pytest.fixture(scope="module", params=[0, 1, 2], ids=["Lmax0", "Lmax1", "Lmax2"])
 def base(request):
     return H.tiny_model(K=K, L_max=request.param, n_pts=24, seed=5)
 
@@ -243,7 +243,7 @@ def test_H1_weights_are_row_major_kp_k_per_l(base):
     block l, other columns zero.  Fails under a transposed read or a wrong block offset."""
     model = copy.deepcopy(base)
     L_max = model["L_max"]; nLM = (L_max + 1) ** 2
-    pick = {l: ((2 * l + 1) % K, (l + 3) % K) for l in range(L_max + 1)}
+    pick = {l: ((2 * l + 1) % K, (2 * l + 2) % K) for l in range(L_max + 1)}
     assert all(a != b for a, b in pick.values())
     model["H1_weights"] = sum((_elementary(K, K, *pick[l]) for l in range(L_max + 1)), [])
     orc = OracleMACE(model)
@@ -315,7 +315,7 @@ def test_Phi1_of_a_single_unit_sender_feature(base):
     geo = (N, ea["node_types"], ea["num_neigh"], ea["neigh_types"])
     orc.compute_Y(ea["xyz"]); orc.compute_R1(*geo, ea["r"])
     j_s, lm2_s, k_s = int(ea["neigh_indices"][3]), 2, 1
-    H1 = np.zeros((N, 4, K)); H1[j_s, lm2_s, k_s] = 1.0
+    H1 = np.zeros((N, (model["L_max"] + 1) ** 2, K)); H1[j_s, lm2_s, k_s] = 1.0
     orc.H1 = H1; orc.compute_Phi1(N, ea["num_neigh"], ea["neigh_indices"])
     Y = orc.Y.reshape(-1, 16); R1 = orc.R1.reshape(-1, P, K)
     recv = _receiver_of_edge(ea)

@@ -550,7 +550,7 @@ def main():
         del m2, m3
         torch.cuda.empty_cache()
         free_b, _ = torch.cuda.mem_get_info()
-        if free_b > 200e9:
+        if free_b > 200e9 and not args.no_cpu:
             cargs = argparse.Namespace(**vars(args))
             cargs.steps, cargs.warmup, cargs.dtype, cargs.rebuild_every = 20, 2, "float32", 10
             line["capacity_config"] = run_capacity(cargs)

@@ -267,15 +267,16 @@ __global__ __launch_bounds__(256, LMAXH >= 2 ? 1 : 2) void k_agg_fwd(const AggPa
         if ((AHEAD || HALF) && nE > 0) request(0, c0, cA, true);
         F w[P][CPL][2 * LMAXH + 1];   // radial value times sender feature per path and sender component
         auto products = [&](F x, auto first, auto last) {
-#pragma unroll
-            for (int q = decltype(first)::value; q < decltype(last)::value; ++q)
+            static_for<decltype(first)::value, decltype(last)::value>([&](auto qc) {
+                constexpr int q = decltype(qc)::value, l2 = PT::l2(q);
 #pragma unroll
                 for (int c = 0; c < CPL; ++c) {
                     const Vec<F, 4> k4 = cf[q][c];
                     const F R = k4.v[0] + x * (k4.v[1] + x * (k4.v[2] + x * k4.v[3]));
 #pragma unroll
-                    for (int m2 = 0; m2 < 2 * PT::l2(q) + 1; ++m2) w[q][c][m2] = R * H[PT::l2(q) * PT::l2(q) + m2].v[c];
+                    for (int m2 = 0; m2 < 2 * l2 + 1; ++m2) w[q][c][m2] = R * H[l2 * l2 + m2].v[c];
                 }
+            });
         };
         // coefficient buffer of this wavefront: [PRE paths][2 halves][64 lanes] 16-byte words
         unsigned char* pre = smem + WL::lists(num_terms) + 4 * WL::per_wave(EC) + (size_t)wave * WL::prefetch_per_wave();
@@ -567,8 +568,11 @@ __global__ __launch_bounds__(256, LMAXH >= 2 ? 1 : 2) void k_agg_bwd(const AggPa
                 Vec<F, 4> buf[LOOKAHEAD ? 2 : 1][ST::MAXLEN];
                 F u[CPL][2 * LMAXH + 1][3];
                 auto load_step = [&](auto sc, Vec<F, 4>* dst) {
+                    // (every table lookup lands in a constexpr variable: left to the optimizer, the path tables of the
+                    // l = 2 instantiation stay behind as loops that run on the device)
                     constexpr int s = decltype(sc)::value, p = ST::path(s), n2 = 2 * PT::l2(p) + 1, len = ST::len(s);
-                    const F* B4 = Bs + boffs + (PT::boff(p) + ST::m0(s) * n2) * 4;
+                    constexpr int first = (PT::boff(p) + ST::m0(s) * n2) * 4;
+                    const F* B4 = Bs + boffs + first;
 #pragma unroll
                     for (int q = 0; q < len; ++q) dst[q] = ldv<F, 4>(B4 + 4 * q);
                 };
@@ -643,8 +647,14 @@ __global__ __launch_bounds__(256, LMAXH >= 2 ? 1 : 2) void k_agg_bwd(const AggPa
                 else { f[0] = fx; f[1] = fy; f[2] = fz; }
             }
         };
-        for (int le = 0; le + 1 < nE; ++le) edge(le, std::true_type{});
-        if (nE > 0) edge(nE - 1, std::false_type{});
+        if constexpr (AHEAD) {
+            for (int le = 0; le + 1 < nE; ++le) edge(le, std::true_type{});
+            if (nE > 0) edge(nE - 1, std::false_type{});
+        } else {
+            // one copy of the edge's code: the unrolled walk of the coupling block is tens of KB of instructions, and
+            // a chunk's whole code path has to stay inside the instruction cache
+            for (int le = 0; le < nE; ++le) edge(le, std::false_type{});
+        }
     }
 }
 

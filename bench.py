@@ -97,6 +97,19 @@ def dense_flops(stage, N, K, n_LM, n_e):
     return per_atom[stage] * N
 
 
+VALU_PEAK = 78.6e12   # vector multiply-add peak of MI355X, flop/s, double or (unpacked) single precision
+
+
+def edge_valu_flops(stage, E, K, L_max):
+    """Multiply-adds the edge stages need by the algorithm (2 flops each), per evaluation: 2 * 16 * K per edge for
+    the layer-0 aggregation, 2 * n_r * K for layer 1 (n_r products of a harmonic with a sender component: 16, 88 or
+    243 for hidden features up to l = 0, 1, 2), and about 3.5 times as much for each adjoint (edge force and sender
+    message).  Radial splines and harmonics come on top and are not counted."""
+    n_r = {0: 16, 1: 88, 2: 243}[L_max]
+    per_edge = {"agg0_fwd": 2 * 16 * K, "agg1_fwd": 2 * n_r * K, "agg0_bwd": 7 * 16 * K, "agg1_bwd": 7 * n_r * K}
+    return per_edge.get(stage, 0) * E
+
+
 def measured_mfma_busy(workload, dtype, stage):
     """Matrix-pipe busy share of the kernel behind a dense stage (SQ_VALU_MFMA_BUSY_CYCLES over SIMD cycles), from
     the rocprofv3 counter summary kept under profiles/; None when the file has no line for that kernel."""
@@ -451,6 +464,12 @@ def main():
             stages_rl[k] = {"kernel": kern_k, "algorithmic_bytes": b_k, "kernel_ms": ms_k, "achieved": ach,
                             "frac": ach / (HBM_PEAK / 1e9),
                             "traffic": measured_traffic(prof_name, dtype, k, kern_k) if profiled else None}
+            fl = edge_valu_flops(k, E if k.startswith("agg0") else E_local, K, L_max)
+            if fl:
+                # the same stage against the vector arithmetic it cannot do without (the bound that bites: about
+                # 20 bytes of HBM data per edge and channel against one to several hundred multiply-adds)
+                stages_rl[k]["valu"] = {"flops": fl, "achieved_tflops": fl / (ms_k * 1e-3) / 1e12,
+                                        "peak_tflops": VALU_PEAK / 1e12, "frac": fl / (ms_k * 1e-3) / VALU_PEAK}
         mfma = {}
         for k in ("A0_lin", "H1", "A1", "H2", "rev_A1", "rev_H1", "rev_A0_lin"):
             ms_k = res["stages"].get(k, 0.0)

@@ -805,6 +805,7 @@ struct Engine : EngineBase {
         p.H2 = H2.p; p.H2_adj = H2_adj.p; p.H1_adj = H1_adj.p; p.M1_adj = M1_adj.p;
         p.node_energies = node_energies.p; p.zero_energies = zero_energies ? 1 : 0; p.energies_copy = energies_copy;
         p.guard = guard_live(); p.guard_clear = guard_status;
+        p.guard_forces = guard_status ? node_forces.p : nullptr; p.guard_forces_n = guard_status ? (long)node_forces.n : 0;
         HIPCHK(launch_tail_fused<F>(p, stream));
         if (guard_status && rows > 0) guard_clear_enqueued = true;
         energies_copy = nullptr;
@@ -819,7 +820,8 @@ struct Engine : EngineBase {
         if (rows < N || H2.n < (size_t)N * k) throw Error(SMX_EINVAL, "readouts called before H1 and H2 exist for these nodes");
         HIPCHK(launch_readout_fused<F>(N, rows, k, nlm, node_types, E0.p, ro1.p, ro2_w1.p, ro2_w2.p, hm.readout_2_scale,
                                        H1.p, H2.p, H2_adj.p, H1_adj.p, node_energies.p, zero_energies ? 1 : 0,
-                                       energies_copy, guard_live(), guard_status, stream));
+                                       energies_copy, guard_live(), guard_status, guard_status ? node_forces.p : nullptr,
+                                       guard_status ? (long)node_forces.n : 0, stream));
         if (guard_status && rows > 0) guard_clear_enqueued = true;
         energies_copy = nullptr;
     }
@@ -869,7 +871,7 @@ struct Engine : EngineBase {
                 carried_edges = E1;
                 carried_accumulate = zero_dxyz ? 0 : 1;
             } else {
-                HIPCHK(launch_fpart_reduce(E1, E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
+                HIPCHK(launch_fpart_reduce(E1, E, S, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream, guard_live()));
             }
             stage_end(ST_FSUM1);
         } else {
@@ -890,7 +892,6 @@ struct Engine : EngineBase {
         }
         stage_end(ST_SRED);
     }
-    bool forces_poisoned = false;   // the last force launch of compute() looked at the guard itself
     bool carry_forces = false;      // compute() lets the layer-1 partial forces wait for the layer-0 adjoint
     long carried_edges = 0;         // ... and the stage left them in fpart for edges [0, carried_edges)
     int carried_accumulate = 1;
@@ -940,7 +941,7 @@ struct Engine : EngineBase {
         stage_end(ST_AGG1B);
         stage_begin(ST_FSUM1);
         if (groups > 1)
-            HIPCHK(launch_fpart_reduce(E1, E, groups, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream));
+            HIPCHK(launch_fpart_reduce(E1, E, groups, fpart.p, node_forces.p, zero_dxyz ? 0 : 1, nullptr, stream, guard_live()));
         stage_end(ST_FSUM1);
         stage_begin(ST_SRED);
         stage_end(ST_SRED);
@@ -968,7 +969,6 @@ struct Engine : EngineBase {
             stage_begin(ST_FSUM0);
             HIPCHK(launch_fpart_reduce(E, E, S, fpart.p, node_forces.p, accumulate, forces_copy, stream, guard_live()));
             forces_copy = nullptr;
-            forces_poisoned = true;
             stage_end(ST_FSUM0);
             return;
         }
@@ -989,7 +989,7 @@ struct Engine : EngineBase {
         stage_end(st_kernel);
         if (groups > 1) {
             stage_begin(st_sum);
-            HIPCHK(launch_fpart_reduce(edges, E, groups, fpart.p, node_forces.p, p.accumulate_forces, nullptr, stream));
+            HIPCHK(launch_fpart_reduce(edges, E, groups, fpart.p, node_forces.p, p.accumulate_forces, nullptr, stream, guard_live()));
             stage_end(st_sum);
         }
     }
@@ -1041,7 +1041,7 @@ struct Engine : EngineBase {
         // range checks come before any kernel that uses these integers as indices: host arrays are checked with a
         // read-back below; device arrays inside the list preparation, whose last launch empties the lists when a
         // check failed (input_guard)
-        guard_status = nullptr; guard_clear_enqueued = false; forces_poisoned = false;
+        guard_status = nullptr; guard_clear_enqueued = false;
         if (on_device) {
             guard_status = flags.p + 2;
             ++device_calls;
@@ -1137,8 +1137,8 @@ struct Engine : EngineBase {
         st_scale(0, N, true);
         stage_begin(ST_REVA0LIN); st_A0_lin(N, true, fuse0); stage_end(ST_REVA0LIN);
         st_agg0_bwd(N);
-        // a skipped evaluation (inputs failed the checks on the device) wrote no force: NaN says so, as for the energies
-        if (guard_status && !forces_poisoned) HIPCHK(launch_poison_forces(guard_live(), node_forces.p, nullptr, 3 * E, stream));
+        // (a skipped evaluation: the readout launch has filled the forces with NaN, and every sum of partial forces
+        // after it looks at the guard itself)
         if (guard_status && !guard_clear_enqueued) HIPCHK(launch_fill<int>(guard_status, 1, 0, stream));
 
         if (energies_copy) HIPCHK(hipMemcpyAsync(energies_copy, node_energies.p, (size_t)N1 * sizeof(double), hipMemcpyDeviceToDevice, stream));

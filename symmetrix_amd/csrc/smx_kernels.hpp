@@ -90,8 +90,6 @@ template <typename F> hipError_t launch_slice_bwd(const SliceParams<F>& p, hipSt
 // `guard`, if not null and raised, makes every force NaN instead: the evaluation was skipped)
 hipError_t launch_fpart_reduce(long edges, long E, int nslices, const double* fpart, double* forces, int accumulate,
                                double* copy, hipStream_t s, const int* guard = nullptr);
-// forces[0, n) and copy[0, n) (may be null) become NaN when *guard is raised
-hipError_t launch_poison_forces(const int* guard, double* forces, double* copy, long n, hipStream_t s);
 
 // H1_adj[j] (+)= sum over edges with sender j of msg[e], in ascending edge order.
 // H_adj[j] (+)= sum of msg[e - e_lo] over the edges e of sender j with e_lo <= e < e_hi, in ascending edge order
@@ -270,12 +268,14 @@ bool gemm_scaled_operand_ok(int Kd, int Nn, size_t elem);
 // ---------------------------------------------------------------------------
 // Readout tail (MACE::compute_readouts, mace.cpp:876-903) in one launch: node_energies[i] (+)= E0[type] +
 // w1 . H1[i, l=0] + MLP_{K->16->1}(H2[i]) with W1[16][K], H2_adj = gradient of the network, H1_adj[rows][num_LM][K]
-// seeded with w1 in the scalar block of the first N rows and zero elsewhere.
+// seeded with w1 in the scalar block of the first N rows and zero elsewhere.  guard / guard_clear / guard_forces: as
+// in TailParams below.
 template <typename F>
 hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,
                                 const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
-                                double* energies_copy, const int* guard, int* guard_clear, hipStream_t s);
+                                double* energies_copy, const int* guard, int* guard_clear, double* guard_forces,
+                                long guard_forces_n, hipStream_t s);
 // H2 (mace.cpp:820-845), the readout tail and reverse_H2 (mace.cpp:847-874) in one launch; K a multiple of 16
 // up to 128 (tail_fused_ok).  Atoms grouped by species (perm, tstart); H1_adj [rows][num_LM][K] is written
 // whole (seed plus the adjoint of H2 in the scalar block, zero elsewhere), M1_adj [N][K] too.
@@ -291,6 +291,8 @@ struct TailParams {
     double* node_energies; int zero_energies; double* energies_copy;
     const int* guard;        // live status of a device-resident evaluation (or null): raised -> energies are NaN
     int* guard_clear;        // the word the input checks of the next evaluation raise (or null): cleared here
+    double* guard_forces;    // raised guard: these guard_forces_n edge-force components become NaN as well (the
+    long guard_forces_n;     // adjoint kernels of a skipped evaluation see no edges and write none)
 };
 bool tail_fused_ok(int K);
 template <typename F> hipError_t launch_tail_fused(const TailParams<F>& p, hipStream_t s);

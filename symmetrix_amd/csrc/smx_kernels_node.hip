@@ -714,18 +714,21 @@ __global__ __launch_bounds__(256) void k_readout_fused(int N, int rows, int K, i
                                                        const double* w2, double scale, const F* H1, const double* H2,
                                                        double* H2_adj, F* H1_adj, double* node_energies,
                                                        int zero_energies, double* energies_copy, const int* guard,
-                                                       int* guard_clear)
+                                                       int* guard_clear, double* guard_forces, long guard_forces_n)
 {
     extern __shared__ double rsm[];
     // every reader of the check word has run (the sender lists come before the readout): clean for the next evaluation
     if (guard_clear && blockIdx.x == 0 && threadIdx.x == 0) *guard_clear = 0;
     if (guard && *guard) {
-        // unchecked species indices: no table lookup, the energies say so
+        // unchecked species indices: no table lookup, the energies say so; so do the edge forces, which the
+        // adjoint kernels of this evaluation will not touch (they see no edges)
         const int i = blockIdx.x * 16 + (threadIdx.x >> 4);
         if ((threadIdx.x & 15) == 0 && i < N) {
             node_energies[i] = __builtin_nan("");
             if (energies_copy) energies_copy[i] = __builtin_nan("");
         }
+        for (long t = (long)blockIdx.x * 256 + threadIdx.x; t < guard_forces_n; t += (long)gridDim.x * 256)
+            guard_forces[t] = __builtin_nan("");
         return;
     }
     const int ldw = K + 1;                 // rows of W1 start two banks apart
@@ -816,6 +819,9 @@ __global__ __launch_bounds__(TAIL_BLOCK) void k_tail_fused(const TailParams<F> p
             p.node_energies[i] = __builtin_nan("");
             if (p.energies_copy) p.energies_copy[i] = __builtin_nan("");
         }
+        // ... and so do the edge forces, which the adjoint kernels will not touch (they see no edges)
+        for (long t = (long)blockIdx.x * TAIL_BLOCK + tid; t < p.guard_forces_n; t += (long)gridDim.x * TAIL_BLOCK)
+            p.guard_forces[t] = __builtin_nan("");
         return;
     }
     // rows beyond the atoms (ghost rows of H1_adj) are cleared by all blocks together
@@ -983,7 +989,8 @@ template <typename F>
 hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* node_types, const double* atomic_energies,
                                 const double* w1, const double* W1, const double* w2, double scale, const F* H1,
                                 const double* H2, double* H2_adj, F* H1_adj, double* node_energies, int zero_energies,
-                                double* energies_copy, const int* guard, int* guard_clear, hipStream_t s)
+                                double* energies_copy, const int* guard, int* guard_clear, double* guard_forces,
+                                long guard_forces_n, hipStream_t s)
 {
     if (rows < N) return hipErrorInvalidValue;
     if (rows <= 0) return hipSuccess;
@@ -996,11 +1003,11 @@ hipError_t launch_readout_fused(int N, int rows, int K, int num_LM, const int* n
     }
     hipLaunchKernelGGL(k_readout_fused<F>, dim3((rows + 15) / 16), dim3(256), lds, s, N, rows, K, num_LM, node_types,
                        atomic_energies, w1, W1, w2, scale, H1, H2, H2_adj, H1_adj, node_energies, zero_energies,
-                       energies_copy, guard, guard_clear);
+                       energies_copy, guard, guard_clear, guard_forces, guard_forces_n);
     return hipGetLastError();
 }
-template hipError_t launch_readout_fused<double>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const double*, const double*, double*, double*, double*, int, double*, const int*, int*, hipStream_t);
-template hipError_t launch_readout_fused<float>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const float*, const double*, double*, float*, double*, int, double*, const int*, int*, hipStream_t);
+template hipError_t launch_readout_fused<double>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const double*, const double*, double*, double*, double*, int, double*, const int*, int*, double*, long, hipStream_t);
+template hipError_t launch_readout_fused<float>(int, int, int, int, const int*, const double*, const double*, const double*, const double*, double, const float*, const double*, double*, float*, double*, int, double*, const int*, int*, double*, long, hipStream_t);
 
 
 // ===========================================================================

@@ -855,22 +855,4 @@ hipError_t launch_fpart_reduce(long edges, long E, int nslices, const double* fp
     return hipGetLastError();
 }
 
-namespace {
-__global__ void k_poison_forces(const int* guard, double* forces, double* copy, long n)
-{
-    if (!*guard) return;
-    for (long t = (long)blockIdx.x * blockDim.x + threadIdx.x; t < n; t += (long)gridDim.x * blockDim.x) {
-        forces[t] = __builtin_nan("");
-        if (copy) copy[t] = __builtin_nan("");
-    }
-}
-}  // namespace
-hipError_t launch_poison_forces(const int* guard, double* forces, double* copy, long n, hipStream_t s)
-{
-    if (!guard || n <= 0) return hipSuccess;
-    hipLaunchKernelGGL(k_poison_forces, dim3((unsigned)std::min<long>((n + 255) / 256, 2048)), dim3(256), 0, s, guard,
-                       forces, copy, n);
-    return hipGetLastError();
-}
-
 }  // namespace smx

@@ -61,7 +61,11 @@ void smx_model_free(smx_model* m);
 
 /* Public scalar members of class MACE, mace.hpp:19-26,115: keys "num_elements",
  * "num_channels", "l_max", "num_lm", "L_max", "num_LM", "has_zbl", "num_lme",
- * "num_lelm1lm2", "precision" (0/1); "r_cut". */
+ * "num_lelm1lm2", "precision" (0/1); "r_cut".  Beyond the reference:
+ * "num_radial_tables_0/1" (radial tables per layer) and "contraction_tables"
+ * (bit 0 / bit 1 set when the symmetric contraction of layer 0 / layer 1 has all
+ * its monomials inside the standard product basis and runs the kernel compiled
+ * for it; a file with other monomials takes the general kernel). */
 int smx_model_get_int(const smx_model* m, const char* key, int* out);
 int smx_model_get_double(const smx_model* m, const char* key, double* out);
 /* atomic_numbers[T], atomic_energies[T], mace.hpp:25-26.  *n receives the length. */

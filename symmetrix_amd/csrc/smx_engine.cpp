@@ -121,6 +121,8 @@ struct EngineBase {
     }
     HostModel hm;
     int precision = 0;
+    int poly_tables = 0;            // bit 0 / bit 1: layer 0 / layer 1 contraction runs the table-specialised kernel
+    int contraction_tables() const { return poly_tables; }
     int device = 0;                 // ordinal of the GPU the model was loaded on
     hipStream_t stream = nullptr;   // stream of the current call
     bool profiling = false;
@@ -187,7 +189,9 @@ struct Engine : EngineBase {
     DVec<const int4*> pp_packed;
     DVec<const int*> pp_chunks;
     DVec<const F*> pp_coef;
+    DVec<F> M0_slabs, M1_slabs;   // coefficients of the straight-line contraction kernel (poly_spec_shape layout)
     DVec<int> pp_nent;
+    bool M0_tables = false, M1_tables = false;   // every polynomial of the layer maps onto its compile-time table
 
     // ---- geometry of the current edge list (device)
     DVec<int> g_node_types, g_num_neigh, g_neigh_indices, g_neigh_types;
@@ -330,6 +334,38 @@ struct Engine : EngineBase {
         pp_packed.upload(vpk.data(), vpk.size(), s); pp_chunks.upload(vch.data(), vch.size(), s);
         pp_coef.upload(vco.data(), vco.size(), s);
         pp_nent.upload(vne.data(), vne.size(), s);
+        M0_tables = hm.num_LM == 1 || hm.num_LM == 4 || hm.num_LM == 9;
+        for (int LM = 0; LM < hm.num_LM; ++LM) M0_tables = M0_tables && hm.P0[LM].table == LM;
+        M1_tables = hm.P1.table == 0;
+        M0_tables = M0_tables && poly_spec_shape((int)sizeof(F), hm.K, hm.num_LM).CB > 0;
+        M1_tables = M1_tables && poly_spec_shape((int)sizeof(F), hm.K, 1).CB > 0;
+        // slabs of the straight-line kernel: [species][channel block][monomial / V][CB][V]
+        auto slabs = [&](DVec<F>& dst, const PolySpec* polys, int NP) {
+            const PolySpecShape sh = poly_spec_shape((int)sizeof(F), hm.K, NP);
+            constexpr int V = 16 / (int)sizeof(F);
+            const size_t slab = sh.slab_bytes / sizeof(F);
+            std::vector<F> h((size_t)hm.T * sh.kblocks * slab, F(0));
+            for (int P = 0; P < NP; ++P) {
+                const int tn = kPolyTableLen[polys[P].table], m0 = poly_spec_offset(P);
+                for (int t = 0; t < hm.T; ++t)
+                    for (int i = 0; i < tn; ++i)
+                        for (int k = 0; k < hm.K; ++k) {
+                            const int m = m0 + i, kb = k / sh.CB, kloc = k % sh.CB;
+                            h[((size_t)t * sh.kblocks + kb) * slab + ((size_t)(m / V) * sh.CB + kloc) * V + m % V] =
+                                (F)polys[P].table_coef[((size_t)t * tn + i) * hm.K + k];
+                        }
+            }
+            dst.upload(h.data(), h.size(), s);
+            HIPCHK(hipStreamSynchronize(s));   // h goes out of scope
+        };
+        if (num_cus == 0) {
+            hipDeviceProp_t prop;
+            HIPCHK(hipGetDeviceProperties(&prop, device));
+            num_cus = prop.multiProcessorCount;
+        }
+        if (M0_tables) slabs(M0_slabs, hm.P0.data(), hm.num_LM);
+        if (M1_tables) slabs(M1_slabs, &hm.P1, 1);
+        poly_tables = (M0_tables ? 1 : 0) | (M1_tables ? 2 : 0);
         flags.resize(8, s);
         HIPCHK(hipStreamSynchronize(s));
     }
@@ -707,6 +743,8 @@ struct Engine : EngineBase {
             p.A = A0.p; p.M = M0.p; p.M_grad = M0_grad.p;
         }
         p.packed = pp_packed.p + off; p.chunks = pp_chunks.p + off; p.coef = pp_coef.p + off; p.num_entries = pp_nent.p + off;
+        p.table_slabs = (layer1 ? M1_tables : M0_tables) ? (layer1 ? M1_slabs.p : M0_slabs.p) : nullptr;
+        p.num_cus = num_cus;
         need(t_perm.p, "species groups");
         p.perm = t_perm.p; p.tstart = t_start.p; p.T = hm.T;
         HIPCHK(launch_poly<F>(p, stream));
@@ -1613,6 +1651,7 @@ int smx_model_get_int(const smx_model* m, const char* key, int* out)
         else if (k == "precision") *out = m->eng->precision;
         else if (k == "num_radial_tables_0") *out = (int)h.tables0.size();
         else if (k == "num_radial_tables_1") *out = (int)h.tables1.size();
+        else if (k == "contraction_tables") *out = m->eng->contraction_tables();
         else throw smx::Error(SMX_EINVAL, "unknown integer key '" + k + "'");
     });
 }

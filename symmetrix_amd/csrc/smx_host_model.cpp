@@ -1,5 +1,6 @@
 // Model-file loader: symmetrix JSON -> HostModel.  See smx_host_model.hpp.
 #include "smx_host_model.hpp"
+#include "smx_poly_tables.inc"
 
 #include <algorithm>
 #include <cmath>
@@ -89,7 +90,7 @@ std::vector<double> build_splines(double h, const Json& values, const Json& deri
 // -> rows sharing the first two factors.  Duplicate monomials keep the first
 // coefficient, as the std::map::insert of multivariate_polynomial.cpp:36-38.
 template <typename CoefFn>
-PolySpec build_poly(int num_lm, int T, int K, const std::vector<std::vector<int>>& monomials, CoefFn coef_of)
+PolySpec build_poly(int num_lm, int T, int K, const std::vector<std::vector<int>>& monomials, CoefFn coef_of, int canon_table)
 {
     constexpr int ONE = 16;
     struct Ent { int i0, i1, c, src; };
@@ -177,6 +178,30 @@ PolySpec build_poly(int num_lm, int T, int K, const std::vector<std::vector<int>
             for (size_t i = 0; i < ents.size(); ++i)
                 P.coef[((size_t)a * (ents.size() + 1) + i) * K + k] = w[ents[i].src];
         }
+    // the standard product basis: every monomial of the file inside the compile-time table of this output slot?
+    int tn = 0;
+    const unsigned char (*tab)[3] = poly_table(canon_table, &tn);
+    if (tab) {
+        std::map<std::tuple<int, int, int>, int> where;
+        for (int i = 0; i < tn; ++i) where[std::make_tuple((int)tab[i][0], (int)tab[i][1], (int)tab[i][2])] = i;
+        std::vector<int> slot(ents.size(), -1);
+        bool inside = true;
+        for (size_t i = 0; i < ents.size() && inside; ++i) {
+            auto it = where.find(std::make_tuple(ents[i].i0, ents[i].i1, ents[i].c));
+            if (it == where.end()) inside = false;
+            else slot[i] = it->second;
+        }
+        if (inside) {
+            P.table = canon_table;
+            P.table_coef.assign((size_t)T * tn * K, 0.0);
+            for (int a = 0; a < T; ++a)
+                for (int k = 0; k < K; ++k) {
+                    const std::vector<double>& w = coef_of(a, k);
+                    for (size_t i = 0; i < ents.size(); ++i)
+                        P.table_coef[((size_t)a * tn + slot[i]) * K + k] = w[ents[i].src];
+                }
+        }
+    }
     return P;
 }
 
@@ -281,7 +306,7 @@ HostModel load_host_model(const std::string& path)
             auto monos = monomial_list(M.at(std::to_string(LM)));
             m.P0[LM] = build_poly(m.num_lm, T, K, monos, [&](int a, int k) -> const std::vector<double>& {
                 return W.at(std::to_string(a)).at(std::to_string(LM)).at(std::to_string(k)).nums;
-            });
+            }, LM);
         }
     }
     m.H1_weights = file.at("H1_weights").as_doubles();
@@ -367,7 +392,7 @@ HostModel load_host_model(const std::string& path)
         auto monos = monomial_list(file.at("M1_monomials"));
         m.P1 = build_poly(m.num_lm, T, K, monos, [&](int a, int k) -> const std::vector<double>& {
             return W.at(std::to_string(a)).at(std::to_string(k)).nums;
-        });
+        }, 0);
     }
     // H2 and readouts, mace.cpp:1017-1029
     {

@@ -42,6 +42,11 @@ struct PolySpec {
     // g = 0 .. POLY_GROUPS-1, so that each group's chunks are contiguous.
     std::vector<int> packed;                     // [4 * (total chunks + POLY_SPARE_CHUNKS)]
     std::vector<int> chunks;                     // [32]: chunks of (v, first part), (v, rest), same order
+    // The same coefficients laid out for the compile-time monomial table `table` of the standard product basis
+    // (smx_poly_tables.inc): [T][table length][K], zero where the file has no such monomial; table = -1 when the
+    // file holds a monomial outside the table (the general kernel then runs).
+    int table = -1;
+    std::vector<double> table_coef;
 };
 
 struct HostModel {

@@ -12,6 +12,28 @@ def tiny_model(K=4, L_max=1, T=(1, 6, 8), r_cut=4.0, n_pts=48, seed=3, pair=True
                                    pair_dependent_radial=pair, zbl=zbl, density_normalisation=density)
 
 
+def add_foreign_monomials(model, layers=(0, 1), seed=0):
+    """One monomial from outside the standard product basis in every polynomial of the given layers (a term linear in
+    a harmonic that cannot couple to the output: Y_1,-1 for scalar outputs, Y_00 for the others), with random
+    coefficients.  Such a file is still a valid symmetrix model; its contraction takes the general kernel."""
+    rng = np.random.default_rng(seed)
+    if 0 in layers:
+        for LM, monos in model["M0_monomials"].items():
+            extra = [1] if int(LM) == 0 else [0]
+            assert extra not in monos
+            monos.append(extra)
+            for a in model["M0_weights"]:
+                for k in model["M0_weights"][a][LM]:
+                    model["M0_weights"][a][LM][k].append(float(rng.normal() * 0.1))
+    if 1 in layers:
+        assert [1] not in model["M1_monomials"]
+        model["M1_monomials"].append([1])
+        for a in model["M1_weights"]:
+            for k in model["M1_weights"][a]:
+                model["M1_weights"][a][k].append(float(rng.normal() * 0.1))
+    return model
+
+
 def write_model(model, path):
     with open(path, "w") as f:
         json.dump(model, f)

@@ -79,19 +79,24 @@ def test_headline_configuration_at_full_size_against_the_oracle(gpu, tmp_models,
 
 @pytest.mark.parametrize("dtype", ["float64", "float32"])
 @pytest.mark.parametrize("L_max", [0, 1])
-def test_contraction_blocks_of_several_atom_groups(gpu, tmp_models, L_max, dtype):
-    """4 400 atoms with K = 32: enough atoms that the symmetric contraction packs two atom groups of 32 channels into
-    one wavefront per variable group, in either precision (single precision takes four atoms per thread and needs
-    more than 4 096 atoms for it), with one polynomial (scalar hidden features) and with four."""
+@pytest.mark.parametrize("foreign", [False, True])
+def test_contraction_blocks_of_several_atom_groups(gpu, tmp_models, L_max, dtype, foreign):
+    """4 400 atoms with K = 32, one polynomial (scalar hidden features) and four.  The kernel of the standard product
+    basis gives every block a run of several passes of eight atoms; with a monomial from outside that basis in every
+    polynomial the general kernel runs, and packs two atom groups of 32 channels into one wavefront per variable group
+    in either precision (single precision takes four atoms per thread and needs more than 4 096 atoms for it)."""
     from oracle.oracle import OracleMACE
     model = H.tiny_model(K=32, L_max=L_max, n_pts=64, seed=40 + L_max, pair=False)
-    path = H.write_model(model, tmp_models / f"groups_{L_max}.json")
+    if foreign:
+        H.add_foreign_monomials(model, seed=5)
+    path = H.write_model(model, tmp_models / f"groups_{L_max}_{int(foreign)}.json")
     pos, cell, sp = H.small_system(4400, seed=9)
     nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
     print(f"case K=32 L_max={L_max} atoms=4400 edges={len(ea['r'])} {dtype}", flush=True)
     orc = OracleMACE(path)
     orc.compute_node_energies_forces(*H.call_args(ea))
     eng = gpu(path, dtype)
+    assert eng._int("contraction_tables") == (0 if foreign else 3)
     eng.compute_node_energies_forces(*H.call_args(ea))
     Eo = orc.node_energies.sum()
     assert abs(eng.node_energies.sum() - Eo) <= TOL[dtype]["E"] * max(abs(Eo), np.abs(orc.node_energies).sum() * 1e-3)

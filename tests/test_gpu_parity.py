@@ -86,6 +86,27 @@ def test_pipeline_matches_oracle(gpu, tmp_models, K, L_max, natoms, pair, dtype)
 
 
 @pytest.mark.parametrize("dtype", ["float64", "float32"])
+@pytest.mark.parametrize("K,L_max,natoms,layers", [(32, 0, 40, (0, 1)), (33, 1, 25, (0, 1)), (96, 0, 48, (1,)),
+                                                   (20, 1, 30, (0,)), (16, 2, 22, (0, 1)), (128, 1, 20, (0, 1))])
+def test_monomials_outside_the_standard_basis_take_the_general_kernel(gpu, tmp_models, K, L_max, natoms, layers, dtype):
+    """The symmetric contraction has a kernel compiled for the monomial lists of the standard product basis (every
+    other model in this file runs it) and a general one that walks whatever lists the file holds.  Files with one
+    more monomial in the polynomials of layer 0, of layer 1 or of both: the loader must send exactly those layers to
+    the general kernel, and all intermediates, energies and forces must still match the oracle."""
+    model = H.add_foreign_monomials(H.tiny_model(K=K, L_max=L_max, n_pts=64, seed=K + L_max, pair=False), layers, seed=K)
+    path = H.write_model(model, tmp_models / f"foreign_{K}_{L_max}_{len(layers)}_{layers[0]}.json")
+    orc = _oracle()(model)
+    eng = gpu(path, dtype)
+    assert eng._int("contraction_tables") == 3 - sum(1 << l for l in layers)
+    pos, cell, sp = H.small_system(natoms, seed=natoms)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K={K} L_max={L_max} atoms={natoms} edges={len(ea['r'])} foreign monomials in layers {layers} {dtype}", flush=True)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    _compare(orc, eng, dtype)
+
+
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
 @pytest.mark.parametrize("K,natoms", [(20, 70), (96, 200), (33, 9)])
 def test_two_species_three_radial_tables(gpu, tmp_models, K, natoms, dtype):
     """Scalar hidden features with a few distinct pair tables: the general edge kernels
@@ -527,7 +548,7 @@ def test_receiver_chunks_of_the_layer1_adjoint_change_nothing(gpu, tmp_models, d
 # (K = 16 is a whole number of 32-byte slices in both precisions): with ghost nodes, ZBL or the density
 # normalisation the force array has other contributions before, between and beside those two.
 MODE_CASES = [(0, "float64", False, False, False), (1, "float64", False, True, True), (0, "float32", False, True, False),
-              (1, "float32", False, True, True)]
+              (1, "float32", False, True, True), (2, "float64", False, True, True)]
 MODE_CASES += [(0, dt, True, zbl, dens) for dt in ("float64", "float32")
                for zbl, dens in ((False, False), (True, False), (False, True), (True, True))]
 

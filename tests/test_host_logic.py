@@ -203,3 +203,23 @@ def test_calculator_keeps_the_reference_signature():
     assert SymmetrixCalculator.EXTRACT_KEYWORDS == ("species", "head", "num_spline_points")
     with pytest.raises(ValueError):
         SymmetrixCalculator("x.json", dtype="float16")
+
+
+def test_compiled_monomial_tables_are_the_generators_output():
+    """smx_poly_tables.inc (the monomial lists the straight-line contraction kernel is compiled for) is committed;
+    it must equal what gen_poly_tables.py writes, and list for every output slot exactly the monomials a generated
+    model carries, in the same order."""
+    import importlib.util
+    csrc = os.path.join(ROOT, "symmetrix_amd", "csrc")
+    spec = importlib.util.spec_from_file_location("gen_poly_tables", os.path.join(csrc, "gen_poly_tables.py"))
+    gen = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(gen)
+    with open(os.path.join(csrc, "smx_poly_tables.inc")) as f:
+        assert f.read() == gen.render()
+    from symmetrix_amd import modelgen
+    model = modelgen.generate_model([1, 8], 2, 2, 4.0, num_spline_points=16, seed=0)
+    tabs = gen.tables()
+    assert len(tabs) == 9
+    for LM, monos in model["M0_monomials"].items():
+        assert [tuple([gen.ONE] * (3 - len(m)) + list(m)) for m in monos] == tabs[int(LM)]
+    assert [tuple([gen.ONE] * (3 - len(m)) + list(m)) for m in model["M1_monomials"]] == tabs[0]

@@ -12,6 +12,8 @@ Prints ONE JSON line.  Besides the driver's fields it carries
   roofline_stages   the same figures for every edge stage (aggregations, their adjoints, the sender-side sum)
   mfma          the dense channel-mixing stages against the matrix-core peak (algorithmic flops / stage time), with the
                 matrix-pipe busy share rocprofv3 counted for the stage's kernel (profiles/)
+  contraction   the two symmetric contractions against the vector-arithmetic peak (flops of the monomial walk / stage
+                time) and their HBM side (variables in, values and gradients out)
   cpu_baseline  the CPU oracle (serial fp64 restatement of the reference path)
                 timed on this host on the same workload
   stages_ms     HIP-event time of every stage of the pipeline
@@ -98,6 +100,25 @@ def dense_flops(stage, N, K, n_LM, n_e):
 
 
 VALU_PEAK = 78.6e12   # vector multiply-add peak of MI355X, flop/s, double or (unpacked) single precision
+
+
+def contraction_work(n_atoms, K, L_max, layer, s_bytes):
+    """Arithmetic and HBM bytes of one symmetric contraction (value and gradient) by the algorithm: per atom, channel
+    and monomial x_a x_b x_c two products and four multiply-adds (10 flops), 7 flops for a monomial of degree two, 3
+    for degree one, with the monomial lists of the standard product basis (harmonics up to l = 3, correlation 3);
+    bytes: the 16 variables in, value and 16 gradient components out, per polynomial."""
+    from symmetrix_amd import cg
+    flops_per = 0
+    polys = 0
+    for L in range((L_max if layer == 0 else 0) + 1):
+        terms = cg.symmetric_contraction_terms(L, 3, 3)
+        for M in range(2 * L + 1):
+            keys = set()
+            for t in terms:
+                keys |= set(t[M].keys())
+            flops_per += sum({1: 3, 2: 7, 3: 10}[len(k)] for k in keys)
+            polys += 1
+    return flops_per * n_atoms * K, (16 + 17 * polys) * K * s_bytes * n_atoms
 
 
 def edge_valu_flops(stage, E, K, L_max):
@@ -409,7 +430,7 @@ def main():
             dt = time.perf_counter() - t0
             eng.set_profiling(False)
             res = dict(ms_sync=1e3 * dt / steps, ms=1e3 * dt_async / steps, stages={k: v / steps for k, v in acc.items()},
-                       tables=eng._int("num_radial_tables_0"))
+                       tables=eng._int("num_radial_tables_0"), contraction_tables=eng._int("contraction_tables"))
             if host_leg:
                 # the same evaluation through the host-array entry point (upload, range checks, download included)
                 hsteps = max(3, min(10, steps // 4))
@@ -483,6 +504,18 @@ def main():
             mfma[k] = {"flops": fl, "kernel_ms": ms_k, "achieved_tflops": fl / (ms_k * 1e-3) / 1e12, "peak_tflops": peak / 1e12,
                        "frac": fl / (ms_k * 1e-3) / peak,
                        "mfma_busy_profiled": measured_mfma_busy(workload, dtype, k) if profiled and not pair_tables else None}
+        # the symmetric contractions: vector arithmetic against the vector peak, and their HBM side
+        contraction = {}
+        for k, layer, n_k in (("M0", 0, N + N_ghost), ("M1", 1, N)):
+            ms_k = res["stages"].get(k, 0.0)
+            if ms_k <= 0.0:
+                continue
+            fl, by = contraction_work(n_k, K, L_max, layer, s_bytes)
+            vpeak = VALU_PEAK * (2 if dtype == "float32" else 1)
+            contraction[k] = {"kernel": "k_poly_spec" if res["contraction_tables"] & (1 << layer) else "k_poly",
+                              "flops": fl, "kernel_ms": ms_k, "achieved_tflops": fl / (ms_k * 1e-3) / 1e12,
+                              "peak_tflops": vpeak / 1e12, "valu_frac": fl / (ms_k * 1e-3) / vpeak,
+                              "algorithmic_bytes": by, "hbm_frac": by / (ms_k * 1e-3) / HBM_PEAK}
         out = dict(
             cfg=cfg, model_path=model_path, ea=ea, N=N, E=E, N_ghost=N_ghost, E_local=E_local, res=res,
             value=N / (res["ms"] * 1e-3),
@@ -497,7 +530,7 @@ def main():
                 "whole_step_algorithmic_bytes": total_bytes,
                 "whole_step_frac": (total_bytes / HBM_PEAK) / (res["ms"] * 1e-3),
             },
-            roofline_stages=stages_rl, mfma=mfma,
+            roofline_stages=stages_rl, mfma=mfma, contraction=contraction,
         )
         if both:
             other = "float32" if dtype == "float64" else "float64"
@@ -537,6 +570,7 @@ def main():
         "roofline": m["roofline"],
         "roofline_stages": m["roofline_stages"],
         "mfma": m["mfma"],
+        "contraction": m["contraction"],
         "stages_ms": res["stages"],
         "ms_per_step_with_event_readback": res["ms_sync"],
         "host_arrays": {"ms_per_step": res["ms_host"], "value": N / (res["ms_host"] * 1e-3),
@@ -554,7 +588,7 @@ def main():
         line["second_config"] = {
             "workload": m2["workload"], "dtype": "f32-features/f64-accumulation", "steps": s2, "warmup": 2,
             "ms_per_step": m2["res"]["ms"], "value": m2["value"], "unit": "atom-steps/s", "roofline": m2["roofline"],
-            "roofline_stages": m2["roofline_stages"], "mfma": m2["mfma"],
+            "roofline_stages": m2["roofline_stages"], "mfma": m2["mfma"], "contraction": m2["contraction"],
             "stages_ms": m2["res"]["stages"], "energy": m2["res"]["energy"],
         }
         # the headline workload with one radial table per species pair (ten tables for four species): more than four

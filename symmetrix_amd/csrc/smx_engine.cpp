@@ -729,18 +729,26 @@ struct Engine : EngineBase {
         HIPCHK(launch_zbl(N, first_neigh.p, node_types, neigh_types, xyz, r, zbl_params(), node_energies.p,
                           node_forces.p, stream));
     }
-    void st_poly(int N, bool layer1)
+    // Layer 0 with several polynomials per channel and the standard product basis: the evaluation keeps no
+    // gradients (16 numbers per polynomial and channel: four times the variables at l <= 1, nine times at l <= 2,
+    // written once and read once); the adjoint stage evaluates them again from the variables instead.
+    bool recompute_M0_grad() const { return M0_tables && NLM() > 1; }
+    // mode 0: values and gradients; 1: values only; 2: layer-0 adjoint from the variables (A0_adj from A0, M0_adj)
+    void st_poly(int N, bool layer1, int mode = 0)
     {
         PolyParams<F> p{};
-        p.num_nodes = N; p.K = K();
+        p.num_nodes = N; p.K = K(); p.mode = mode;
         const int off = layer1 ? NLM() : 0;
         p.NP = layer1 ? 1 : NLM();
         if (layer1) {
             M1.size_to((size_t)N * K(), stream); M1_grad.size_to((size_t)N * 16 * K(), stream);
             p.A = A1.p; p.M = M1.p; p.M_grad = M1_grad.p;
+        } else if (mode == 2) {
+            p.A = A0.p; p.M_adj = M0_adj.p; p.A_adj = A0_adj.p;
         } else {
-            M0.size_to((size_t)N * NLM() * K(), stream); M0_grad.size_to((size_t)N * NLM() * 16 * K(), stream);
-            p.A = A0.p; p.M = M0.p; p.M_grad = M0_grad.p;
+            M0.size_to((size_t)N * NLM() * K(), stream);
+            if (mode == 0) M0_grad.size_to((size_t)N * NLM() * 16 * K(), stream);
+            p.A = A0.p; p.M = M0.p; p.M_grad = mode == 0 ? M0_grad.p : nullptr;
         }
         p.packed = pp_packed.p + off; p.chunks = pp_chunks.p + off; p.coef = pp_coef.p + off; p.num_entries = pp_nent.p + off;
         p.table_slabs = (layer1 ? M1_tables : M0_tables) ? (layer1 ? M1_slabs.p : M0_slabs.p) : nullptr;
@@ -865,10 +873,16 @@ struct Engine : EngineBase {
     }
     // node counts for which compute() left A1_adj / A0_adj unwritten (-1: they are current)
     int pending_A1_adj = -1, pending_A0_adj = -1;
-    void materialise_adjoints()
+    int pending_M0_grad = -1;   // compute() kept no layer-0 gradients for this many nodes: formed when somebody asks
+    void materialise_adjoints(bool gradients)
     {
         if (pending_A1_adj >= 0) { st_reverse_M1(pending_A1_adj); pending_A1_adj = -1; }
         if (pending_A0_adj >= 0) { st_reverse_M0(pending_A0_adj); pending_A0_adj = -1; }
+        if (gradients && pending_M0_grad >= 0) {
+            const int n = pending_M0_grad;
+            pending_M0_grad = -1;
+            if (n > 0) { build_type_groups(n); st_poly(n, false, 0); }
+        }
     }
     void st_reverse_M1(int N)
     {
@@ -880,7 +894,12 @@ struct Engine : EngineBase {
         A0_adj.size_to(A0.n, stream);
         if (A0.n > (size_t)N * 16 * K())
             HIPCHK(hipMemsetAsync(A0_adj.p, 0, A0_adj.n * sizeof(F), stream));  // mace.cpp:376-377
-        HIPCHK(launch_poly_reverse<F>(N, NLM(), K(), M0_grad.p, M0_adj.p, A0_adj.p, stream));
+        if (pending_M0_grad >= 0) {
+            need(t_perm.p, "species groups");
+            st_poly(N, false, 2);
+        } else {
+            HIPCHK(launch_poly_reverse<F>(N, NLM(), K(), M0_grad.p, M0_adj.p, A0_adj.p, stream));
+        }
     }
     void st_agg1_bwd(int N, bool zero_dxyz, bool zero_H1_adj)
     {
@@ -1133,7 +1152,8 @@ struct Engine : EngineBase {
         stage_begin(ST_AGG0F); st_agg0_fwd(N); stage_end(ST_AGG0F);
         stage_begin(ST_A0LIN); st_A0_lin(N, false); stage_end(ST_A0LIN);
         st_scale(0, N, false);
-        stage_begin(ST_M0); st_poly(N, false); stage_end(ST_M0);
+        pending_M0_grad = recompute_M0_grad() ? N : -1;
+        stage_begin(ST_M0); st_poly(N, false, pending_M0_grad >= 0 ? 1 : 0); stage_end(ST_M0);
         stage_begin(ST_H1); st_H1(N, false); stage_end(ST_H1);
         // per-species node groups and the degree order of the receivers cover the nodes of the current stages
         auto node_lists_for = [&](int n) {
@@ -1194,7 +1214,7 @@ struct Engine : EngineBase {
         const std::string s(name);
         energies_copy = nullptr; forces_copy = nullptr;
         carried_edges = 0; carry_forces = false; fuse_reverse_H1 = false; guard_status = nullptr;
-        materialise_adjoints();
+        materialise_adjoints(true);
         if (N < 0) throw Error(SMX_EINVAL, "negative num_nodes");
         // A stage may cover the leading nodes of a longer edge list (the pair style runs layer 1 on its local
         // nodes with the arrays of local + ghost nodes, pair_symmetrix_mace.cpp:681-693): the edge arrays keep
@@ -1283,7 +1303,7 @@ struct Engine : EngineBase {
     {
         const std::string s(name);
         hipStream_t st = stream;
-        materialise_adjoints();
+        materialise_adjoints(s == "M0_grad");
         const double* src = nullptr;
         size_t len = 0;
         if (s == "Y" || s == "Y_grad") {
@@ -1326,7 +1346,7 @@ struct Engine : EngineBase {
         const std::string s(name);
         hipStream_t st = stream;
         if (n < 0) throw Error(SMX_EINVAL, "negative length");
-        materialise_adjoints();
+        materialise_adjoints(true);
         Named v = find(s);
         if (s == "R0" || s == "R1")
             throw Error(SMX_EUNSUPPORTED, "unsupported: '" + s + "' is evaluated from r inside the edge kernels and never "
@@ -1355,7 +1375,7 @@ struct Engine : EngineBase {
     {
         const std::string s(name);
         if (n < 0) throw Error(SMX_EINVAL, "negative length");
-        materialise_adjoints();
+        materialise_adjoints(true);
         Named v = find(s);
         if ((!v.f && !v.d) || s == "H0_weights" || s == "M0_grad" || s == "M1_grad")
             throw Error(SMX_EINVAL, "array '" + s + "' cannot be set");

@@ -227,6 +227,11 @@ struct PolyParams {
     // straight-line kernel runs; else null.
     const F* table_slabs;
     int num_cus;
+    // with table_slabs only: 0 values and gradients; 1 values only (M_grad unused); 2 adjoint,
+    // A_adj[N][16][K] = sum_p M_adj[N][NP][K] * dM_p/dA recomputed from A (M and M_grad unused)
+    int mode;
+    const F* M_adj;
+    F* A_adj;
 };
 
 // Coefficient slabs of the straight-line contraction kernel.  The monomials of polynomials 0..NP-1 follow one another,

@@ -642,17 +642,16 @@ template <typename F> __device__ __forceinline__ void pin_reg(F& v) { asm volati
 template <typename F> constexpr int spec_group() { return sizeof(F) == 8 ? 4 : 8; }   // coefficients per request
 constexpr int SPEC_BT = 256;     // threads per block
 
-template <typename F, int LM>
-__device__ __forceinline__ void poly_spec_body(const PolyParams<F>& a, const unsigned char* slab_k, int row_stride_bytes,
-                                               F (&x)[16], bool live, int node, int k)
+// MODE 0: values and gradients (M, M_grad); 1: values only; 2: adjoint, A_adj = sum over the polynomials of
+// M_adj[polynomial] * gradient, recomputed from the variables (the coefficient is scaled, the value dropped).
+template <typename F, int LM, int MODE>
+__device__ __forceinline__ void poly_spec_body(const unsigned char* slab_k, int row_stride_bytes, F (&x)[16], F (&g)[16], F& f,
+                                               F madj)
 {
     using TB = PolyTable<LM>;
     constexpr int V = 16 / (int)sizeof(F);
     typedef F V4 __attribute__((ext_vector_type(V)));
     constexpr int row0 = poly_spec_offset(LM) / V;   // first 16-byte group of this polynomial in the slab
-    F g[16], f = F(0);   // x is not const: it passes through the register pins below (its values never change)
-#pragma unroll
-    for (int q = 0; q < 16; ++q) g[q] = F(0);
     // Coefficients come in small groups: the next group is requested before the current one is used; compiler
     // and scheduling barriers keep all groups from being requested at once (the variables would spill).
     constexpr int G = spec_group<F>(), NG = (TB::N + G - 1) / G, RG = G / V;
@@ -661,7 +660,7 @@ __device__ __forceinline__ void poly_spec_body(const PolyParams<F>& a, const uns
         constexpr int r0 = decltype(gc)::value * RG;
 #pragma unroll
         for (int j = 0; j < RG; ++j)
-            if (( r0 + j) * V < poly_spec_padded(TB::N))
+            if ((r0 + j) * V < poly_spec_padded(TB::N))
                 w[j] = *reinterpret_cast<const V4*>(slab_k + (size_t)(row0 + r0 + j) * row_stride_bytes);
     };
     request(std::integral_constant<int, 0>{}, wbuf[0]);
@@ -673,42 +672,42 @@ __device__ __forceinline__ void poly_spec_body(const PolyParams<F>& a, const uns
         static_for<gi * G, (gi * G + G < TB::N ? gi * G + G : TB::N)>([&](auto ic) {
             constexpr int i = decltype(ic)::value;
             constexpr int ia = TB::m[i][0], ib = TB::m[i][1], jc = TB::m[i][2];
-            const F w = wbuf[gi & 1][(i - gi * G) / V][(i - gi * G) % V];
+            F w = wbuf[gi & 1][(i - gi * G) / V][(i - gi * G) % V];
+            if constexpr (MODE == 2) w *= madj;
             if constexpr (ib == 16) {            // degree 1
-                g[jc] += w;
-                f += w * x[jc];
+                if constexpr (MODE != 1) g[jc] += w;
+                if constexpr (MODE != 2) f += w * x[jc];
             } else if constexpr (ia == 16) {     // degree 2
                 const F t = w * x[ib];
-                g[jc] += t;
-                g[ib] += w * x[jc];
-                f += t * x[jc];
+                if constexpr (MODE != 1) {
+                    g[jc] += t;
+                    g[ib] += w * x[jc];
+                }
+                if constexpr (MODE != 2) f += t * x[jc];
             } else {
                 const F wa = w * x[ia], pbc = x[ib] * x[jc];
-                g[ia] += w * pbc;
-                g[ib] += wa * x[jc];
-                g[jc] += wa * x[ib];
-                f += wa * pbc;
+                if constexpr (MODE != 1) {
+                    g[ia] += w * pbc;
+                    g[ib] += wa * x[jc];
+                    g[jc] += wa * x[ib];
+                }
+                if constexpr (MODE != 2) f += wa * pbc;
             }
         });
         // The sums are final here and the variables are new values for the next group: without this the arithmetic
         // of all groups sinks below the last request (the coefficients of the whole polynomial live at once) and the
         // pairwise products of the variables are hoisted above the first group (over a hundred more live values).
-        pin_reg(f);
+        if constexpr (MODE != 2) pin_reg(f);
 #pragma unroll
         for (int q = 0; q < 16; ++q) {
-            pin_reg(g[q]);
-            pin_reg(x[q]);
+            if constexpr (MODE != 1) pin_reg(g[q]);
+            pin_reg(x[q]);   // (x is not const for this: its values never change)
         }
         __builtin_amdgcn_sched_barrier(0);
     });
-    if (live) {
-#pragma unroll
-        for (int q = 0; q < 16; ++q) a.M_grad[(((size_t)node * a.NP + LM) * 16 + q) * a.K + k] = g[q];
-        a.M[((size_t)node * a.NP + LM) * a.K + k] = f;
-    }
 }
 
-template <typename F, int COUNT>
+template <typename F, int COUNT, int MODE>
 __global__ __launch_bounds__(SPEC_BT, sizeof(F) == 8 ? 4 : 5) void k_poly_spec(const PolyParams<F> a, const PolySpecShape sh, int chunk)
 {
     extern __shared__ __align__(16) unsigned char spec_lds[];
@@ -741,14 +740,39 @@ __global__ __launch_bounds__(SPEC_BT, sizeof(F) == 8 ? 4 : 5) void k_poly_spec(c
         const int j = jb + ag;
         const bool live = klive && j < j1;
         const int node = a.perm[seg0 + (j < seg_n ? j : seg_n - 1)];
-        F x[16];
+        F x[16], g[16], madj = F(1);
 #pragma unroll
         for (int q = 0; q < 16; ++q) x[q] = a.A[((size_t)node * 16 + q) * a.K + kk];
+        if constexpr (MODE == 2) {
+            madj = a.M_adj[(size_t)node * COUNT * a.K + kk];
+#pragma unroll
+            for (int q = 0; q < 16; ++q) g[q] = F(0);
+        }
         // one polynomial after the other: the variables are read once
         static_for<0, COUNT>([&](auto pc) {
             constexpr int P = decltype(pc)::value;
-            poly_spec_body<F, P>(a, slab_k, row_stride, x, live, node, k);
+            F f = F(0), madj_next = F(1);
+            if constexpr (MODE == 2 && P + 1 < COUNT) madj_next = a.M_adj[((size_t)node * COUNT + P + 1) * a.K + kk];
+            if constexpr (MODE == 0) {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) g[q] = F(0);
+            }
+            poly_spec_body<F, P, MODE>(slab_k, row_stride, x, g, f, madj);
+            madj = madj_next;
+            if (live) {
+                if constexpr (MODE == 0) {
+#pragma unroll
+                    for (int q = 0; q < 16; ++q) a.M_grad[(((size_t)node * COUNT + P) * 16 + q) * a.K + k] = g[q];
+                }
+                if constexpr (MODE != 2) a.M[((size_t)node * COUNT + P) * a.K + k] = f;
+            }
         });
+        if constexpr (MODE == 2) {
+            if (live) {
+#pragma unroll
+                for (int q = 0; q < 16; ++q) a.A_adj[((size_t)node * 16 + q) * a.K + k] = g[q];
+            }
+        }
     }
 }
 
@@ -797,22 +821,28 @@ hipError_t launch_poly(const PolyParams<F>& p, hipStream_t s)
         chunk = (chunk + sh.AG - 1) / sh.AG * sh.AG;
         const unsigned units = (unsigned)((p.num_nodes + chunk - 1) / chunk + p.T);
         const dim3 grid(units * sh.kblocks), block(SPEC_BT);
-        auto go = [&](auto cc) -> hipError_t {
-            constexpr int COUNT = decltype(cc)::value;
+        auto go = [&](auto cc, auto mc) -> hipError_t {
+            constexpr int COUNT = decltype(cc)::value, MODE = decltype(mc)::value;
             static bool attr_done = false;   // per instantiation
             if (!attr_done) {
-                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_poly_spec<F, COUNT>),
+                hipError_t err = hipFuncSetAttribute(reinterpret_cast<const void*>(k_poly_spec<F, COUNT, MODE>),
                                                      hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
                 if (err != hipSuccess) return err;
                 attr_done = true;
             }
-            hipLaunchKernelGGL((k_poly_spec<F, COUNT>), grid, block, sh.slab_bytes, s, p, sh, chunk);
+            hipLaunchKernelGGL((k_poly_spec<F, COUNT, MODE>), grid, block, sh.slab_bytes, s, p, sh, chunk);
             return hipGetLastError();
         };
-        if (p.NP == 1) return go(std::integral_constant<int, 1>{});
-        if (p.NP == 4) return go(std::integral_constant<int, 4>{});
-        return go(std::integral_constant<int, 9>{});
+        auto with_count = [&](auto mc) -> hipError_t {
+            if (p.NP == 1) return go(std::integral_constant<int, 1>{}, mc);
+            if (p.NP == 4) return go(std::integral_constant<int, 4>{}, mc);
+            return go(std::integral_constant<int, 9>{}, mc);
+        };
+        if (p.mode == 1) return with_count(std::integral_constant<int, 1>{});
+        if (p.mode == 2) return with_count(std::integral_constant<int, 2>{});
+        return with_count(std::integral_constant<int, 0>{});
     }
+    if (p.mode != 0) return hipErrorInvalidValue;   // the general kernel has the one mode
     const PolyShape sh = poly_shape(p.K, (p.num_nodes + poly_nb<F>() - 1) / poly_nb<F>());
     const int kblocks = (p.K + sh.CB - 1) / sh.CB;
     const int per_block = poly_nb<F>() * sh.AG;

@@ -19,7 +19,9 @@ pytestmark = pytest.mark.gpu
 GOLD = os.path.join(os.path.dirname(__file__), "golden")
 TOL = {"float64": dict(E=1e-10, F=1e-8, inter=1e-11), "float32": dict(E=1e-5, F=1e-4, inter=2e-5)}
 INTERMEDIATES = ["Y", "Y_grad", "R0", "R1", "A0", "M0", "H1", "Phi1", "A1", "M1", "H2", "H2_adj", "M1_adj",
-                 "A1_adj", "Phi1_adj", "H1_adj", "M0_adj", "A0_adj"]
+                 "A1_adj", "Phi1_adj", "H1_adj", "M0_adj", "A0_adj", "M1_grad", "M0_grad"]
+# (M0_grad last: with several polynomials per channel an evaluation keeps no layer-0 gradients, the adjoint forms
+# them again from A0; asking for the array evaluates them from the A0 the evaluation left)
 
 
 @pytest.fixture(scope="module")

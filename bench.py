@@ -102,12 +102,16 @@ def dense_flops(stage, N, K, n_LM, n_e):
 VALU_PEAK = 78.6e12   # vector multiply-add peak of MI355X, flop/s, double or (unpacked) single precision
 
 
-def contraction_work(n_atoms, K, L_max, layer, s_bytes):
-    """Arithmetic and HBM bytes of one symmetric contraction (value and gradient) by the algorithm: per atom, channel
-    and monomial x_a x_b x_c two products and four multiply-adds (10 flops), 7 flops for a monomial of degree two, 3
-    for degree one, with the monomial lists of the standard product basis (harmonics up to l = 3, correlation 3);
-    bytes: the 16 variables in, value and 16 gradient components out, per polynomial."""
+def contraction_work(n_atoms, K, L_max, layer, s_bytes, mode="both"):
+    """Arithmetic and HBM bytes of one symmetric-contraction launch by the algorithm, with the monomial lists of the
+    standard product basis (harmonics up to l = 3, correlation 3).  Per atom, channel and monomial x_a x_b x_c:
+    value and gradient ("both") two products and four multiply-adds (10 flops; 7 and 3 for degrees two and one);
+    value only ("value") two products and one multiply-add (4; 3; 2); the adjoint that forms the gradient again
+    ("adjoint") three products and three multiply-adds (9; 5; 2).  Bytes: the 16 variables in; out, per polynomial,
+    the value ("both", "value") and its 16 gradient components ("both"); the adjoint reads the polynomials' adjoints
+    and writes 16 sums."""
     from symmetrix_amd import cg
+    per_degree = {"both": {1: 3, 2: 7, 3: 10}, "value": {1: 2, 2: 3, 3: 4}, "adjoint": {1: 2, 2: 5, 3: 9}}[mode]
     flops_per = 0
     polys = 0
     for L in range((L_max if layer == 0 else 0) + 1):
@@ -116,9 +120,10 @@ def contraction_work(n_atoms, K, L_max, layer, s_bytes):
             keys = set()
             for t in terms:
                 keys |= set(t[M].keys())
-            flops_per += sum({1: 3, 2: 7, 3: 10}[len(k)] for k in keys)
+            flops_per += sum(per_degree[len(k)] for k in keys)
             polys += 1
-    return flops_per * n_atoms * K, (16 + 17 * polys) * K * s_bytes * n_atoms
+    words = {"both": 16 + 17 * polys, "value": 16 + polys, "adjoint": 32 + polys}[mode]
+    return flops_per * n_atoms * K, words * K * s_bytes * n_atoms
 
 
 def edge_valu_flops(stage, E, K, L_max):
@@ -506,13 +511,17 @@ def main():
                        "mfma_busy_profiled": measured_mfma_busy(workload, dtype, k) if profiled and not pair_tables else None}
         # the symmetric contractions: vector arithmetic against the vector peak, and their HBM side
         contraction = {}
-        for k, layer, n_k in (("M0", 0, N + N_ghost), ("M1", 1, N)):
+        # (layer 0 with several polynomials per channel and the standard basis keeps no gradients: values in M0,
+        # the gradient formed again in rev_M0)
+        split0 = bool(res["contraction_tables"] & 1) and n_LM > 1
+        for k, layer, n_k, mode in (("M0", 0, N + N_ghost, "value" if split0 else "both"), ("M1", 1, N, "both"),
+                                    ("rev_M0", 0, N + N_ghost, "adjoint")):
             ms_k = res["stages"].get(k, 0.0)
-            if ms_k <= 0.0:
+            if ms_k <= 0.0 or (k == "rev_M0" and not split0):
                 continue
-            fl, by = contraction_work(n_k, K, L_max, layer, s_bytes)
-            vpeak = VALU_PEAK * (2 if dtype == "float32" else 1)
-            contraction[k] = {"kernel": "k_poly_spec" if res["contraction_tables"] & (1 << layer) else "k_poly",
+            fl, by = contraction_work(n_k, K, L_max, layer, s_bytes, mode)
+            vpeak = VALU_PEAK
+            contraction[k] = {"kernel": "k_poly_spec" if res["contraction_tables"] & (1 << layer) else "k_poly", "mode": mode,
                               "flops": fl, "kernel_ms": ms_k, "achieved_tflops": fl / (ms_k * 1e-3) / 1e12,
                               "peak_tflops": vpeak / 1e12, "valu_frac": fl / (ms_k * 1e-3) / vpeak,
                               "algorithmic_bytes": by, "hbm_frac": by / (ms_k * 1e-3) / HBM_PEAK}

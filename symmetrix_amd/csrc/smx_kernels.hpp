@@ -270,6 +270,8 @@ inline PolySpecShape poly_spec_shape(int elem, int K, int NP)
     return best;
 }
 template <typename F> hipError_t launch_poly(const PolyParams<F>& p, hipStream_t s);
+// the table_slabs branch of launch_poly (smx_kernels_poly.hip)
+template <typename F> hipError_t launch_poly_spec(const PolyParams<F>& p, hipStream_t s);
 
 // A_adj[i,lm,k] = sum_LM M_grad[i,LM,lm,k] * M_adj[i,LM,k]   (reverse_M0 / reverse_M1)
 template <typename F>

@@ -881,7 +881,9 @@ struct Engine : EngineBase {
         if (gradients && pending_M0_grad >= 0) {
             const int n = pending_M0_grad;
             pending_M0_grad = -1;
-            if (n > 0) { build_type_groups(n); st_poly(n, false, 0); }
+            // (the species groups of the evaluation are still in place: compute() leaves them built for all its nodes,
+            // and every call that rebuilds them comes through here first; the caller's arrays are not read again)
+            if (n > 0) st_poly(n, false, 0);
         }
     }
     void st_reverse_M1(int N)

@@ -223,3 +223,22 @@ def test_compiled_monomial_tables_are_the_generators_output():
     for LM, monos in model["M0_monomials"].items():
         assert [tuple([gen.ONE] * (3 - len(m)) + list(m)) for m in monos] == tabs[int(LM)]
     assert [tuple([gen.ONE] * (3 - len(m)) + list(m)) for m in model["M1_monomials"]] == tabs[0]
+
+
+def test_contraction_slab_shapes_are_valid_for_every_channel_count(tmp_path):
+    """The loader lays the coefficient slabs of the contraction kernel out with the function the launcher sizes its
+    blocks with (smx_poly_shape.hpp, plain C++): for every channel count up to 512, one, four and nine polynomials
+    and both precisions the shape must be one the kernel can run (channel block a multiple of 16 that tiles the
+    padded channel count, at most 256 threads per pass, slabs of all resident blocks within the LDS of a CU)."""
+    import subprocess
+    exe = str(tmp_path / "poly_shape_check")
+    r = subprocess.run(["g++", "-std=c++17", "-Wall", "-Wextra", "-I", os.path.join(ROOT, "symmetrix_amd", "csrc"), "-o", exe,
+                        os.path.join(ROOT, "tests", "cpp", "poly_shape_check.cpp")], capture_output=True)
+    assert r.returncode == 0, r.stderr.decode()
+    r = subprocess.run([exe], capture_output=True)
+    out = r.stdout.decode()
+    assert r.returncode == 0 and "BAD" not in out, out
+    # the padded monomial counts in front of polynomials 1, 4, 9 (94 | 112 92 112 | 90 97 95 97 98, each to a multiple of 4)
+    assert "offsets 96 412 900" in out
+    # the headline shape: 96 channels, one polynomial, double: 32 channels and 24 KB per block, four blocks per CU
+    assert "elem 8 NP 1 K 96: CB 32 AG 8 kblocks 3 blocks 4 slab 24576" in out

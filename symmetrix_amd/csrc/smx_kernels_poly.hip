@@ -11,15 +11,15 @@
 namespace smx {
 
 namespace {
-// The same contraction for the standard product basis (harmonics up to l = 3, correlation order 3): the monomials
-// of output slot LM are a compile-time table (smx_poly_tables.inc), so the walk is straight-line code and the 16
-// variables of an atom stay in registers -- no index loads, no variables in LDS.  The LDS holds the coefficients
-// instead: a block owns one species and one block of CB channels, copies that slab ([monomials of all polynomials]
-// [CB], laid out by the loader as 16-byte groups per channel, see poly_spec_shape) once and then takes a run of
-// `chunk` atoms of the species, AG atoms at a time, one thread per (atom, channel).  Per monomial x_a x_b x_c the
-// thread forms w x_a and x_b x_c once; three multiply-adds give the gradient terms (the product rule holds as written
-// for repeated indices) and one more the value: six instructions.  Used when every polynomial of the launch maps onto
-// its table (the loader checks).
+// For harmonics up to l = 3 and correlation order 3 the monomials of output slot LM are a compile-time table
+// (smx_poly_tables.inc), so the walk is straight-line code and the 16 variables of an atom stay in registers -- no
+// index loads, no variables in LDS.  The LDS holds the coefficients instead: a block owns one species and one block
+// of CB channels, copies that slab ([monomials of all polynomials][CB], laid out by the loader as 16-byte groups per
+// channel, see poly_spec_shape) once and then takes a run of `chunk` atoms of the species, AG atoms at a time, one
+// thread per (atom, channel).  Per monomial x_a x_b x_c the thread forms w x_a and x_b x_c once; three multiply-adds
+// give the gradient terms (the product rule holds as written for repeated indices) and one more the value: six
+// instructions.  Used when every polynomial of the launch maps onto its table (the loader checks); other files take
+// the list-walking kernel of smx_kernels_node.hip.
 template <typename F> __device__ __forceinline__ void pin_reg(F& v) { asm volatile("" : "+v"(v)); }
 template <typename F> constexpr int spec_group() { return sizeof(F) == 8 ? 4 : 8; }   // coefficients per request
 constexpr int SPEC_BT = 256;     // threads per block

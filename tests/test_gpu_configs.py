@@ -103,6 +103,33 @@ def test_contraction_blocks_of_several_atom_groups(gpu, tmp_models, L_max, dtype
     assert np.abs(eng.node_forces - orc.node_forces).max() <= TOL[dtype]["F"] * max(1.0, np.abs(orc.node_forces).max())
 
 
+def test_contraction_runs_of_several_passes(gpu, tmp_models):
+    """30 000 atoms with 16 channels and four polynomials per channel: more atoms than the contraction kernel of the
+    standard product basis has thread slots on the chip, so every block walks its run of atoms in two (single
+    precision) or three (double) passes with the coefficient slab it loaded once; values, the recomputing adjoint
+    and the layer-1 launch against the oracle (about 20 s of CPU, once for both precisions)."""
+    from oracle.oracle import OracleMACE
+    model = H.tiny_model(K=16, L_max=1, n_pts=64, seed=77, pair=False)
+    path = H.write_model(model, tmp_models / "passes.json")
+    pos, cell, sp = H.small_system(30000, seed=5)
+    nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+    print(f"case K=16 L_max=1 atoms=30000 edges={len(ea['r'])}", flush=True)
+    orc = OracleMACE(path)
+    orc.compute_node_energies_forces(*H.call_args(ea))
+    Eo = orc.node_energies.sum()
+    for dtype in ("float64", "float32"):
+        eng = gpu(path, dtype)
+        assert eng._int("contraction_tables") == 3
+        eng.compute_node_energies_forces(*H.call_args(ea))
+        assert abs(eng.node_energies.sum() - Eo) <= TOL[dtype]["E"] * max(abs(Eo), np.abs(orc.node_energies).sum() * 1e-3)
+        assert np.abs(eng.node_energies - orc.node_energies).max() <= TOL[dtype]["E"] * max(1.0, np.abs(orc.node_energies).max()) * 10
+        assert np.abs(eng.node_forces - orc.node_forces).max() <= TOL[dtype]["F"] * max(1.0, np.abs(orc.node_forces).max())
+        for name in ("M0", "M1", "A0_adj", "M0_grad"):
+            a, b = getattr(orc, name), getattr(eng, name)
+            tol = 1e-10 if dtype == "float64" else 2e-4      # the bound test_gpu_parity.py puts on intermediates
+            assert a.shape == b.shape and np.abs(a - b).max() <= tol * max(1.0, np.abs(a).max()), name
+
+
 def test_water_box_with_ghost_nodes_at_full_size(gpu, tmp_models):
     """25 002 atoms, K = 128, hidden features up to l = 1, r_cut 5.0 A, through the full neighbour list with ghost
     atoms as extra nodes (the pair style's no_mpi_message_passing layout on one rank): node energies bit-equal to

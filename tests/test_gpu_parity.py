@@ -794,3 +794,41 @@ def test_device_resident_call_checks_its_inputs_on_the_device(gpu, tmp_models, L
         with pytest.raises(ValueError):
             eng.synchronize()                   # the skipped replay is still reported, once
         eng.synchronize()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["float64", "float32"])
+def test_layer0_gradients_on_request_follow_the_calls(gpu, tmp_models, dtype):
+    """With several polynomials per channel the whole-pipeline call keeps no M0_grad (its adjoint recomputes it); the
+    array is formed when it is asked for, from the evaluation that ran last, and stage-level calls made afterwards
+    (which do store gradients, as the reference's methods do) see consistent arrays.  Sequence: evaluation A, ask;
+    evaluation B on fewer atoms, reverse_M0 as a stage call (needs the gradients of B), ask; evaluation A again:
+    bit-identical to the first."""
+    model = H.tiny_model(K=24, L_max=1, n_pts=64, seed=31, pair=False)
+    path = H.write_model(model, tmp_models / "lazy_grad.json")
+    eng = gpu(path, dtype)
+    assert eng._int("contraction_tables") == 3
+    tol = 1e-10 if dtype == "float64" else 2e-4
+    runs = {}
+    for tag, n in (("A", 60), ("B", 23)):
+        pos, cell, sp = H.small_system(n, seed=n)
+        nl, ea = H.edges_of(pos, cell, sp, model["r_cut"])
+        orc = _oracle()(model)
+        orc.compute_node_energies_forces(*H.call_args(ea))
+        runs[tag] = (ea, orc)
+    ea, orc = runs["A"]
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    fA, eA = eng.node_forces.copy(), eng.node_energies.copy()
+    assert np.abs(eng.M0_grad - orc.M0_grad).max() <= tol * max(1.0, np.abs(orc.M0_grad).max())
+    ea, orc = runs["B"]
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    a0_adj = eng.A0_adj.copy()
+    assert np.abs(a0_adj - orc.A0_adj).max() <= tol * max(1.0, np.abs(orc.A0_adj).max())
+    eng.reverse_M0(ea["num_nodes"], ea["node_types"])          # stage call: streams over stored gradients
+    assert np.abs(eng.A0_adj - a0_adj).max() <= tol * max(1.0, np.abs(a0_adj).max())
+    assert eng.M0_grad.shape == orc.M0_grad.shape
+    assert np.abs(eng.M0_grad - orc.M0_grad).max() <= tol * max(1.0, np.abs(orc.M0_grad).max())
+    ea, orc = runs["A"]
+    eng.compute_node_energies_forces(*H.call_args(ea))
+    assert np.array_equal(eng.node_forces, fA) and np.array_equal(eng.node_energies, eA)
+    assert np.abs(eng.M0_grad - orc.M0_grad).max() <= tol * max(1.0, np.abs(orc.M0_grad).max())
